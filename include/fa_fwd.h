@@ -1,0 +1,129 @@
+/*
+ * fa_fwd.h — C ABI of the MI355X (gfx950) flash-attention forward launcher.
+ *
+ * This is the boundary a host framework binds to.  It replaces, for the forward path only,
+ * the vendor calls that torch_mlu's launcher `mha_varlen_fwd` makes
+ * (/root/reference path: torch_mlu/csrc/aten/operators/cnnl/internal/FlashAttention_internal.cpp:57-267):
+ *
+ *   cnnlCreate/SetFlashAttentionDescriptor + CnnlTensorDescriptor::set x8 (:131-180)  -> fa_fwd_params (one POD struct)
+ *   cnnlGetFlashAttentionForwardWorkspaceSize_v2 (:215-228)                         -> fa_fwd_workspace_bytes
+ *   cnnlFlashAttentionForward_v2 (:231-258)                                         -> fa_fwd_launch
+ *   cnnlGetFlashAttentionGeneratedRandomNumbers (:181-197)                          -> not needed: dropout_p must be 0
+ *
+ * Plain C: pointers, sizes and strides only.  No torch types, no exceptions, no allocation, no
+ * host/device synchronisation, no global mutable state: the library may be dlopen()ed from any
+ * language and called from any host thread.  All work is enqueued on the caller's HIP stream.
+ */
+#ifndef FA_FWD_H_
+#define FA_FWD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FA_FWD_ABI_VERSION 1
+
+/* element types accepted for q/k/v/out (FlashAttention_internal.cpp:73-80 allows exactly these two) */
+#define FA_DTYPE_FP16 0
+#define FA_DTYPE_BF16 1
+
+/* return codes */
+#define FA_OK 0
+#define FA_ERR_BAD_ARG (-1)     /* null pointer, non-positive size, misaligned pointer/stride, short workspace */
+#define FA_ERR_UNSUPPORTED (-2) /* shape or dtype outside the supported envelope */
+#define FA_ERR_LAUNCH (-3)      /* the HIP runtime refused the launch (hipGetLastError != hipSuccess) */
+
+/* kernel selection */
+#define FA_KERNEL_AUTO 0     /* split-KV kernel when seqlen_q == 1 and heads_q/heads_k <= 16, else the tile kernel */
+#define FA_KERNEL_TILE 1     /* MFMA tile (prefill) kernel */
+#define FA_KERNEL_SPLITKV 2  /* HBM-bound single-query split-KV kernel + merge */
+
+/*
+ * One attention-forward problem:  for every sequence b and query head h
+ *     S   = scale * Q[b,h] K[b,h/(heads_q/heads_k)]^T      (fp32 accumulate)
+ *     S   = -inf where is_causal and col > row + Lk_b - Lq_b (bottom-right aligned)
+ *     LSE = ln sum_j exp(S[:,j]),   out = softmax_row(S) V
+ * which is what cnnlFlashAttentionForward_v2 is asked to compute (FlashAttention_internal.cpp:147-161,231-258).
+ *
+ * Addressing (all strides are in ELEMENTS, row (b,s,h) of X starts at X + b*x_stride_b + s*x_stride_s + h*x_stride_h,
+ * the head_dim elements of a row are contiguous — the "contiguous last dimension" the reference demands at :101-108):
+ *   dense  (cu_seqlens_q == NULL): every sequence has seqlen_q / seqlen_k rows.
+ *   packed (cu_seqlens_q != NULL): sequence b owns rows [cu[b], cu[b+1]) of the packed [total, heads, head_dim]
+ *          tensors; *_stride_b is ignored; seqlen_q / seqlen_k are upper bounds (max_seqlen) used to size the grid.
+ *          cu_seqlens are int32 device arrays of batch+1 non-decreasing entries starting at 0 (:81-84,125-127) and
+ *          are only ever read on the device.
+ * LSE element (b,h,s) is written at lse + b*lse_stride_b + h*lse_stride_h + s*lse_stride_s; in packed mode s is the
+ * packed row index and lse_stride_b is ignored (the reference's kernel-side buffer is [heads_q, total_q], :129).
+ * Rows with no visible key (possible only when is_causal and Lk < Lq, or Lk == 0) get out = 0 and LSE = +inf.
+ */
+typedef struct fa_fwd_params {
+  const void* q;   /* device, 16-byte aligned */
+  const void* k;
+  const void* v;
+  void* out;
+  float* lse;
+  const int32_t* cu_seqlens_q; /* device int32[batch+1] or NULL */
+  const int32_t* cu_seqlens_k; /* device int32[batch+1] or NULL (both or neither) */
+
+  int64_t q_stride_b, q_stride_s, q_stride_h;
+  int64_t k_stride_b, k_stride_s, k_stride_h;
+  int64_t v_stride_b, v_stride_s, v_stride_h;
+  int64_t o_stride_b, o_stride_s, o_stride_h;
+  int64_t lse_stride_b, lse_stride_h, lse_stride_s;
+
+  int32_t batch;     /* > 0 */
+  int32_t heads_q;   /* > 0, multiple of heads_k (:122-124) */
+  int32_t heads_k;   /* > 0 */
+  int32_t seqlen_q;  /* dense: rows per sequence; packed: max over sequences */
+  int32_t seqlen_k;
+  int32_t head_dim;  /* multiple of 8, 8..256 (:119-121) */
+
+  float scale;       /* softmax scale, already resolved (attention.cpp:174-175 passes it as float) */
+  int32_t dtype;     /* FA_DTYPE_* */
+  int32_t is_causal; /* 0/1 */
+  int32_t kernel;    /* FA_KERNEL_* */
+  int32_t num_splits; /* split-KV only: 0 = choose, else 1..FA_MAX_SPLITS */
+  int32_t reserved;  /* must be 0 */
+} fa_fwd_params;
+
+#define FA_MAX_SPLITS 64
+
+/* ABI version of the loaded library (== FA_FWD_ABI_VERSION it was built with). */
+int fa_fwd_version(void);
+
+/* Static text for a return code. */
+const char* fa_fwd_error_string(int rc);
+
+/*
+ * Validate `p` without touching the GPU.  Returns FA_OK or a negative code; the same checks run inside
+ * fa_fwd_workspace_bytes / fa_fwd_launch.  Host-only, so callable on a machine with no device.
+ */
+int fa_fwd_validate(const fa_fwd_params* p);
+
+/*
+ * Bytes of device scratch fa_fwd_launch needs for `p` (0 for the tile kernel; partial (m, l, o) per split for the
+ * split-KV kernel).  Mirrors cnnlGetFlashAttentionForwardWorkspaceSize_v2.  Returns 0 also when `p` is invalid.
+ */
+size_t fa_fwd_workspace_bytes(const fa_fwd_params* p);
+
+/*
+ * Enqueue the forward pass on `stream` (a hipStream_t passed as void*; NULL = the null stream).
+ * `workspace` must hold at least fa_fwd_workspace_bytes(p) bytes (may be NULL when that is 0) and must stay
+ * alive until the enqueued work has run; stream-ordered allocators satisfy this.  Never allocates, never
+ * synchronises, never throws.  Returns FA_OK or a negative code (nothing is enqueued on error).
+ */
+int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Which kernel fa_fwd_launch would run for `p` (FA_KERNEL_TILE / FA_KERNEL_SPLITKV) and with how many splits;
+ * negative code when `p` is invalid.  Host-only.
+ */
+int fa_fwd_plan(const fa_fwd_params* p, int32_t* kernel, int32_t* num_splits);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FA_FWD_H_ */

@@ -1,0 +1,79 @@
+"""In-tree build recipes: hipcc for the HIP kernels + C-ABI library, g++ for the ATen extension.
+
+Everything is built for gfx950 only and lands in torch_mlu_amd/lib/ so that the shared objects travel
+with the source tree.  No JIT, no caches outside the tree.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(_HERE)
+CSRC = os.path.join(_HERE, "csrc")
+LIBDIR = os.path.join(_HERE, "lib")
+INCLUDE = os.path.join(ROOT, "include")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# Packed-fp32 VALU forms are switched off for all device code.
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wno-inline-asm", "-Wno-unused-command-line-argument",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _run(cmd, **kw):
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, **kw)
+    out = "\n".join(l for l in r.stdout.splitlines() if "is not a recognized feature for this target" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("build step failed: " + " ".join(cmd) + "\n" + out)
+    return out
+
+
+def build_kernels(verbose: bool = False) -> str:
+    """hipcc: csrc/fa_fwd_kernels.hip -> lib/libfa_fwd.so (the C ABI of include/fa_fwd.h)."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    out = os.path.join(LIBDIR, "libfa_fwd.so")
+    tmp = out + ".tmp"
+    log = _run([HIPCC, *HIP_FLAGS, "-shared", f"-I{INCLUDE}", os.path.join(CSRC, "fa_fwd_kernels.hip"), "-o", tmp])
+    os.replace(tmp, out)
+    if verbose and log.strip():
+        print(log)
+    return out
+
+
+def build_aten(verbose: bool = False) -> str:
+    """g++: csrc/fa_aten.cpp -> lib/libfa_aten.so (registers the two aten ops; links libfa_fwd.so by $ORIGIN)."""
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    os.makedirs(LIBDIR, exist_ok=True)
+    out = os.path.join(LIBDIR, "libfa_aten.so")
+    tmp = out + ".tmp"
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    inc = [f"-I{p}" for p in ce.include_paths("cuda")] + [f"-I{INCLUDE}"]
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    cmd = [
+        "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+        "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
+        *inc, os.path.join(CSRC, "fa_aten.cpp"), "-o", tmp,
+        f"-L{LIBDIR}", "-lfa_fwd", f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
+        "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}", "-Wl,--no-as-needed",
+    ]
+    log = _run(cmd)
+    os.replace(tmp, out)
+    if verbose and log.strip():
+        print(log)
+    return out
+
+
+def build_all(verbose: bool = False) -> None:
+    build_kernels(verbose)
+    build_aten(verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)
+    print("built:", sorted(os.listdir(LIBDIR)))

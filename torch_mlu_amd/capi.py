@@ -1,0 +1,207 @@
+"""ctypes binding of the C ABI in include/fa_fwd.h (libfa_fwd.so).
+
+This is the thinnest possible host side: torch is used only to own device memory and to name the
+current HIP stream.  The ATen extension (csrc/fa_aten.cpp) is the product path for
+`F.scaled_dot_product_attention`; this module exists so that the launcher can be driven and tested
+without the dispatcher in between, the way the reference's internal launcher `mha_varlen_fwd`
+(torch_mlu/csrc/aten/operators/cnnl/internal/FlashAttention_internal.cpp:57-267) sits below
+`cnnl__flash_attention_forward` (torch_mlu/csrc/aten/operators/cnnl/transformers/attention.cpp:161-203).
+
+There is no CPU fallback: if the shared library is missing, importing the symbols raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+import os
+from typing import Optional, Tuple
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libfa_fwd.so")
+
+FA_DTYPE_FP16 = 0
+FA_DTYPE_BF16 = 1
+FA_OK = 0
+FA_ERR_BAD_ARG = -1
+FA_ERR_UNSUPPORTED = -2
+FA_ERR_LAUNCH = -3
+FA_KERNEL_AUTO = 0
+FA_KERNEL_TILE = 1
+FA_KERNEL_SPLITKV = 2
+FA_MAX_SPLITS = 64
+
+# every symbol include/fa_fwd.h declares
+EXPORTED_SYMBOLS = (
+    "fa_fwd_version",
+    "fa_fwd_error_string",
+    "fa_fwd_validate",
+    "fa_fwd_workspace_bytes",
+    "fa_fwd_launch",
+    "fa_fwd_plan",
+)
+
+
+class FaFwdParams(ctypes.Structure):
+    """Mirror of `struct fa_fwd_params`."""
+
+    _fields_ = [
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("lse", ctypes.c_void_p),
+        ("cu_seqlens_q", ctypes.c_void_p),
+        ("cu_seqlens_k", ctypes.c_void_p),
+        ("q_stride_b", ctypes.c_int64), ("q_stride_s", ctypes.c_int64), ("q_stride_h", ctypes.c_int64),
+        ("k_stride_b", ctypes.c_int64), ("k_stride_s", ctypes.c_int64), ("k_stride_h", ctypes.c_int64),
+        ("v_stride_b", ctypes.c_int64), ("v_stride_s", ctypes.c_int64), ("v_stride_h", ctypes.c_int64),
+        ("o_stride_b", ctypes.c_int64), ("o_stride_s", ctypes.c_int64), ("o_stride_h", ctypes.c_int64),
+        ("lse_stride_b", ctypes.c_int64), ("lse_stride_h", ctypes.c_int64), ("lse_stride_s", ctypes.c_int64),
+        ("batch", ctypes.c_int32),
+        ("heads_q", ctypes.c_int32),
+        ("heads_k", ctypes.c_int32),
+        ("seqlen_q", ctypes.c_int32),
+        ("seqlen_k", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32),
+        ("scale", ctypes.c_float),
+        ("dtype", ctypes.c_int32),
+        ("is_causal", ctypes.c_int32),
+        ("kernel", ctypes.c_int32),
+        ("num_splits", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """Load libfa_fwd.so (built in-tree by torch_mlu_amd._build); raises if it is missing."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'`; "
+                "there is no fallback path")
+        L = ctypes.CDLL(LIB_PATH)
+        L.fa_fwd_version.restype = ctypes.c_int
+        L.fa_fwd_version.argtypes = []
+        L.fa_fwd_error_string.restype = ctypes.c_char_p
+        L.fa_fwd_error_string.argtypes = [ctypes.c_int]
+        L.fa_fwd_validate.restype = ctypes.c_int
+        L.fa_fwd_validate.argtypes = [ctypes.POINTER(FaFwdParams)]
+        L.fa_fwd_workspace_bytes.restype = ctypes.c_size_t
+        L.fa_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FaFwdParams)]
+        L.fa_fwd_launch.restype = ctypes.c_int
+        L.fa_fwd_launch.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        L.fa_fwd_plan.restype = ctypes.c_int
+        L.fa_fwd_plan.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.POINTER(ctypes.c_int32),
+                                  ctypes.POINTER(ctypes.c_int32)]
+        _lib = L
+    return _lib
+
+
+def error_string(rc: int) -> str:
+    return lib().fa_fwd_error_string(rc).decode()
+
+
+class FaFwdError(RuntimeError):
+    def __init__(self, rc: int):
+        super().__init__(f"fa_fwd_launch failed: rc={rc} ({error_string(rc)})")
+        self.rc = rc
+
+
+def _dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float16:
+        return FA_DTYPE_FP16
+    if dt == torch.bfloat16:
+        return FA_DTYPE_BF16
+    raise TypeError("FlashAttention only support fp16 and bf16 data type")
+
+
+def make_params(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor, *,
+                cu_seqlens_q: Optional[torch.Tensor] = None, cu_seqlens_k: Optional[torch.Tensor] = None,
+                max_seqlen_q: int = 0, max_seqlen_k: int = 0, scale: Optional[float] = None,
+                is_causal: bool = False, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0) -> FaFwdParams:
+    """Fill a params struct.
+
+    Dense: q/out are [B, Sq, Hq, D] *views* (any strides with a contiguous last dim), k/v [B, Sk, Hk, D],
+    lse [B, Hq, Sq].  Packed: q/out [Tq, Hq, D], k/v [Tk, Hk, D], lse [Hq, Tq], cu_seqlens int32 [B+1].
+    """
+    p = FaFwdParams()
+    p.q, p.k, p.v, p.out, p.lse = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr()
+    D = q.shape[-1]
+    if cu_seqlens_q is None:
+        B, Sq, Hq, _ = q.shape
+        Sk, Hk = k.shape[1], k.shape[2]
+        p.q_stride_b, p.q_stride_s, p.q_stride_h = q.stride(0), q.stride(1), q.stride(2)
+        p.k_stride_b, p.k_stride_s, p.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
+        p.v_stride_b, p.v_stride_s, p.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
+        p.o_stride_b, p.o_stride_s, p.o_stride_h = out.stride(0), out.stride(1), out.stride(2)
+        p.lse_stride_b, p.lse_stride_h, p.lse_stride_s = lse.stride(0), lse.stride(1), lse.stride(2)
+        p.cu_seqlens_q = None
+        p.cu_seqlens_k = None
+    else:
+        B = cu_seqlens_q.numel() - 1
+        Hq, Hk = q.shape[1], k.shape[1]
+        Sq, Sk = max_seqlen_q, max_seqlen_k
+        p.q_stride_s, p.q_stride_h = q.stride(0), q.stride(1)
+        p.k_stride_s, p.k_stride_h = k.stride(0), k.stride(1)
+        p.v_stride_s, p.v_stride_h = v.stride(0), v.stride(1)
+        p.o_stride_s, p.o_stride_h = out.stride(0), out.stride(1)
+        p.lse_stride_h, p.lse_stride_s = lse.stride(0), lse.stride(1)
+        p.cu_seqlens_q = cu_seqlens_q.data_ptr()
+        p.cu_seqlens_k = cu_seqlens_k.data_ptr()
+    p.batch, p.heads_q, p.heads_k = B, Hq, Hk
+    p.seqlen_q, p.seqlen_k, p.head_dim = Sq, Sk, D
+    # the reference resolves the default scale and narrows it to float before the launcher sees it
+    # (torch_mlu/csrc/aten/operators/cnnl/transformers/sdp_utils.h:40-47, attention.cpp:174-175)
+    p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
+    p.dtype = _dtype_code(q.dtype)
+    p.is_causal = 1 if is_causal else 0
+    p.kernel = kernel
+    p.num_splits = num_splits
+    p.reserved = 0
+    return p
+
+
+def launch(p: FaFwdParams, device: torch.device) -> None:
+    """Allocate the workspace the plan asks for and enqueue on torch's current stream of `device`."""
+    L = lib()
+    need = L.fa_fwd_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(need, dtype=torch.uint8, device=device) if need else None
+    stream = torch.cuda.current_stream(device).cuda_stream
+    rc = L.fa_fwd_launch(ctypes.byref(p), ws.data_ptr() if ws is not None else None, need, stream)
+    if rc != FA_OK:
+        raise FaFwdError(rc)
+
+
+def fa_forward_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, is_causal: bool = False,
+                     scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO,
+                     num_splits: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """q [B, Hq, Sq, D], k/v [B, Hk, Sk, D] (any strides, contiguous last dim) -> out [B, Hq, Sq, D] (stored
+    [B, Sq, Hq, D] like the reference's dense wrapper, attention.cpp:146-148), lse [B, Hq, Sq] fp32."""
+    B, Hq, Sq, D = q.shape
+    out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    p = make_params(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), out, lse, scale=scale,
+                    is_causal=is_causal, kernel=kernel, num_splits=num_splits)
+    launch(p, q.device)
+    return out.transpose(1, 2), lse
+
+
+def fa_forward_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                      cu_seqlens_k: torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, *, is_causal: bool = False,
+                      scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO,
+                      num_splits: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """q [Tq, Hq, D], k/v [Tk, Hk, D], cu_seqlens int32 [B+1] on the device -> out [Tq, Hq, D], lse [Hq, Tq]."""
+    Tq, Hq, D = q.shape
+    out = torch.empty((Tq, Hq, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((Hq, Tq), dtype=torch.float32, device=q.device)
+    p = make_params(q, k, v, out, lse, cu_seqlens_q=cu_seqlens_q, cu_seqlens_k=cu_seqlens_k,
+                    max_seqlen_q=max_seqlen_q, max_seqlen_k=max_seqlen_k, scale=scale, is_causal=is_causal,
+                    kernel=kernel, num_splits=num_splits)
+    launch(p, q.device)
+    return out, lse

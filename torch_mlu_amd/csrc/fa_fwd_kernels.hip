@@ -1,0 +1,889 @@
+// Flash-attention forward for MI355X (gfx950): HIP kernels and the C-ABI launcher declared in include/fa_fwd.h.
+//
+// Replaces the single vendor call cnnlFlashAttentionForward_v2 that torch_mlu's launcher makes
+// (torch_mlu/csrc/aten/operators/cnnl/internal/FlashAttention_internal.cpp:231-258) together with its
+// descriptor / workspace plumbing (:131-230).
+//
+// Two kernels:
+//   fa_tile_kernel     — MFMA-bound.  One workgroup (4 wavefronts) owns 128 query rows of one (sequence, head);
+//                        each wavefront keeps its 32 query rows in registers as the B operand of
+//                        v_mfma_f32_32x32x16 and computes S^T = K Q^T, so one lane owns one query row's scores
+//                        (row max / row sum need a single cross-lane exchange) and P^T is already in B-operand
+//                        layout for O^T += V^T P^T.  K/V tiles of 64 rows are double-buffered in LDS by
+//                        global->LDS DMA (16 bytes per lane, no staging registers); V^T fragments come from
+//                        ds_read_b64_tr_b16.  Causal and ragged (cu_seqlens) work is handled by the tile
+//                        scheduler: heavy tiles first, fully masked tiles skipped, partially masked tiles masked.
+//   fa_splitkv_kernel  — HBM-bound single-query (decode) shape.  One workgroup owns a contiguous slice of one
+//                        (sequence, kv head); every wavefront streams its own 32-row K/V blocks through a private
+//                        two-stage LDS ring by global->LDS DMA (no workgroup barriers in the loop), serves all
+//                        query heads of the GQA group from one pass over K/V with v_mfma_f32_16x16x32, and the
+//                        partial (m, l, o) triples are merged in LDS and, across slices, by fa_merge_kernel.
+//
+// All arithmetic is bf16/fp16 inputs, fp32 accumulate and fp32 softmax in the exp2 domain
+// (the reference asks the vendor kernel for compute_dtype = FLOAT, HIGH_PRECISION: :147-148).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fa_fwd.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+#define LDS_AS __attribute__((address_space(3)))
+#define GLB_AS __attribute__((address_space(1)))
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Kernel arguments: fa_fwd_params plus what the host derives once.
+struct KArgs {
+  const unsigned char* q;
+  const unsigned char* k;
+  const unsigned char* v;
+  unsigned char* out;
+  float* lse;
+  const int32_t* cu_q;
+  const int32_t* cu_k;
+  int64_t q_sb, q_ss, q_sh;  // byte strides
+  int64_t k_sb, k_ss, k_sh;
+  int64_t v_sb, v_ss, v_sh;
+  int64_t o_sb, o_ss, o_sh;
+  int64_t lse_sb, lse_sh, lse_ss;  // element strides
+  int32_t batch, heads_q, heads_k, group;
+  int32_t seqlen_q, seqlen_k, head_dim;
+  int32_t n_mblk;     // tile kernel: query blocks per sequence
+  int32_t n_splits;   // split-KV kernel
+  int32_t is_causal;
+  int32_t neg_scale;  // scale < 0: Q is negated on load and |scale| is used, so that max() tracks the true row max
+  float scale_log2;   // |scale| * log2(e)
+  float* ws_o;        // split-KV partials: [batch*heads_q*n_splits][head_dim] fp32, unnormalised
+  float* ws_ml;       // [batch*heads_q*n_splits][2]: m (log2 domain), l
+};
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<__bf16> {
+  static __device__ __forceinline__ f32x16 m32(s16x8 a, s16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16(s16x8 a, s16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ unsigned pack2(float a, float b) {
+    f32x2 f = {a, b};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
+  }
+};
+template <>
+struct Mma<_Float16> {
+  static __device__ __forceinline__ f32x16 m32(s16x8 a, s16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16(s16x8 a, s16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ unsigned pack2(float a, float b) {
+    f32x2 f = {a, b};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f, f16x2));
+  }
+};
+
+// 16-byte global -> LDS DMA.  Lane i of the wavefront writes LDS bytes [lds_wave_base + 16 i, +16); the global
+// address is per lane.  lds_wave_base must be wavefront-uniform.  Written as inline assembly on purpose: the
+// compiler then does not know these loads write LDS, so it does not put a conservative "wait for every
+// outstanding load" in front of the LDS reads of the tile being computed.  Completion is tracked by hand
+// with WAIT_VMCNT (the loads retire in order).
+__device__ __forceinline__ void dma16(const unsigned char* gptr, unsigned char* lds_wave_base) {
+  const unsigned lds = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(LDS_AS unsigned char*)lds_wave_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds), "v"(gptr) : "memory", "m0");
+}
+
+// Transposed LDS read: within each group of 16 lanes, lane j receives element (j % 4) of the four 8-byte pieces
+// addressed by lanes 4 i + j / 4 (i = 0..3) of the same group.
+__device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 LDS_AS*)p);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// max over the lane pair (l, l ^ 32)
+__device__ __forceinline__ float pair_max32(float x) {
+  unsigned u = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+}
+__device__ __forceinline__ float pair_sum32(float x) {
+  unsigned u = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+}
+
+#define WAIT_VMCNT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
+
+// ---------------------------------------------------------------------------------------------------------
+// Tile kernel
+// ---------------------------------------------------------------------------------------------------------
+// LDS layouts (rows of DP elements = CPR chunks of 16 bytes; a tile is 64 rows):
+//   K tile: physical chunk = logical chunk ^ swzK(row) so that the 16 lanes of a ds_read_b128 (16 different rows,
+//           same logical chunk) hit 16 different 16-byte bank groups.
+//   V tile: physical chunk = logical chunk ^ swzV(row) so that the 4 rows x 64 bytes a half-wave reads with
+//           ds_read_b64_tr_b16 cover all 64 banks once.
+template <int DP>
+__device__ __forceinline__ int swzK(int row) {
+  if constexpr (DP == 64) return (row >> 1) & 7;
+  return row & 15;
+}
+template <int DP>
+__device__ __forceinline__ int swzV(int row) {
+  if constexpr (DP == 64) return ((row >> 1) & 1) << 2;
+  return (row & 3) << 2;
+}
+
+template <typename T, int DP, int MINB>
+__global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
+  constexpr int CPR = DP / 8;          // 16-byte chunks per row
+  constexpr int ROWB = DP * 2;         // bytes per LDS row
+  constexpr int BM = 128, BN = 64;
+  constexpr int TILE = BN * ROWB;      // bytes per K (or V) tile
+  constexpr int NI = TILE / 1024 / 4;  // DMA instructions per wavefront per tile
+  constexpr int RPI = 64 / CPR;        // rows covered by one DMA instruction
+  constexpr int KS = DP / 16;          // MFMA k-steps over the head dim
+  constexpr int MB = DP / 32;          // 32-row blocks of O^T
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // K0 K1 V0 V1
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 5, c32 = lane & 31;
+
+  // ---- which (sequence, head, query block): XCD-aware, heavy blocks first -------------------------------
+  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical ids so that
+  // all query blocks of one (sequence, kv head) share that XCD's L2.
+  int lid = blockIdx.x;
+  {
+    const int total = gridDim.x, per = total >> 3;
+    if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
+  }
+  const int mi = a.n_mblk - 1 - (lid % a.n_mblk);
+  const int bh = lid / a.n_mblk;
+  const int h = bh % a.heads_q, b = bh / a.heads_q;
+  const int hk = h / a.group;
+
+  int q0 = 0, k0 = 0, Lq = a.seqlen_q, Lk = a.seqlen_k;
+  int64_t qb = (int64_t)b * a.q_sb, kb = (int64_t)b * a.k_sb, vb = (int64_t)b * a.v_sb, ob = (int64_t)b * a.o_sb;
+  int64_t lb = (int64_t)b * a.lse_sb;
+  if (a.cu_q) {
+    q0 = a.cu_q[b];
+    Lq = a.cu_q[b + 1] - q0;
+    k0 = a.cu_k[b];
+    Lk = a.cu_k[b + 1] - k0;
+    qb = kb = vb = ob = 0;
+    lb = 0;
+  }
+  const int m0 = mi * BM;
+  if (m0 >= Lq) return;
+  const int off = Lk - Lq;  // causal: col visible iff col <= row + off
+  int n_end = Lk;
+  if (a.is_causal) n_end = min(Lk, m0 + BM + off);
+  if (n_end < 0) n_end = 0;
+  const int ntiles = (n_end + BN - 1) / BN;
+
+  const unsigned char* qp = a.q + qb + (int64_t)q0 * a.q_ss + (int64_t)h * a.q_sh;
+  const unsigned char* kp = a.k + kb + (int64_t)k0 * a.k_ss + (int64_t)hk * a.k_sh;
+  const unsigned char* vp = a.v + vb + (int64_t)k0 * a.v_ss + (int64_t)hk * a.v_sh;
+  const int D = a.head_dim;
+  const int row = m0 + 32 * wave + c32;  // this lane's query row (lanes l and l^32 share it)
+
+  // ---- DMA bookkeeping: lane -> (row in instruction block, logical chunk) --------------------------------
+  const int dma_r = wave * RPI + lane / CPR;  // row within tile for instruction 0; instruction i adds 4*RPI*i
+  const int dma_pc = lane % CPR;
+  // head_dim < DP: pad chunks are pointed at chunk 0 (valid memory); they meet zeros of Q / are never stored.
+  // The swizzles only use row bits that the per-instruction row step (4 RPI) leaves alone, except swzK at
+  // DP == 256 where odd instructions toggle bit 3.
+  int lck = dma_pc ^ swzK<DP>(dma_r);
+  int lck_odd = (DP == 256) ? (lck ^ 8) : lck;
+  int lcv = dma_pc ^ swzV<DP>(dma_r);
+  if (lck * 8 >= D) lck = 0;
+  if (lck_odd * 8 >= D) lck_odd = 0;
+  if (lcv * 8 >= D) lcv = 0;
+  const unsigned char* kp_lane = kp + lck * 16;
+  const unsigned char* kp_lane_odd = kp + lck_odd * 16;
+  const unsigned char* vp_lane = vp + lcv * 16;
+  const unsigned k_ss = (unsigned)a.k_ss, v_ss = (unsigned)a.v_ss;
+  const int last_k = Lk - 1;
+
+  auto issue_tile = [&](int j, int buf) {
+    unsigned char* kdst = smem + buf * TILE + wave * 1024;
+    unsigned char* vdst = smem + 2 * TILE + buf * TILE + wave * 1024;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int r = min(j * BN + dma_r + i * 4 * RPI, last_k);
+      dma16(((DP == 256 && (i & 1)) ? kp_lane_odd : kp_lane) + (uint64_t)(unsigned)r * k_ss, kdst + i * 4096);
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int r = min(j * BN + dma_r + i * 4 * RPI, last_k);
+      dma16(vp_lane + (uint64_t)(unsigned)r * v_ss, vdst + i * 4096);
+    }
+  };
+
+  if (ntiles > 0) issue_tile(0, 0);
+
+  // ---- Q fragments (B operand): lane (c32, g) holds Q[row][16 ks + 8 g .. +8] -----------------------------
+  s16x8 qf[KS];
+  {
+    const int qr = min(row, Lq - 1);
+    const unsigned char* qrow = qp + (int64_t)qr * a.q_ss;
+    const unsigned flip = a.neg_scale ? 0x80008000u : 0u;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int ch = 2 * ks + g;
+      u32x4 x = {0, 0, 0, 0};
+      if (ch * 8 < D) x = *(const u32x4*)(qrow + ch * 16);
+      x ^= flip;
+      qf[ks] = __builtin_bit_cast(s16x8, x);
+    }
+  }
+
+  f32x16 o[MB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = a.scale_log2;
+
+  // per-lane LDS read offsets
+  const int ksw = swzK<DP>(c32);  // same for rows c32 and 32 + c32
+  const int L = lane & 15, G = lane >> 4;
+  // V^T fragment for (mblk, t, half): row 16 t + 8 half + 4 g + (L >> 2), logical chunk 4 mblk + 2 (G & 1) + ((L & 3) >> 1)
+  const int v_row = 4 * g + (L >> 2);
+  const int v_lc0 = 2 * (G & 1) + ((L & 3) >> 1);
+  const int v_sw = swzV<DP>(v_row);  // rows differ by multiples of 8 across (t, half): same swizzle
+  const int v_lane_off = v_row * ROWB + (L & 1) * 8;
+
+  const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
+
+  for (int j = 0; j < ntiles; ++j) {
+    const int buf = j & 1;
+    WAIT_VMCNT(0);       // my DMA for tile j has landed
+    __syncthreads();     // everyone's has; everyone is done reading the other buffer
+    if (j + 1 < ntiles) issue_tile(j + 1, buf ^ 1);
+
+    // wavefront-uniform skip: every score of this tile is masked for all 32 rows of this wavefront
+    const int wave_row_hi = m0 + 32 * wave + 31;
+    if (a.is_causal && j * BN > wave_row_hi + off) continue;
+
+    const unsigned char* kt = smem + buf * TILE;
+    const unsigned char* vt = smem + 2 * TILE + buf * TILE;
+
+    // ---- S^T = K Q^T : two 32(kv) x 32(q) blocks ----
+    f32x16 s0, s1;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int pc = (2 * ks + g) ^ ksw;
+      const s16x8 a0 = *(const s16x8*)(kt + c32 * ROWB + pc * 16);
+      const s16x8 a1 = *(const s16x8*)(kt + (32 + c32) * ROWB + pc * 16);
+      s0 = Mma<T>::m32(a0, qf[ks], s0);
+      s1 = Mma<T>::m32(a1, qf[ks], s1);
+    }
+
+    // ---- mask (tail of K, causal diagonal) ----
+    const int wave_row_lo = m0 + 32 * wave;
+    const bool need_mask = (j * BN + BN > Lk) || (a.is_causal && j * BN + BN - 1 > wave_row_lo + off);
+    if (need_mask) {
+      const int lim = min(last_k, causal_row_lim) - j * BN - 4 * g;  // element index e is visible iff e <= lim
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int e = 8 * (v >> 2) + (v & 3);
+        if (e > lim) s0[v] = -INFINITY;
+        if (32 + e > lim) s1[v] = -INFINITY;
+      }
+    }
+
+    // ---- online softmax (one lane = one query row x 32 of the 64 columns) ----
+    float mx = fmaxf(s0[0], s1[0]);
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(s0[v], s1[v]));
+    mx = pair_max32(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = fast_exp2((m_run - m_use) * c);
+    const float mc = m_use * c;
+    m_run = m_new;
+    float rs = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      s0[v] = fast_exp2(s0[v] * c - mc);
+      s1[v] = fast_exp2(s1[v] * c - mc);
+      rs += s0[v] + s1[v];
+    }
+    l_run = l_run * alpha + rs;
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
+
+    // ---- P^T as B operands: k-step t covers kv 16 t .. 16 t + 15 of the tile ----
+    s16x8 pb[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      u32x4 w;
+#pragma unroll
+      for (int e2 = 0; e2 < 4; ++e2) {
+        const int v = 8 * (t & 1) + 2 * e2;
+        w[e2] = (t < 2) ? Mma<T>::pack2(s0[v], s0[v + 1]) : Mma<T>::pack2(s1[v], s1[v + 1]);
+      }
+      pb[t] = __builtin_bit_cast(s16x8, w);
+    }
+
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int pc = (4 * mb + v_lc0) ^ v_sw;
+      const unsigned char* vbase = vt + v_lane_off + pc * 16;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const s16x4 lo = lds_read_tr(vbase + (16 * t) * ROWB);
+        const s16x4 hi = lds_read_tr(vbase + (16 * t + 8) * ROWB);
+        const s16x8 av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        o[mb] = Mma<T>::m32(av, pb[t], o[mb]);
+      }
+    }
+  }
+
+  // ---- epilogue ----
+  l_run = pair_sum32(l_run);
+  const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
+  if (row < Lq) {
+    unsigned char* orow = a.out + ob + (int64_t)(q0 + row) * a.o_ss + (int64_t)h * a.o_sh;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const int d = 32 * mb + 8 * v4 + 4 * g;
+        if (d < D) {
+          u32x2 w;
+          w[0] = Mma<T>::pack2(o[mb][4 * v4 + 0] * inv, o[mb][4 * v4 + 1] * inv);
+          w[1] = Mma<T>::pack2(o[mb][4 * v4 + 2] * inv, o[mb][4 * v4 + 3] * inv);
+          *(u32x2*)(orow + d * 2) = w;
+        }
+      }
+    if (g == 0) {
+      const float lse = (l_run > 0.f) ? (m_run * c + __builtin_log2f(l_run)) * kLn2 : INFINITY;
+      a.lse[lb + (int64_t)h * a.lse_sh + (int64_t)(q0 + row) * a.lse_ss] = lse;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Split-KV kernel (seqlen_q == 1, group <= 16)
+// ---------------------------------------------------------------------------------------------------------
+template <int DP>
+__device__ __forceinline__ int swzKd(int row) {  // 16 lanes = 16 rows, same logical chunk, ds_read_b128
+  if constexpr (DP == 64) return (row >> 1) & 7;
+  return row & 15;
+}
+template <int DP>
+__device__ __forceinline__ int swzVd(int row) {  // 8 rows x 32 bytes per half-wave, ds_read_b64_tr_b16
+  if constexpr (DP == 64) return ((row >> 1) & 3) << 1;
+  return (row & 7) << 1;
+}
+
+template <int DP>
+struct SplitCfg {
+  static constexpr int NW = (DP == 256) ? 2 : 4;        // wavefronts per workgroup
+  static constexpr int STAGE = 2 * 32 * DP * 2;         // K block + V block, 32 rows each
+  static constexpr int RING = 2 * STAGE;                // per wavefront
+  static constexpr int LDS = NW * RING;
+};
+
+template <typename T, int DP>
+__global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(const KArgs a) {
+  constexpr int NW = SplitCfg<DP>::NW;
+  constexpr int CPR = DP / 8;
+  constexpr int ROWB = DP * 2;
+  constexpr int BLK = 32 * ROWB;        // bytes of a 32-row K (or V) block
+  constexpr int NI = BLK / 1024;        // DMA instructions per block
+  constexpr int RPI = 64 / CPR;         // rows per DMA instruction
+  constexpr int KS = DP / 32;           // k-steps of the 16x16x32 MFMA over head dim
+  constexpr int MB = DP / 16;           // 16-row blocks of O^T
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int L = lane & 15, G = lane >> 4;
+
+  const int split = blockIdx.x % a.n_splits;
+  const int bhk = blockIdx.x / a.n_splits;
+  const int hk = bhk % a.heads_k, b = bhk / a.heads_k;
+
+  int q0 = 0, k0 = 0, Lk = a.seqlen_k;  // dense: the query of sequence b is row 0 of batch b
+  int64_t qb = (int64_t)b * a.q_sb, kb = (int64_t)b * a.k_sb, vb = (int64_t)b * a.v_sb, ob = (int64_t)b * a.o_sb;
+  int64_t lb = (int64_t)b * a.lse_sb;
+  int Lq = 1;
+  if (a.cu_q) {
+    q0 = a.cu_q[b];
+    Lq = a.cu_q[b + 1] - q0;
+    k0 = a.cu_k[b];
+    Lk = a.cu_k[b + 1] - k0;
+    qb = kb = vb = ob = 0;
+    lb = (int64_t)q0 * a.lse_ss;
+  }
+  const int D = a.head_dim;
+  const int group = a.group;
+  const int h0 = hk * group;
+
+  // slice of 32-row blocks owned by this workgroup, then by this wavefront (interleaved)
+  const int nblk = (Lk + 31) >> 5;
+  const int per = (nblk + a.n_splits - 1) / a.n_splits;
+  const int blk_begin = split * per;
+  const int blk_end = min(nblk, blk_begin + per);
+  const int last_k = Lk - 1;
+
+  const unsigned char* kp = a.k + kb + (int64_t)k0 * a.k_ss + (int64_t)hk * a.k_sh;
+  const unsigned char* vp = a.v + vb + (int64_t)k0 * a.v_ss + (int64_t)hk * a.v_sh;
+  const unsigned k_ss = (unsigned)a.k_ss, v_ss = (unsigned)a.v_ss;
+
+  unsigned char* ring = smem + wave * SplitCfg<DP>::RING;
+  const int dma_r = lane / CPR, dma_pc = lane % CPR;
+
+  auto issue_block = [&](int blk, int stage) {
+    unsigned char* kdst = ring + stage * SplitCfg<DP>::STAGE;
+    unsigned char* vdst = kdst + BLK;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int r = dma_r + i * RPI;
+      int lc = dma_pc ^ swzKd<DP>(r);
+      if (lc * 8 >= D) lc = 0;
+      const int gr = min(blk * 32 + r, last_k);
+      dma16(kp + (uint64_t)(unsigned)gr * k_ss + lc * 16, kdst + i * 1024);
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int r = dma_r + i * RPI;
+      int lc = dma_pc ^ swzVd<DP>(r);
+      if (lc * 8 >= D) lc = 0;
+      const int gr = min(blk * 32 + r, last_k);
+      dma16(vp + (uint64_t)(unsigned)gr * v_ss + lc * 16, vdst + i * 1024);
+    }
+  };
+
+  int blk = blk_begin + wave;
+  if (blk < blk_end && Lq > 0) issue_block(blk, 0);
+
+  // Q^T as B operand of 16x16x32: lane (q slot = L, G) holds Q[h0 + L][32 ks + 8 G .. +8]; slots >= group are zero
+  s16x8 qf[KS];
+  {
+    const unsigned flip = a.neg_scale ? 0x80008000u : 0u;
+    const unsigned char* qrow = a.q + qb + (int64_t)q0 * a.q_ss + (int64_t)(h0 + L) * a.q_sh;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int ch = 4 * ks + G;
+      u32x4 x = {0, 0, 0, 0};
+      if (L < group && ch * 8 < D && Lq > 0) {
+        x = *(const u32x4*)(qrow + ch * 16);
+        x ^= flip;
+      }
+      qf[ks] = __builtin_bit_cast(s16x8, x);
+    }
+  }
+
+  f32x4 o[MB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;  // per q slot (replicated over G); l_run is this lane's partial sum
+  const float c = a.scale_log2;
+
+  const int ksw = swzKd<DP>(L);                 // rows L and 16 + L
+  const int vrow = 4 * G + (L >> 2);            // + 16 for the second half of the contraction
+  const int vsw = swzVd<DP>(vrow);              // same for vrow + 16
+  const int v_lane_off = vrow * ROWB + (L & 1) * 8;
+  const int v_lc0 = (L & 3) >> 1;
+
+  int stage = 0;
+  for (; blk < blk_end && Lq > 0; blk += NW) {
+    const int nxt = blk + NW;
+    if (nxt < blk_end) {
+      issue_block(nxt, stage ^ 1);
+      if constexpr (NI == 4) WAIT_VMCNT(8);
+      else if constexpr (NI == 8) WAIT_VMCNT(16);
+      else WAIT_VMCNT(32);
+    } else {
+      WAIT_VMCNT(0);
+    }
+    const unsigned char* kt = ring + stage * SplitCfg<DP>::STAGE;
+    const unsigned char* vt = kt + BLK;
+
+    // S^T (kv x q slot): two 16-row tiles
+    f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int pc = (4 * ks + G) ^ ksw;
+      const s16x8 a0 = *(const s16x8*)(kt + L * ROWB + pc * 16);
+      const s16x8 a1 = *(const s16x8*)(kt + (16 + L) * ROWB + pc * 16);
+      sa = Mma<T>::m16(a0, qf[ks], sa);
+      sb = Mma<T>::m16(a1, qf[ks], sb);
+    }
+    if (blk * 32 + 32 > Lk) {
+      const int lim = last_k - blk * 32 - 4 * G;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        if (v > lim) sa[v] = -INFINITY;
+        if (16 + v > lim) sb[v] = -INFINITY;
+      }
+    }
+    float mx = fmaxf(fmaxf(sa[0], sa[1]), fmaxf(sa[2], sa[3]));
+    mx = fmaxf(mx, fmaxf(fmaxf(sb[0], sb[1]), fmaxf(sb[2], sb[3])));
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = pair_max32(mx);
+    const float m_new = fmaxf(m_run, mx);  // a visited block always has at least one visible row: m_new is finite
+    const float alpha = fast_exp2((m_run - m_new) * c);
+    const float mc = m_new * c;
+    m_run = m_new;
+    float rs = 0.f;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      sa[v] = fast_exp2(sa[v] * c - mc);
+      sb[v] = fast_exp2(sb[v] * c - mc);
+      rs += sa[v] + sb[v];
+    }
+    l_run = l_run * alpha + rs;
+#pragma unroll
+    for (int i = 0; i < MB; ++i) o[i] *= alpha;
+
+    u32x4 w;
+    w[0] = Mma<T>::pack2(sa[0], sa[1]);
+    w[1] = Mma<T>::pack2(sa[2], sa[3]);
+    w[2] = Mma<T>::pack2(sb[0], sb[1]);
+    w[3] = Mma<T>::pack2(sb[2], sb[3]);
+    const s16x8 pb = __builtin_bit_cast(s16x8, w);
+
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int pc = (2 * mb + v_lc0) ^ vsw;
+      const unsigned char* vbase = vt + v_lane_off + pc * 16;
+      const s16x4 lo = lds_read_tr(vbase);
+      const s16x4 hi = lds_read_tr(vbase + 16 * ROWB);
+      const s16x8 av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      o[mb] = Mma<T>::m16(av, pb, o[mb]);
+    }
+    stage ^= 1;
+  }
+
+  // ---- merge the NW wavefronts' partials through LDS ----
+  l_run += __shfl_xor(l_run, 16);
+  l_run = pair_sum32(l_run);
+  __syncthreads();  // all rings are idle (every wavefront waited for its last DMA before its last block)
+  float* so = (float*)smem;                       // [NW][16][DP]
+  float* sml = (float*)(smem + NW * 16 * DP * 4); // [NW][16][2]
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) so[(wave * 16 + L) * DP + 16 * mb + 4 * G + v] = o[mb][v];
+  if (G == 0) {
+    sml[(wave * 16 + L) * 2 + 0] = (m_run == -INFINITY) ? -INFINITY : m_run * c;
+    sml[(wave * 16 + L) * 2 + 1] = l_run;
+  }
+  __syncthreads();
+  if (Lq <= 0) return;
+  // thread -> (q slot, 16 d-values)
+  constexpr int TPQ = DP / 16;  // threads per q slot
+  for (int item = tid; item < group * TPQ; item += NW * 64) {
+    const int qs = item / TPQ, d0 = (item % TPQ) * 16;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, sml[(w * 16 + qs) * 2]);
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    float lsum = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const float mw = sml[(w * 16 + qs) * 2];
+      const float sc = (mw == -INFINITY) ? 0.f : fast_exp2(mw - M);
+      lsum += sml[(w * 16 + qs) * 2 + 1] * sc;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] += so[(w * 16 + qs) * DP + d0 + i] * sc;
+    }
+    const int h = h0 + qs;
+    if (a.n_splits == 1) {
+      const float inv = (lsum > 0.f) ? 1.f / lsum : 0.f;
+      if (d0 < D) {
+        unsigned char* orow = a.out + ob + (int64_t)q0 * a.o_ss + (int64_t)h * a.o_sh + d0 * 2;
+        u32x4 w0, w1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          w0[i] = Mma<T>::pack2(acc[2 * i] * inv, acc[2 * i + 1] * inv);
+          w1[i] = Mma<T>::pack2(acc[8 + 2 * i] * inv, acc[8 + 2 * i + 1] * inv);
+        }
+        *(u32x4*)orow = w0;
+        if (d0 + 8 < D) *(u32x4*)(orow + 16) = w1;
+      }
+      if (d0 == 0) a.lse[lb + (int64_t)h * a.lse_sh] = (lsum > 0.f) ? (M + __builtin_log2f(lsum)) * kLn2 : INFINITY;
+    } else {
+      const int64_t slot = ((int64_t)b * a.heads_q + h) * a.n_splits + split;
+      if (d0 < D) {
+        float* dst = a.ws_o + slot * D + d0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (d0 + i < D) dst[i] = acc[i];
+      }
+      if (d0 == 0) {
+        a.ws_ml[slot * 2 + 0] = M;
+        a.ws_ml[slot * 2 + 1] = lsum;
+      }
+    }
+  }
+}
+
+// Merge the per-slice partials: one wavefront per (sequence, query head); lane -> head_dim elements lane, lane+64, ...
+template <typename T>
+__global__ void __launch_bounds__(64) fa_merge_kernel(const KArgs a) {
+  const int bh = blockIdx.x;
+  const int h = bh % a.heads_q, b = bh / a.heads_q;
+  const int lane = threadIdx.x;
+  const int D = a.head_dim, ns = a.n_splits;
+  int q0 = 0;
+  int64_t ob = (int64_t)b * a.o_sb, lb = (int64_t)b * a.lse_sb;
+  if (a.cu_q) {
+    q0 = a.cu_q[b];
+    if (a.cu_q[b + 1] - q0 <= 0) return;
+    ob = 0;
+    lb = (int64_t)q0 * a.lse_ss;
+  }
+  const float* ml = a.ws_ml + (int64_t)bh * ns * 2;
+  const float* po = a.ws_o + (int64_t)bh * ns * D;
+  float M = -INFINITY;
+  for (int s = 0; s < ns; ++s) M = fmaxf(M, ml[2 * s]);
+  float lsum = 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};  // head_dim <= 256
+  for (int s = 0; s < ns; ++s) {
+    const float ms = ml[2 * s];
+    const float sc = (ms == -INFINITY) ? 0.f : fast_exp2(ms - M);
+    lsum += ml[2 * s + 1] * sc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < D) acc[i] += po[(int64_t)s * D + d] * sc;
+    }
+  }
+  const float inv = (lsum > 0.f) ? 1.f / lsum : 0.f;
+  T* orow = (T*)(a.out + ob + (int64_t)q0 * a.o_ss + (int64_t)h * a.o_sh);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d < D) orow[d] = (T)(acc[i] * inv);
+  }
+  if (lane == 0) a.lse[lb + (int64_t)h * a.lse_sh] = (lsum > 0.f) ? (M + __builtin_log2f(lsum)) * kLn2 : INFINITY;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------------------------
+int padded_dim(int d) { return d <= 64 ? 64 : (d <= 128 ? 128 : 256); }
+
+int validate(const fa_fwd_params* p) {
+  if (!p) return FA_ERR_BAD_ARG;
+  if (!p->q || !p->k || !p->v || !p->out || !p->lse) return FA_ERR_BAD_ARG;
+  if ((p->cu_seqlens_q == nullptr) != (p->cu_seqlens_k == nullptr)) return FA_ERR_BAD_ARG;
+  if (p->batch <= 0 || p->heads_q <= 0 || p->heads_k <= 0) return FA_ERR_BAD_ARG;
+  if (p->seqlen_q < 0 || p->seqlen_k < 0 || p->head_dim <= 0) return FA_ERR_BAD_ARG;
+  if (p->reserved != 0) return FA_ERR_BAD_ARG;
+  if (p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_UNSUPPORTED;
+  if (p->head_dim > 256 || (p->head_dim & 7)) return FA_ERR_UNSUPPORTED;
+  if (p->heads_q % p->heads_k) return FA_ERR_UNSUPPORTED;
+  if (p->kernel < FA_KERNEL_AUTO || p->kernel > FA_KERNEL_SPLITKV) return FA_ERR_BAD_ARG;
+  if (p->num_splits < 0 || p->num_splits > FA_MAX_SPLITS) return FA_ERR_BAD_ARG;
+  // 16-byte vector access on every row: base pointers and row strides must be multiples of 8 elements
+  const uintptr_t al = (uintptr_t)p->q | (uintptr_t)p->k | (uintptr_t)p->v | (uintptr_t)p->out;
+  if (al & 15) return FA_ERR_BAD_ARG;
+  if ((uintptr_t)p->lse & 3) return FA_ERR_BAD_ARG;
+  const int64_t st[] = {p->q_stride_s, p->q_stride_h, p->k_stride_s, p->k_stride_h, p->v_stride_s, p->v_stride_h,
+                        p->o_stride_s, p->o_stride_h};
+  for (int64_t s : st)
+    if (s < 0 || (s & 7)) return FA_ERR_BAD_ARG;
+  if (!p->cu_seqlens_q) {
+    const int64_t sb[] = {p->q_stride_b, p->k_stride_b, p->v_stride_b, p->o_stride_b};
+    for (int64_t s : sb)
+      if (s < 0 || (s & 7)) return FA_ERR_BAD_ARG;
+    if (p->lse_stride_b < 0) return FA_ERR_BAD_ARG;
+  }
+  if (p->lse_stride_h < 0 || p->lse_stride_s < 0) return FA_ERR_BAD_ARG;
+  // the kernels form per-row byte offsets as 32-bit row x 32-bit stride
+  if (p->k_stride_s * 2 > 0x7fffffffLL || p->v_stride_s * 2 > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
+  if (p->kernel == FA_KERNEL_SPLITKV) {
+    if (p->seqlen_q != 1 || p->heads_q / p->heads_k > 16) return FA_ERR_UNSUPPORTED;
+  }
+  return FA_OK;
+}
+
+void plan(const fa_fwd_params* p, int* kernel, int* splits) {
+  int kern = p->kernel;
+  const int group = p->heads_q / p->heads_k;
+  if (kern == FA_KERNEL_AUTO) kern = (p->seqlen_q == 1 && group <= 16 && p->seqlen_k >= 256) ? FA_KERNEL_SPLITKV : FA_KERNEL_TILE;
+  int ns = 1;
+  if (kern == FA_KERNEL_SPLITKV) {
+    ns = p->num_splits;
+    if (ns == 0) {
+      // enough workgroups to fill 256 CUs several times over, but no slice shorter than 512 rows
+      const int64_t units = (int64_t)p->batch * p->heads_k;
+      const int nblk = (p->seqlen_k + 31) / 32;
+      ns = 1;
+      while (ns < FA_MAX_SPLITS && units * ns < 2048 && nblk / (ns * 2) >= 16) ns *= 2;
+    }
+    const int nblk = (p->seqlen_k + 31) / 32;
+    if (ns > nblk) ns = nblk > 0 ? nblk : 1;
+  }
+  *kernel = kern;
+  *splits = ns;
+}
+
+size_t workspace_bytes(const fa_fwd_params* p, int kern, int ns) {
+  if (kern != FA_KERNEL_SPLITKV || ns <= 1) return 0;
+  const size_t slots = (size_t)p->batch * p->heads_q * ns;
+  return slots * (size_t)p->head_dim * 4 + slots * 8;
+}
+
+KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
+  KArgs a;
+  a.q = (const unsigned char*)p->q;
+  a.k = (const unsigned char*)p->k;
+  a.v = (const unsigned char*)p->v;
+  a.out = (unsigned char*)p->out;
+  a.lse = p->lse;
+  a.cu_q = p->cu_seqlens_q;
+  a.cu_k = p->cu_seqlens_k;
+  a.q_sb = p->q_stride_b * 2; a.q_ss = p->q_stride_s * 2; a.q_sh = p->q_stride_h * 2;
+  a.k_sb = p->k_stride_b * 2; a.k_ss = p->k_stride_s * 2; a.k_sh = p->k_stride_h * 2;
+  a.v_sb = p->v_stride_b * 2; a.v_ss = p->v_stride_s * 2; a.v_sh = p->v_stride_h * 2;
+  a.o_sb = p->o_stride_b * 2; a.o_ss = p->o_stride_s * 2; a.o_sh = p->o_stride_h * 2;
+  a.lse_sb = p->lse_stride_b; a.lse_sh = p->lse_stride_h; a.lse_ss = p->lse_stride_s;
+  a.batch = p->batch; a.heads_q = p->heads_q; a.heads_k = p->heads_k; a.group = p->heads_q / p->heads_k;
+  a.seqlen_q = p->seqlen_q; a.seqlen_k = p->seqlen_k; a.head_dim = p->head_dim;
+  a.n_mblk = (p->seqlen_q + 127) / 128;
+  a.n_splits = ns;
+  a.is_causal = p->is_causal ? 1 : 0;
+  a.neg_scale = p->scale < 0.f ? 1 : 0;
+  a.scale_log2 = (p->scale < 0.f ? -p->scale : p->scale) * kLog2e;
+  a.ws_o = nullptr;
+  a.ws_ml = nullptr;
+  if (ws && ns > 1) {
+    const size_t slots = (size_t)p->batch * p->heads_q * ns;
+    a.ws_o = (float*)ws;
+    a.ws_ml = (float*)((unsigned char*)ws + slots * (size_t)p->head_dim * 4);
+  }
+  return a;
+}
+
+template <typename T, int DP, int MINB>
+int launch_tile(const KArgs& a, hipStream_t st) {
+  constexpr int lds = 4 * 64 * DP * 2;
+  auto kfn = fa_tile_kernel<T, DP, MINB>;
+  if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+    (void)hipGetLastError();
+    return FA_ERR_LAUNCH;
+  }
+  const int64_t grid = (int64_t)a.batch * a.heads_q * a.n_mblk;
+  if (grid <= 0) return FA_OK;
+  if (grid > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(256), lds, st, a);
+  return hipGetLastError() == hipSuccess ? FA_OK : FA_ERR_LAUNCH;
+}
+
+template <typename T, int DP>
+int launch_splitkv(const KArgs& a, hipStream_t st) {
+  constexpr int lds = SplitCfg<DP>::LDS;
+  auto kfn = fa_splitkv_kernel<T, DP>;
+  if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+    (void)hipGetLastError();
+    return FA_ERR_LAUNCH;
+  }
+  const int64_t grid = (int64_t)a.batch * a.heads_k * a.n_splits;
+  if (grid > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(SplitCfg<DP>::NW * 64), lds, st, a);
+  if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
+  if (a.n_splits > 1) {
+    hipLaunchKernelGGL(fa_merge_kernel<T>, dim3((unsigned)(a.batch * a.heads_q)), dim3(64), 0, st, a);
+    if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
+  }
+  return FA_OK;
+}
+
+template <typename T>
+int dispatch(const KArgs& a, int kern, hipStream_t st) {
+  const int dp = padded_dim(a.head_dim);
+  if (kern == FA_KERNEL_SPLITKV) {
+    if (dp == 64) return launch_splitkv<T, 64>(a, st);
+    if (dp == 128) return launch_splitkv<T, 128>(a, st);
+    return launch_splitkv<T, 256>(a, st);
+  }
+  if (dp == 64) return launch_tile<T, 64, 2>(a, st);
+  if (dp == 128) return launch_tile<T, 128, 2>(a, st);
+  return launch_tile<T, 256, 1>(a, st);
+}
+
+}  // namespace
+
+extern "C" {
+
+int fa_fwd_version(void) { return FA_FWD_ABI_VERSION; }
+
+const char* fa_fwd_error_string(int rc) {
+  switch (rc) {
+    case FA_OK: return "ok";
+    case FA_ERR_BAD_ARG: return "bad argument (null pointer, non-positive size, misaligned pointer or stride, short workspace)";
+    case FA_ERR_UNSUPPORTED: return "unsupported shape or dtype";
+    case FA_ERR_LAUNCH: return "HIP launch failure";
+    default: return "unknown error";
+  }
+}
+
+int fa_fwd_validate(const fa_fwd_params* p) { return validate(p); }
+
+int fa_fwd_plan(const fa_fwd_params* p, int32_t* kernel, int32_t* num_splits) {
+  const int rc = validate(p);
+  if (rc != FA_OK) return rc;
+  int k, s;
+  plan(p, &k, &s);
+  if (kernel) *kernel = k;
+  if (num_splits) *num_splits = s;
+  return FA_OK;
+}
+
+size_t fa_fwd_workspace_bytes(const fa_fwd_params* p) {
+  if (validate(p) != FA_OK) return 0;
+  int k, s;
+  plan(p, &k, &s);
+  return workspace_bytes(p, k, s);
+}
+
+int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_bytes_given, void* stream) {
+  const int rc = validate(p);
+  if (rc != FA_OK) return rc;
+  int kern, ns;
+  plan(p, &kern, &ns);
+  const size_t need = workspace_bytes(p, kern, ns);
+  if (need > 0 && (!workspace || workspace_bytes_given < need || ((uintptr_t)workspace & 15))) return FA_ERR_BAD_ARG;
+  if (p->seqlen_q == 0) return FA_OK;  // nothing to write
+  const KArgs a = make_args(p, ns, workspace);
+  hipStream_t st = (hipStream_t)stream;
+  return p->dtype == FA_DTYPE_BF16 ? dispatch<__bf16>(a, kern, st) : dispatch<_Float16>(a, kern, st);
+}
+
+}  // extern "C"
