@@ -1,0 +1,163 @@
+"""CPU restatement of the reference's attention oracle.  TEST INFRASTRUCTURE ONLY — never imported by the product.
+
+What is restated, and from where (paths under the reference tree):
+
+* `construct_local_mask`  test/torch_ops/test_scaled_dot_product_attention.py:46-75
+      causal mask, bottom-right aligned: column j of row i is masked iff  j > i + Lk - Lq.
+* `attention_ref`         test/torch_ops/test_scaled_dot_product_attention.py:78-161
+      upcast -> GQA by repeating each kv head g times ("b s h d -> b s (h g) d", :119-120, i.e. query head h uses
+      kv head h // g) -> scores = (q / sqrt(d) or q * scale) k^T -> mask -> softmax -> rows with no visible key
+      set to 0 (:142-146) -> P V.
+* `get_tolerances`        test/torch_ops/test_scaled_dot_product_attention.py:166-204
+* default scale           torch_mlu/csrc/aten/operators/cnnl/transformers/sdp_utils.h:40-47 (1/sqrt(D))
+* what the vendor kernel is asked for: fp32 compute, causal-or-none mask, packed (cu_seqlens) mode
+                          torch_mlu/csrc/aten/operators/cnnl/internal/FlashAttention_internal.cpp:147-161
+* LSE buffer layout [Hq, total_q] in packed mode
+                          torch_mlu/csrc/aten/operators/cnnl/internal/FlashAttention_internal.cpp:129
+
+The reference never checks logsumexp values; LSE here is the textbook  ln sum_j exp(scale q_i.k_j)  over visible j,
+pinned in tests/test_oracle.py against torch.logsumexp, against PyTorch's CPU flash op (which returns LSE) and
+against closed forms.  Convention for a row with no visible key: out = 0 (reference oracle, :142-146) and
+LSE = +inf (so that exp(score - LSE) is 0 for every column).
+
+All functions take numpy arrays or torch tensors (any float dtype) and compute in float64 unless told otherwise.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import numpy as np
+
+# test/torch_ops/test_scaled_dot_product_attention.py:164-165 (keys are dtype names here)
+default_atol = {"float16": 1e-3, "bfloat16": 1e-3, "float32": 1e-5}
+default_rtol = {"float16": 1e-3, "bfloat16": 1.6e-2, "float32": 1.3e-6}
+
+
+def _np(x, dtype=np.float64) -> np.ndarray:
+    try:
+        import torch
+
+        if isinstance(x, torch.Tensor):
+            return x.detach().to("cpu").to(torch.float64).numpy().astype(dtype, copy=False)
+    except ImportError:  # pragma: no cover
+        pass
+    return np.asarray(x).astype(dtype, copy=False)
+
+
+def construct_local_mask(seqlen_q: int, seqlen_k: int, window_size=(-1, -1)) -> np.ndarray:
+    """True where masked.  Restates test_scaled_dot_product_attention.py:46-75 without padding masks."""
+    row = np.arange(seqlen_q, dtype=np.int64)[:, None]
+    col = np.arange(seqlen_k, dtype=np.int64)[None, :]
+    sk, sq = seqlen_k, seqlen_q
+    if window_size[0] < 0:
+        return col > row + sk - sq + window_size[1]
+    return np.logical_or(col > np.minimum(row + sk - sq + window_size[1], sk), col < row + sk - sq - window_size[0])
+
+
+def attention_ref(q, k, v, scale: Optional[float] = None, causal: bool = False, dtype=np.float64
+                  ) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
+    """q [B, Sq, Hq, D], k/v [B, Sk, Hk, D]  (the reference oracle's layout, :94-97).
+
+    Returns (output [B, Hq, Sq, D], attention [B, Hq, Sq, Sk], lse [B, Hq, Sq]) — the first two are what the
+    reference's `attention_ref` returns (:103-105, :161); lse is added.
+    """
+    q, k, v = _np(q, dtype), _np(k, dtype), _np(v, dtype)
+    B, Sq, Hq, D = q.shape
+    Sk, Hk = k.shape[1], k.shape[2]
+    assert Hq % Hk == 0
+    g = Hq // Hk
+    window = (-1, 0) if causal else (-1, -1)  # :110-111
+    k = np.repeat(k, g, axis=2)  # "b s h d -> b s (h g) d": head h*g+j <- kv head h
+    v = np.repeat(v, g, axis=2)
+    inv = math.sqrt(D) if scale is None else (1.0 / scale) if scale != 0 else math.inf  # :122
+    qs = q / inv if scale != 0 else q * 0.0
+    qh = np.ascontiguousarray(qs.transpose(0, 2, 1, 3))  # [B,H,Sq,D]
+    kh = np.ascontiguousarray(k.transpose(0, 2, 3, 1))   # [B,H,D,Sk]
+    vh = np.ascontiguousarray(v.transpose(0, 2, 1, 3))   # [B,H,Sk,D]
+    scores = np.matmul(qh, kh)                           # einsum("bthd,bshd->bhts")
+    masked_rows = None
+    if window[0] >= 0 or window[1] >= 0:
+        mask = construct_local_mask(Sq, Sk, window)
+        scores = np.where(mask[None, None], -np.inf, scores)
+        masked_rows = mask.all(axis=-1)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        m = scores.max(axis=-1, keepdims=True) if Sk > 0 else np.full(scores.shape[:-1] + (1,), -np.inf)
+        m_safe = np.where(np.isfinite(m), m, 0.0)
+        e = np.exp(scores - m_safe)
+        s = e.sum(axis=-1, keepdims=True)
+        attention = np.where(s > 0, e / np.where(s > 0, s, 1.0), 0.0)  # fully masked rows -> 0 (:142-146)
+        lse = np.where(s[..., 0] > 0, m_safe[..., 0] + np.log(np.where(s[..., 0] > 0, s[..., 0], 1.0)), np.inf)
+    if masked_rows is not None and masked_rows.any():
+        attention[:, :, masked_rows, :] = 0.0
+        lse[:, :, masked_rows] = np.inf
+    output = np.matmul(attention, vh)                    # einsum("bhts,bshd->bthd") then transpose(1,2)
+    return output, attention, lse
+
+
+def sdpa_oracle(q, k, v, is_causal: bool = False, scale: Optional[float] = None, dtype=np.float64
+                ) -> Tuple[np.ndarray, np.ndarray]:
+    """Dense op layout: q [B, Hq, Sq, D], k/v [B, Hk, Sk, D] -> (out [B, Hq, Sq, D], lse [B, Hq, Sq]).
+
+    The [B,H,S,D] -> [B,S,H,D] transposes are the ones the reference's dense wrapper makes
+    (torch_mlu/csrc/aten/operators/cnnl/transformers/attention.cpp:105-107) before the kernel.
+    """
+    q, k, v = _np(q, dtype), _np(k, dtype), _np(v, dtype)
+    out, _, lse = attention_ref(q.transpose(0, 2, 1, 3), k.transpose(0, 2, 1, 3), v.transpose(0, 2, 1, 3),
+                                scale=scale, causal=is_causal, dtype=dtype)
+    return out, lse
+
+
+def varlen_oracle(q, k, v, cu_seqlens_q, cu_seqlens_k, is_causal: bool = False, scale: Optional[float] = None,
+                  dtype=np.float64) -> Tuple[np.ndarray, np.ndarray]:
+    """Packed op layout: q [Tq, Hq, D], k/v [Tk, Hk, D], cu_seqlens [B+1] -> (out [Tq, Hq, D], lse [Hq, Tq]).
+
+    Sequence b owns rows [cu[b], cu[b+1]); each sequence is an independent dense problem — what "pack mode"
+    means for the vendor call (FlashAttention_internal.cpp:147-161) and what the reference's padding-mask oracle
+    computes per batch entry (test_scaled_dot_product_attention.py:55-66).
+    """
+    q, k, v = _np(q, dtype), _np(k, dtype), _np(v, dtype)
+    cq = np.asarray(cu_seqlens_q.cpu() if hasattr(cu_seqlens_q, "cpu") else cu_seqlens_q, dtype=np.int64)
+    ck = np.asarray(cu_seqlens_k.cpu() if hasattr(cu_seqlens_k, "cpu") else cu_seqlens_k, dtype=np.int64)
+    Tq, Hq, D = q.shape
+    out = np.zeros((Tq, Hq, D), dtype=dtype)
+    lse = np.full((Hq, Tq), np.inf, dtype=dtype)
+    for b in range(len(cq) - 1):
+        q0, q1, k0, k1 = cq[b], cq[b + 1], ck[b], ck[b + 1]
+        if q1 <= q0:
+            continue
+        o, _, l = attention_ref(q[None, q0:q1], k[None, k0:k1], v[None, k0:k1], scale=scale, causal=is_causal,
+                                dtype=dtype)
+        out[q0:q1] = o[0].transpose(1, 0, 2)
+        lse[:, q0:q1] = l[0]
+    return out, lse
+
+
+def get_tolerances(true_value, computed_value, dtype_name: str, fudge_factor: Optional[float] = 2.0
+                   ) -> Tuple[float, float]:
+    """Restates test_scaled_dot_product_attention.py:166-204: the allowed error is `fudge_factor` times the error
+    of doing the same math naively in the low-precision dtype, floored at the dtype's default."""
+    t, c = _np(true_value), _np(computed_value)
+    fudge = fudge_factor if fudge_factor is not None else 1.0
+    dev = t - c
+    atol = float(np.abs(dev).max()) if dev.size else 0.0
+    with np.errstate(invalid="ignore", divide="ignore"):
+        rel = np.abs(dev / t)
+    rel = np.where(np.isnan(rel), default_rtol[dtype_name], rel)
+    rtol = float(rel.max()) if rel.size else 0.0
+    atol = fudge * max(atol, default_atol[dtype_name])
+    rtol = fudge * max(rtol, default_rtol[dtype_name])
+    if rtol > 1e30:
+        rtol = default_rtol[dtype_name]
+    return atol, rtol
+
+
+def cpu_sdpa_flash(q, k, v, is_causal: bool = False, scale: Optional[float] = None):
+    """PyTorch's own CPU flash SDPA (`aten::_scaled_dot_product_flash_attention_for_cpu`), torch tensors in
+    [B, H, S, D] with Hq == Hk.  A library routine used (a) to pin the restatement above and (b) as the CPU
+    baseline that bench.py times next to the GPU kernel.  Returns (out, lse [B, H, Sq])."""
+    import torch
+
+    out, lse = torch.ops.aten._scaled_dot_product_flash_attention_for_cpu(q, k, v, 0.0, is_causal, attn_mask=None,
+                                                                         scale=scale)
+    return out, lse

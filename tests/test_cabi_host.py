@@ -1,0 +1,126 @@
+"""Host-only checks of the C ABI (include/fa_fwd.h / libfa_fwd.so): the library loads, exports every declared
+symbol, and its argument validation / planning — which never touch the GPU — return the documented codes."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from torch_mlu_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "fa_fwd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fa_fwd_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    syms = _declared_symbols()
+    assert syms == sorted(capi.EXPORTED_SYMBOLS)
+    L = ctypes.CDLL(capi.LIB_PATH)
+    for s in syms:
+        assert hasattr(L, s), s
+
+
+def test_version_and_error_strings():
+    L = capi.lib()
+    assert L.fa_fwd_version() == 1
+    assert capi.error_string(0) == "ok"
+    for rc in (-1, -2, -3, -99):
+        assert capi.error_string(rc)
+
+
+def _good(**over):
+    """A syntactically valid params struct with fake (aligned, never dereferenced) device addresses."""
+    p = capi.FaFwdParams()
+    p.q, p.k, p.v, p.out, p.lse = 0x1000, 0x2000, 0x3000, 0x4000, 0x5000
+    B, Hq, Hk, Sq, Sk, D = 2, 8, 2, 128, 256, 128
+    p.q_stride_b, p.q_stride_s, p.q_stride_h = Sq * Hq * D, Hq * D, D
+    p.k_stride_b, p.k_stride_s, p.k_stride_h = Sk * Hk * D, Hk * D, D
+    p.v_stride_b, p.v_stride_s, p.v_stride_h = Sk * Hk * D, Hk * D, D
+    p.o_stride_b, p.o_stride_s, p.o_stride_h = Sq * Hq * D, Hq * D, D
+    p.lse_stride_b, p.lse_stride_h, p.lse_stride_s = Hq * Sq, Sq, 1
+    p.batch, p.heads_q, p.heads_k, p.seqlen_q, p.seqlen_k, p.head_dim = B, Hq, Hk, Sq, Sk, D
+    p.scale, p.dtype, p.is_causal, p.kernel, p.num_splits, p.reserved = 0.088, capi.FA_DTYPE_BF16, 1, 0, 0, 0
+    for k, v in over.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_validate_accepts_good_params():
+    assert capi.lib().fa_fwd_validate(ctypes.byref(_good())) == capi.FA_OK
+    assert capi.lib().fa_fwd_validate(ctypes.byref(_good(dtype=capi.FA_DTYPE_FP16, head_dim=64))) == capi.FA_OK
+
+
+@pytest.mark.parametrize("over,rc", [
+    (dict(q=None), capi.FA_ERR_BAD_ARG),
+    (dict(out=None), capi.FA_ERR_BAD_ARG),
+    (dict(lse=None), capi.FA_ERR_BAD_ARG),
+    (dict(q=0x1008), capi.FA_ERR_BAD_ARG),              # not 16-byte aligned
+    (dict(k_stride_s=130), capi.FA_ERR_BAD_ARG),        # rows not 16-byte aligned
+    (dict(q_stride_h=-128), capi.FA_ERR_BAD_ARG),
+    (dict(batch=0), capi.FA_ERR_BAD_ARG),               # "batch size must be positive"
+    (dict(heads_k=0), capi.FA_ERR_BAD_ARG),
+    (dict(reserved=1), capi.FA_ERR_BAD_ARG),
+    (dict(num_splits=65), capi.FA_ERR_BAD_ARG),
+    (dict(kernel=7), capi.FA_ERR_BAD_ARG),
+    (dict(cu_seqlens_q=0x6000), capi.FA_ERR_BAD_ARG),   # only one of the two cu_seqlens
+    (dict(dtype=5), capi.FA_ERR_UNSUPPORTED),           # "only support fp16 and bf16"
+    (dict(head_dim=264), capi.FA_ERR_UNSUPPORTED),      # "head dimension at most 256"
+    (dict(head_dim=100), capi.FA_ERR_UNSUPPORTED),      # not a multiple of 8
+    (dict(heads_k=3), capi.FA_ERR_UNSUPPORTED),         # "must divide number of heads in query"
+    (dict(kernel=capi.FA_KERNEL_SPLITKV), capi.FA_ERR_UNSUPPORTED),  # split-KV needs seqlen_q == 1
+])
+def test_validate_rejects(over, rc):
+    p = _good(**over)
+    L = capi.lib()
+    assert L.fa_fwd_validate(ctypes.byref(p)) == rc
+    assert L.fa_fwd_workspace_bytes(ctypes.byref(p)) == 0
+    # launch refuses before touching the device
+    assert L.fa_fwd_launch(ctypes.byref(p), None, 0, None) == rc
+
+
+def test_null_params():
+    L = capi.lib()
+    assert L.fa_fwd_validate(None) == capi.FA_ERR_BAD_ARG
+    assert L.fa_fwd_workspace_bytes(None) == 0
+    assert L.fa_fwd_launch(None, None, 0, None) == capi.FA_ERR_BAD_ARG
+
+
+def _plan(p):
+    k, s = ctypes.c_int32(-1), ctypes.c_int32(-1)
+    rc = capi.lib().fa_fwd_plan(ctypes.byref(p), ctypes.byref(k), ctypes.byref(s))
+    return rc, k.value, s.value
+
+
+def test_plan_prefill_uses_tile_kernel_without_workspace():
+    p = _good()
+    assert _plan(p) == (capi.FA_OK, capi.FA_KERNEL_TILE, 1)
+    assert capi.lib().fa_fwd_workspace_bytes(ctypes.byref(p)) == 0
+
+
+def test_plan_decode_uses_splitkv_and_sizes_workspace():
+    """BASELINE config 5 shape: B=64, Hq=32, Hkv=8, Sq=1, Skv=8192, D=128."""
+    p = _good(batch=64, heads_q=32, heads_k=8, seqlen_q=1, seqlen_k=8192, is_causal=0)
+    rc, kern, ns = _plan(p)
+    assert rc == capi.FA_OK and kern == capi.FA_KERNEL_SPLITKV and 1 <= ns <= capi.FA_MAX_SPLITS
+    need = capi.lib().fa_fwd_workspace_bytes(ctypes.byref(p))
+    assert need == (0 if ns == 1 else 64 * 32 * ns * (128 * 4 + 8))
+    # a short or missing workspace is refused on the host
+    if need:
+        assert capi.lib().fa_fwd_launch(ctypes.byref(p), None, 0, None) == capi.FA_ERR_BAD_ARG
+        assert capi.lib().fa_fwd_launch(ctypes.byref(p), 0x7000, need - 1, None) == capi.FA_ERR_BAD_ARG
+    # explicit split count is honoured and capped by the number of 32-row blocks
+    p.num_splits = 4
+    assert _plan(p) == (capi.FA_OK, capi.FA_KERNEL_SPLITKV, 4)
+    p.seqlen_k, p.num_splits, p.kernel = 40, 8, capi.FA_KERNEL_SPLITKV
+    assert _plan(p) == (capi.FA_OK, capi.FA_KERNEL_SPLITKV, 2)
+    # short KV: the automatic choice is the tile kernel
+    p.kernel = capi.FA_KERNEL_AUTO
+    assert _plan(p)[1] == capi.FA_KERNEL_TILE
+    # wide GQA groups (> 16 query heads per kv head) fall back to the tile kernel
+    p = _good(batch=1, heads_q=32, heads_k=1, seqlen_q=1, seqlen_k=4096)
+    assert _plan(p)[1] == capi.FA_KERNEL_TILE

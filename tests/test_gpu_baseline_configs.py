@@ -1,0 +1,124 @@
+"""BASELINE.json configs 2-5 at full size on the GPU: all heads against an fp32 math reference on the device, sampled
+heads against the CPU oracle, plus size-independent properties (Q = 0 -> running mean of V and LSE = ln n; split-KV
+== tile kernel)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import torch_mlu_amd
+from tests._gpu_ref import sdpa_fp32
+from tests._util import LSE_TOL, OUT_TOL, lse_close, out_close, seeded
+from torch_mlu_amd import capi
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF, HF = torch.bfloat16, torch.float16
+
+
+def _full_check(q, k, v, causal, out, lse, sample):
+    ro, rl = sdpa_fp32(q, k, v, causal)
+    err = (out.float() - ro).abs().max().item()
+    lerr = (lse - rl).abs().max().item()
+    assert err <= OUT_TOL[q.dtype], err
+    assert lerr <= LSE_TOL, lerr
+    for (b, h) in sample:
+        g = q.shape[1] // k.shape[1]
+        oo, ol = oracle.sdpa_oracle(q[b:b + 1, h:h + 1].cpu(), k[b:b + 1, h // g:h // g + 1].cpu(),
+                                    v[b:b + 1, h // g:h // g + 1].cpu(), is_causal=causal)
+        out_close(out[b:b + 1, h:h + 1].float().cpu().numpy(), oo, q.dtype)
+        lse_close(lse[b:b + 1, h:h + 1].cpu().numpy(), ol)
+    return err, lerr
+
+
+def test_config2_causal_prefill_bf16_mha():
+    """B=4, Hq=Hkv=32, S=4096, D=128, causal, N(0, 0.5^2) bf16, through F.scaled_dot_product_attention."""
+    B, H, S, D = 4, 32, 4096, 128
+    q, k, v = (seeded((B, H, S, D), 1 + i, BF).to(DEV) for i in range(3))
+    n0 = torch_mlu_amd.launch_count()
+    out = torch_mlu_amd.sdpa(q, k, v, is_causal=True)
+    assert torch_mlu_amd.launch_count() == n0 + 1
+    _, lse, *_ = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False)
+    err, lerr = _full_check(q, k, v, True, out, lse, [(0, 0), (3, 31)])
+    print(f"cfg2 max|dout|={err:.3e} max|dlse|={lerr:.3e}")
+    # property at full size: Q = 0 -> out[i] = mean(V[:i+1]), LSE[i] = ln(i+1)
+    out0, lse0, *_ = torch.ops.aten._scaled_dot_product_flash_attention(torch.zeros_like(q), k, v, 0.0, True, False)
+    n = torch.arange(1, S + 1, device=DEV, dtype=torch.float32)
+    assert (lse0 - torch.log(n)[None, None]).abs().max().item() <= 1e-4
+    cm = torch.cumsum(v[:, :2].float(), dim=2) / n[None, None, :, None]
+    assert (out0[:, :2].float() - cm).abs().max().item() <= 2e-2
+
+
+def test_config3_causal_prefill_bf16_gqa():
+    """B=8, Hq=32, Hkv=8, S=2048, D=128, causal, through F.scaled_dot_product_attention(enable_gqa=True)."""
+    B, Hq, Hk, S, D = 8, 32, 8, 2048, 128
+    q = seeded((B, Hq, S, D), 2, BF).to(DEV)
+    k, v = seeded((B, Hk, S, D), 3, BF).to(DEV), seeded((B, Hk, S, D), 4, BF).to(DEV)
+    n0 = torch_mlu_amd.launch_count()
+    out = torch_mlu_amd.sdpa(q, k, v, is_causal=True, enable_gqa=True)
+    assert torch_mlu_amd.launch_count() == n0 + 1
+    _, lse, *_ = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False)
+    err, lerr = _full_check(q, k, v, True, out, lse, [(0, 5), (7, 30)])
+    print(f"cfg3 max|dout|={err:.3e} max|dlse|={lerr:.3e}")
+    # GQA == MHA over repeat_interleaved K/V
+    o2 = torch_mlu_amd.sdpa(q[:2], k[:2].repeat_interleave(4, dim=1), v[:2].repeat_interleave(4, dim=1), is_causal=True)
+    assert torch.equal(out[:2], o2)
+
+
+def test_config4_varlen_packed_causal_fp16():
+    """16 sequences, lengths ~U[256,2048] (seed 3), H=16, D=128, fp16, through _flash_attention_forward."""
+    g = torch.Generator().manual_seed(3)
+    lens = torch.randint(256, 2049, (16,), generator=g).tolist()
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    T, H, D = int(cu[-1]), 16, 128
+    q, k, v = (seeded((T, H, D), 30 + i, HF).to(DEV) for i in range(3))
+    cud = cu.to(DEV)
+    out, lse, seed, offset, dbg = torch.ops.aten._flash_attention_forward(q, k, v, cud, cud, max(lens), max(lens), 0.0,
+                                                                         True, False)
+    assert out.shape == (T, H, D) and lse.shape == (H, T)
+    worst = 0.0
+    for b, L in enumerate(lens):
+        s, e = int(cu[b]), int(cu[b + 1])
+        ro, rl = sdpa_fp32(q[s:e].transpose(0, 1)[None], k[s:e].transpose(0, 1)[None], v[s:e].transpose(0, 1)[None], True)
+        err = (out[s:e].transpose(0, 1)[None].float() - ro).abs().max().item()
+        worst = max(worst, err)
+        assert err <= OUT_TOL[HF], (b, L, err)
+        assert (lse[:, s:e][None] - rl).abs().max().item() <= LSE_TOL
+    # two sequences (the shortest and the longest) against the CPU oracle, all heads
+    for b in (int(np.argmin(lens)), int(np.argmax(lens))):
+        s, e = int(cu[b]), int(cu[b + 1])
+        oo, ol = oracle.varlen_oracle(q[s:e].cpu(), k[s:e].cpu(), v[s:e].cpu(), [0, e - s], [0, e - s], is_causal=True)
+        out_close(out[s:e].float().cpu().numpy(), oo, HF)
+        lse_close(lse[:, s:e].cpu().numpy(), ol)
+    print(f"cfg4 T={T} max|dout|={worst:.3e}")
+
+
+def test_config5_decode_bf16_gqa():
+    """B=64, Hq=32, Hkv=8, Sq=1, Skv=8192, D=128, non-causal, through F.scaled_dot_product_attention(enable_gqa=True)."""
+    B, Hq, Hk, Sk, D = 64, 32, 8, 8192, 128
+    q = seeded((B, Hq, 1, D), 4, BF).to(DEV)
+    k, v = seeded((B, Hk, Sk, D), 5, BF).to(DEV), seeded((B, Hk, Sk, D), 6, BF).to(DEV)
+    n0 = torch_mlu_amd.launch_count()
+    out = torch_mlu_amd.sdpa(q, k, v, enable_gqa=True)
+    assert torch_mlu_amd.launch_count() == n0 + 1
+    _, lse, *_ = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, 0.0, False, False)
+    # fp32 reference, vectorised over the batch: scores [B, Hq, Sk]
+    kk = k.float().repeat_interleave(4, dim=1)
+    s = torch.einsum("bhd,bhsd->bhs", q[:, :, 0].float(), kk) / math.sqrt(D)
+    rl = torch.logsumexp(s, -1)
+    ro = torch.einsum("bhs,bhsd->bhd", torch.softmax(s, -1), v.float().repeat_interleave(4, dim=1))
+    err = (out[:, :, 0].float() - ro).abs().max().item()
+    lerr = (lse[:, :, 0] - rl).abs().max().item()
+    assert err <= OUT_TOL[BF] and lerr <= LSE_TOL, (err, lerr)
+    for (b, h) in ((0, 0), (63, 31), (17, 9)):
+        oo, ol = oracle.sdpa_oracle(q[b:b + 1, h:h + 1].cpu(), k[b:b + 1, h // 4:h // 4 + 1].cpu(),
+                                    v[b:b + 1, h // 4:h // 4 + 1].cpu())
+        out_close(out[b:b + 1, h:h + 1].float().cpu().numpy(), oo, BF)
+        lse_close(lse[b:b + 1, h:h + 1].cpu().numpy(), ol)
+    # the automatic plan is the split-KV kernel; the tile kernel gives the same answer
+    o_tile, l_tile = capi.fa_forward_dense(q[:4], k[:4], v[:4], kernel=capi.FA_KERNEL_TILE)
+    assert (o_tile.float() - out[:4].float()).abs().max().item() <= 4e-3
+    assert (l_tile - lse[:4]).abs().max().item() <= 1e-4
+    print(f"cfg5 max|dout|={err:.3e} max|dlse|={lerr:.3e}")

@@ -1,0 +1,317 @@
+// ATen extension: registers `_scaled_dot_product_flash_attention` and `_flash_attention_forward` for HIP tensors
+// and hands them to the C-ABI launcher in libfa_fwd.so.
+//
+// Host-side mirror of torch_mlu's op layer for this path:
+//   cnnl__scaled_dot_product_flash_attention  torch_mlu/csrc/aten/operators/cnnl/transformers/attention.cpp:48-159
+//   cnnl__flash_attention_forward             torch_mlu/csrc/aten/operators/cnnl/transformers/attention.cpp:161-203
+//   mha_varlen_fwd (validation + launch)      torch_mlu/csrc/aten/operators/cnnl/internal/FlashAttention_internal.cpp:57-267
+//   generated dispatcher wrapper              codegen/dest/gen_external_mlu.py:483-549 (device guard)
+//   registration                              codegen/templates/RegisterMLU.cpp:185-187 (TORCH_LIBRARY_IMPL)
+//
+// Differences from the reference, all forced by the installed PyTorch or by the no-copy design:
+//   * the schemas are the installed PyTorch's (optional cum_seq, window/alibi/seqused arguments that must be
+//     unset); the tuple positions and meanings are the reference's (codegen/mlu_functions.yaml:1313,1315);
+//   * Q/K/V are never copied: their strides go to the launcher (the reference makes up to three transposing
+//     copies at attention.cpp:124-129);
+//   * Hq may be a multiple of Hkv at the dense op too (the inner launcher already allowed it,
+//     FlashAttention_internal.cpp:122-124);
+//   * LSE is returned as [B, Hq, Sq] (dense) / [Hq, total_q] (packed) without the pad-to-16 of
+//     FlashAttention_internal.cpp:261-265, which is what the installed PyTorch's shape contract says.
+#include <ATen/ATen.h>
+#include <ATen/hip/HIPContext.h>
+#include <c10/hip/HIPGraphsC10Utils.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/core/DeviceGuard.h>
+#include <c10/util/Logging.h>
+#include <torch/library.h>
+
+#include <atomic>
+#include <cmath>
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "fa_fwd.h"
+
+namespace torch_mlu_amd {
+
+namespace {
+
+std::atomic<int64_t> g_launches{0};  // how many times this extension enqueued the HIP kernels (test hook)
+
+// sdp::calculate_scale, torch_mlu/csrc/aten/operators/cnnl/transformers/sdp_utils.h:40-47, then narrowed to float
+// as at attention.cpp:174-175.
+float resolve_scale(const at::Tensor& query, std::optional<double> scale) {
+  const double s = scale.has_value() ? *scale : 1.0 / std::sqrt(static_cast<double>(query.size(-1)));
+  return static_cast<float>(s);
+}
+
+struct Packed {
+  const at::Tensor* cu_q;
+  const at::Tensor* cu_k;
+  int64_t max_q, max_k;
+};
+
+// The checks of mha_varlen_fwd (FlashAttention_internal.cpp:73-127) in the reference's order and wording.
+// `dense` inputs are [B, S, H, D] views, packed ones [T, H, D].
+void check_inputs(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const Packed* pk, bool require_device) {
+  const auto q_dtype = q.scalar_type();
+  TORCH_CHECK(q_dtype == at::kHalf || q_dtype == at::kBFloat16, "FlashAttention only support fp16 and bf16 data type");
+  TORCH_CHECK(k.scalar_type() == q_dtype, "query and key must have the same dtype");
+  TORCH_CHECK(v.scalar_type() == q_dtype, "query and value must have the same dtype");
+  if (pk) {
+    TORCH_CHECK(pk->cu_q->scalar_type() == at::kInt, "cu_seqlens_q must have dtype int32");
+    TORCH_CHECK(pk->cu_k->scalar_type() == at::kInt, "cu_seqlens_k must have dtype int32");
+  }
+  if (require_device) {
+    TORCH_CHECK(q.is_cuda(), "Input tensor must be on HIP device");
+    TORCH_CHECK(k.is_cuda(), "Input tensor must be on HIP device");
+    TORCH_CHECK(v.is_cuda(), "Input tensor must be on HIP device");
+    if (pk) {
+      TORCH_CHECK(pk->cu_q->is_cuda(), "cu_seqlens_q must be on HIP device");
+      TORCH_CHECK(pk->cu_k->is_cuda(), "cu_seqlens_k must be on HIP device");
+    }
+    TORCH_CHECK(k.device() == q.device() && v.device() == q.device(), "Input tensors must be on the same device");
+  }
+  TORCH_CHECK(q.dim() == (pk ? 3 : 4) && k.dim() == q.dim() && v.dim() == q.dim(),
+              pk ? "packed query, key and value must have shape (total, num_heads, head_size)"
+                 : "query, key and value must have shape (batch_size, seqlen, num_heads, head_size)");
+  TORCH_CHECK(q.stride(-1) == 1, "Input tensor must have contiguous last dimension");
+  TORCH_CHECK(k.stride(-1) == 1, "Input tensor must have contiguous last dimension");
+  TORCH_CHECK(v.stride(-1) == 1, "Input tensor must have contiguous last dimension");
+  if (pk) {
+    TORCH_CHECK(pk->cu_q->is_contiguous(), "cu_seqlens_q must be contiguous");
+    TORCH_CHECK(pk->cu_k->is_contiguous(), "cu_seqlens_k must be contiguous");
+  }
+  const int64_t batch = pk ? pk->cu_q->numel() - 1 : q.size(0);
+  const int64_t heads = q.size(-2), heads_k = k.size(-2), head_size = q.size(-1);
+  TORCH_CHECK(batch > 0, "batch size must be positive");
+  TORCH_CHECK(head_size <= 256, "FlashAttention forward only supports head dimension at most 256");
+  TORCH_CHECK(head_size % 8 == 0 && head_size > 0, "FlashAttention forward only supports head dimensions that are a multiple of 8");
+  TORCH_CHECK(heads_k > 0 && heads % heads_k == 0, "Number of heads in key/value must divide number of heads in query");
+  TORCH_CHECK(k.size(-1) == head_size && v.size(-1) == head_size, "query, key and value must have the same head dimension");
+  TORCH_CHECK(v.size(-2) == heads_k, "key and value must have the same number of heads");
+  if (pk) {
+    TORCH_CHECK(pk->cu_q->dim() == 1, "cu_seqlens_q must have shape (batch_size + 1)");
+    TORCH_CHECK(pk->cu_k->dim() == 1 && pk->cu_k->numel() == batch + 1, "cu_seqlens_k must have shape (batch_size + 1)");
+    TORCH_CHECK(k.size(0) == v.size(0), "Key and Value must have the same sequence length");
+    TORCH_CHECK(pk->max_q >= 0 && pk->max_k >= 0, "max_seqlen must be non-negative");
+  } else {
+    TORCH_CHECK(k.size(0) == batch && v.size(0) == batch, "query, key and value must have the same batch size");
+    TORCH_CHECK(k.size(1) == v.size(1), "Key and Value must have the same sequence length");
+  }
+}
+
+// 16-byte vector access needs 8-element-aligned rows; anything else gets one copy (never hit by dense layouts).
+at::Tensor aligned_or_copy(const at::Tensor& t) {
+  bool ok = reinterpret_cast<uintptr_t>(t.data_ptr()) % 16 == 0;
+  for (int64_t i = 0; i + 1 < t.dim(); ++i) ok = ok && (t.size(i) == 1 || (t.stride(i) % 8 == 0 && t.stride(i) >= 0));
+  if (ok) return t;
+  TORCH_WARN_ONCE("flash attention: input rows are not 16-byte aligned; making one contiguous copy");
+  return t.contiguous();
+}
+
+void fill_strides(const at::Tensor& t, bool packed, int64_t& sb, int64_t& ss, int64_t& sh) {
+  if (packed) {
+    sb = 0; ss = t.stride(0); sh = t.stride(1);
+  } else {
+    sb = t.stride(0); ss = t.stride(1); sh = t.stride(2);
+  }
+  // a size-1 dimension may carry any stride; keep it harmless for the launcher's alignment rule
+  if (!packed && t.size(0) == 1) sb = 0;
+  if (t.size(packed ? 0 : 1) == 1) ss = 0;
+  if (t.size(packed ? 1 : 2) == 1) sh = 0;
+}
+
+}  // namespace
+
+// ---- _flash_attention_forward ---------------------------------------------------------------------------------
+// cnnl__flash_attention_forward, attention.cpp:161-203.  cum_seq given: packed [T, H, D] inputs (the reference's
+// only mode); absent: dense [B, S, H, D] inputs (installed-PyTorch extension of the schema).
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> flash_attention_forward(
+    const at::Tensor& query, const at::Tensor& key, const at::Tensor& value,
+    const std::optional<at::Tensor>& cum_seq_q, const std::optional<at::Tensor>& cum_seq_k, int64_t max_q,
+    int64_t max_k, double dropout_p, bool is_causal, bool return_debug_mask, std::optional<double> scale,
+    std::optional<int64_t> window_size_left, std::optional<int64_t> window_size_right,
+    const std::optional<at::Tensor>& seqused_k, const std::optional<at::Tensor>& alibi_slopes) {
+  const bool packed = cum_seq_q.has_value() && cum_seq_q->defined();
+  TORCH_CHECK(packed == (cum_seq_k.has_value() && cum_seq_k->defined()),
+              "cum_seq_q and cum_seq_k must be given together");
+  TORCH_CHECK(dropout_p == 0.0, "flash attention forward: dropout_p > 0 is not supported by this build");
+  TORCH_CHECK(!window_size_left.has_value() || *window_size_left < 0, "flash attention forward: sliding window is not supported");
+  TORCH_CHECK(!window_size_right.has_value() || *window_size_right < 0 || (is_causal && *window_size_right == 0),
+              "flash attention forward: sliding window is not supported");
+  TORCH_CHECK(!(seqused_k.has_value() && seqused_k->defined()), "flash attention forward: seqused_k is not supported");
+  TORCH_CHECK(!(alibi_slopes.has_value() && alibi_slopes->defined()), "flash attention forward: alibi_slopes is not supported");
+
+  Packed pk{packed ? &*cum_seq_q : nullptr, packed ? &*cum_seq_k : nullptr, max_q, max_k};
+  check_inputs(query, key, value, packed ? &pk : nullptr, /*require_device=*/true);
+
+  // HIP tensors carry the "cuda" device type in PyTorch-ROCm: the generic guard resolves to the HIP implementation
+  const c10::OptionalDeviceGuard guard(query.device());
+  const float softmax_scale = resolve_scale(query, scale);
+
+  const at::Tensor q = aligned_or_copy(query), k = aligned_or_copy(key), v = aligned_or_copy(value);
+  // out = empty_like(query) over a contiguous query in the reference (attention.cpp:176): dense [B,S,H,D] storage
+  at::Tensor output = at::empty(q.sizes(), q.options());
+  const int64_t batch = packed ? cum_seq_q->numel() - 1 : q.size(0);
+  const int64_t heads = q.size(-2), head_size = q.size(-1);
+  const int64_t seqlen_q = packed ? max_q : q.size(1);
+  const int64_t seqlen_k = packed ? max_k : k.size(1);
+  const int64_t total_q = packed ? q.size(0) : batch * seqlen_q;
+  // kernel-side LSE buffer: [Hq, total_q] packed (FlashAttention_internal.cpp:129), [B, Hq, Sq] dense
+  at::Tensor lse = packed ? at::empty({heads, total_q}, q.options().dtype(at::kFloat))
+                          : at::empty({batch, heads, seqlen_q}, q.options().dtype(at::kFloat));
+  TORCH_CHECK(seqlen_q <= INT32_MAX && seqlen_k <= INT32_MAX && batch <= INT32_MAX, "sequence length too large");
+
+  fa_fwd_params p{};
+  p.q = q.data_ptr(); p.k = k.data_ptr(); p.v = v.data_ptr(); p.out = output.data_ptr();
+  p.lse = lse.data_ptr<float>();
+  p.cu_seqlens_q = packed ? cum_seq_q->data_ptr<int32_t>() : nullptr;
+  p.cu_seqlens_k = packed ? cum_seq_k->data_ptr<int32_t>() : nullptr;
+  fill_strides(q, packed, p.q_stride_b, p.q_stride_s, p.q_stride_h);
+  fill_strides(k, packed, p.k_stride_b, p.k_stride_s, p.k_stride_h);
+  fill_strides(v, packed, p.v_stride_b, p.v_stride_s, p.v_stride_h);
+  fill_strides(output, packed, p.o_stride_b, p.o_stride_s, p.o_stride_h);
+  if (packed) {
+    p.lse_stride_b = 0; p.lse_stride_h = lse.stride(0); p.lse_stride_s = lse.stride(1);
+  } else {
+    p.lse_stride_b = lse.stride(0); p.lse_stride_h = lse.stride(1); p.lse_stride_s = lse.stride(2);
+  }
+  p.batch = static_cast<int32_t>(batch);
+  p.heads_q = static_cast<int32_t>(heads);
+  p.heads_k = static_cast<int32_t>(k.size(-2));
+  p.seqlen_q = static_cast<int32_t>(seqlen_q);
+  p.seqlen_k = static_cast<int32_t>(seqlen_k);
+  p.head_dim = static_cast<int32_t>(head_size);
+  p.scale = softmax_scale;
+  p.dtype = q.scalar_type() == at::kBFloat16 ? FA_DTYPE_BF16 : FA_DTYPE_FP16;
+  p.is_causal = is_causal ? 1 : 0;
+  p.kernel = FA_KERNEL_AUTO;
+  p.num_splits = 0;
+
+  if (total_q > 0) {
+    // workspace: stream-ordered caching allocator, as the reference does (FlashAttention_internal.cpp:215-230)
+    const size_t ws_bytes = fa_fwd_workspace_bytes(&p);
+    at::Tensor ws;
+    if (ws_bytes) ws = at::empty({static_cast<int64_t>(ws_bytes)}, q.options().dtype(at::kByte));
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
+    const int rc = fa_fwd_launch(&p, ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, stream);
+    TORCH_CHECK(rc == FA_OK, "fa_fwd_launch failed: ", fa_fwd_error_string(rc), " (rc=", rc, ")");
+    g_launches.fetch_add(1, std::memory_order_relaxed);
+  }
+
+  // p == 0: the reference returns two uninitialised 0-d int64 tensors (FlashAttention_internal.cpp:211-213)
+  at::Tensor seed_t = at::empty({}, q.options().dtype(at::kLong));
+  at::Tensor offset_t = at::empty({}, q.options().dtype(at::kLong));
+  // return_debug_mask only has an effect with dropout (attention.cpp:178-199)
+  (void)return_debug_mask;
+  at::Tensor debug_attn_mask = at::empty({0}, q.options());
+  return std::make_tuple(output, lse, seed_t, offset_t, debug_attn_mask);
+}
+
+namespace {
+
+// Uniform prefix sums arange(0, (B+1) S, S) as the reference fabricates on every call (attention.cpp:109-119).
+// They are immutable, so one copy per (device, B, S) is kept; a miss costs one arange plus one stream sync so
+// that the cached tensor is safe on every stream afterwards.  While a HIP graph is being captured the cache is
+// bypassed (no sync, no allocation that outlives the capture).
+at::Tensor uniform_cu_seqlens(int64_t batch, int64_t seqlen, const at::Tensor& like) {
+  const auto opts = like.options().dtype(at::kInt);
+  auto make = [&] { return at::arange(0, (batch + 1) * seqlen, seqlen > 0 ? seqlen : 1, opts); };
+  if (seqlen == 0) return at::zeros({batch + 1}, opts);
+  if (c10::hip::currentStreamCaptureStatusMayInitCtx() != c10::hip::CaptureStatus::None) return make();
+  static std::mutex mu;
+  static std::map<std::tuple<int, int64_t, int64_t>, at::Tensor> cache;
+  const auto key = std::make_tuple(static_cast<int>(like.device().index()), batch, seqlen);
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = cache.find(key);
+  if (it != cache.end()) return it->second;
+  if (cache.size() >= 256) cache.clear();
+  at::Tensor t = make();
+  c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(like.device().index()).synchronize();
+  cache.emplace(key, t);
+  return t;
+}
+
+}  // namespace
+
+// ---- _scaled_dot_product_flash_attention ----------------------------------------------------------------------
+// cnnl__scaled_dot_product_flash_attention, attention.cpp:48-159.
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::SymInt, at::Tensor, at::Tensor, at::Tensor>
+scaled_dot_product_flash_attention(const at::Tensor& query, const at::Tensor& key, const at::Tensor& value,
+                                   double dropout_p, bool is_causal, bool return_debug_mask,
+                                   std::optional<double> scale) {
+  C10_LOG_API_USAGE_ONCE("torch.sdpa.flash_attention");  // attention.cpp:67
+  // attention.cpp:70-100
+  TORCH_CHECK(query.dim() == 4 && key.dim() == 4 && value.dim() == 4,
+              "query, key and value must be 4-dimensional (batch, num_heads, seq_len, head_dim)");
+  TORCH_CHECK(query.size(0) == key.size(0) && query.size(0) == value.size(0),
+              "query, key and value must have the same batch size");
+  TORCH_CHECK(key.size(2) == value.size(2), "Key and Value must have the same sequence length");
+  TORCH_CHECK(key.size(1) == value.size(1), "key and value must have the same number of heads");
+  // relaxed from equality (attention.cpp:82-83) to the divisibility the launcher already accepts
+  TORCH_CHECK(key.size(1) > 0 && query.size(1) % key.size(1) == 0,
+              "Number of heads in key/value must divide number of heads in query");
+  TORCH_CHECK(query.size(3) == key.size(3), "query and key must have the same head dimension");
+
+  const int64_t batch_size = query.size(0);
+  const int64_t max_seqlen_batch_q = query.size(2);
+  const int64_t max_seqlen_batch_k = key.size(2);
+
+  // [B,H,S,D] -> [B,S,H,D] views; no contiguous copies (attention.cpp:105-107 without :124-129)
+  const at::Tensor q_t = query.transpose(1, 2);
+  const at::Tensor k_t = key.transpose(1, 2);
+  const at::Tensor v_t = value.transpose(1, 2);
+
+  auto [attention, log_sumexp, philox_seed, philox_offset, debug_attn_mask] = at::_flash_attention_forward(
+      q_t, k_t, v_t, std::nullopt, std::nullopt, max_seqlen_batch_q, max_seqlen_batch_k, dropout_p, is_causal,
+      return_debug_mask, scale, std::nullopt, std::nullopt, std::nullopt, std::nullopt);
+
+  const at::Tensor cumulative_sequence_length_q = uniform_cu_seqlens(batch_size, max_seqlen_batch_q, query);
+  const at::Tensor cumulative_sequence_length_k = uniform_cu_seqlens(batch_size, max_seqlen_batch_k, query);
+
+  // [B,S,H,D] storage returned as the [B,H,S,D] view (attention.cpp:146-148)
+  attention = attention.transpose(1, 2);
+  return std::make_tuple(attention, log_sumexp, cumulative_sequence_length_q, cumulative_sequence_length_k,
+                         c10::SymInt(max_seqlen_batch_q), c10::SymInt(max_seqlen_batch_k), philox_seed,
+                         philox_offset, debug_attn_mask);
+}
+
+// ---- test hooks -----------------------------------------------------------------------------------------------
+int64_t launch_count() { return g_launches.load(std::memory_order_relaxed); }
+
+// Runs only the launcher's input checks; with require_device == false they can be exercised on CPU tensors.
+void validate_flash_inputs(const at::Tensor& query, const at::Tensor& key, const at::Tensor& value,
+                           const std::optional<at::Tensor>& cum_seq_q, const std::optional<at::Tensor>& cum_seq_k,
+                           int64_t max_q, int64_t max_k, bool require_device) {
+  const bool packed = cum_seq_q.has_value() && cum_seq_q->defined();
+  TORCH_CHECK(packed == (cum_seq_k.has_value() && cum_seq_k->defined()), "cum_seq_q and cum_seq_k must be given together");
+  Packed pk{packed ? &*cum_seq_q : nullptr, packed ? &*cum_seq_k : nullptr, max_q, max_k};
+  check_inputs(query, key, value, packed ? &pk : nullptr, require_device);
+}
+
+}  // namespace torch_mlu_amd
+
+// HIP tensors carry the CUDA dispatch key in PyTorch-ROCm; registering here replaces PyTorch's own kernels for
+// the two ops (the dispatcher prints one "overriding a previously registered kernel" warning per op).
+TORCH_LIBRARY_IMPL(aten, CUDA, m) {
+  m.impl("_scaled_dot_product_flash_attention", TORCH_FN(torch_mlu_amd::scaled_dot_product_flash_attention));
+  m.impl("_flash_attention_forward", TORCH_FN(torch_mlu_amd::flash_attention_forward));
+}
+
+TORCH_LIBRARY(torch_mlu_amd, m) {
+  m.def("_launch_count() -> int", &torch_mlu_amd::launch_count);
+  m.def(
+      "_validate_flash_inputs(Tensor query, Tensor key, Tensor value, Tensor? cum_seq_q, Tensor? cum_seq_k, "
+      "int max_q, int max_k, bool require_device) -> ()",
+      &torch_mlu_amd::validate_flash_inputs);
+  // the same two entry points under a private namespace, so that a test can call this build's implementation
+  // by name no matter what else is registered for the aten ops
+  m.def(
+      "_flash_attention_forward(Tensor query, Tensor key, Tensor value, Tensor? cum_seq_q, Tensor? cum_seq_k, "
+      "int max_q, int max_k, float dropout_p, bool is_causal, bool return_debug_mask, *, float? scale=None, "
+      "int? window_size_left=None, int? window_size_right=None, Tensor? seqused_k=None, Tensor? alibi_slopes=None) "
+      "-> (Tensor, Tensor, Tensor, Tensor, Tensor)",
+      &torch_mlu_amd::flash_attention_forward);
+}

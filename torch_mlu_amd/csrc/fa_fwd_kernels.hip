@@ -781,6 +781,9 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   a.is_causal = p->is_causal ? 1 : 0;
   a.neg_scale = p->scale < 0.f ? 1 : 0;
   a.scale_log2 = (p->scale < 0.f ? -p->scale : p->scale) * kLog2e;
+  // scale == 0: masked scores are -inf and -inf * 0 is NaN; a tiny positive factor keeps -inf masked and maps every
+  // finite score to (numerically) zero, which is the scale == 0 answer.
+  if (!(a.scale_log2 > 0.f)) a.scale_log2 = 1e-30f;
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
   if (ws && ns > 1) {
