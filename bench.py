@@ -1,0 +1,257 @@
+#!/usr/bin/env python3
+"""Benchmark of the flash-attention forward path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5] [--no-extras] [--no-cpu-baseline]
+
+A "step" is one call of the registered op on one batch of seeded synthetic input that is already resident in HBM.
+The headline workload is BASELINE.json configs[1] (causal prefill, bf16 MHA, B=4 H=32 S=4096 D=128); the other
+configs are timed as extras and the decode config (cfg5) carries the HBM roofline.  One JSON line is printed.
+
+FLOPs are algorithmic: 4*B*Hq*Sq*Sk*D, halved for causal (exp / max / rescale not counted).
+Decode bytes are K+V only: 2*B*Hkv*Sk*D*2.
+Peaks are MI355X's published dense figures (bf16/fp16 MFMA 2.5 PFLOP/s, HBM3E 8 TB/s).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+PEAK_MFMA_TFLOPS = 2500.0  # dense bf16 / fp16
+PEAK_HBM_GBS = 8000.0
+
+
+def seeded(shape, seed, dtype, std=0.5):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g, dtype=torch.float32) * std).to(dtype)
+
+
+def make_workload(name, dev):
+    """-> dict(call=callable doing one step, flops, bytes_kv, desc, check=callable returning (out_err, lse_err))."""
+    bf, hf = torch.bfloat16, torch.float16
+    aten = torch.ops.aten
+    if name in ("cfg2", "cfg3"):
+        if name == "cfg2":
+            B, Hq, Hk, S, D, seed = 4, 32, 32, 4096, 128, 1
+        else:
+            B, Hq, Hk, S, D, seed = 8, 32, 8, 2048, 128, 2
+        q = seeded((B, Hq, S, D), seed, bf).to(dev)
+        k = seeded((B, Hk, S, D), seed + 1, bf).to(dev)
+        v = seeded((B, Hk, S, D), seed + 2, bf).to(dev)
+
+        def call():
+            return aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False)
+
+        def check():
+            out, lse = call()[:2]
+            return _check_heads(q, k, v, out, lse, True, [(0, 0), (B - 1, Hq - 1)])
+
+        return dict(call=call, check=check, flops=4 * B * Hq * S * S * D / 2, bytes_kv=2 * B * Hk * S * D * 2,
+                    desc=f"causal prefill bf16 B={B} Hq={Hq} Hkv={Hk} S={S} D={D}", dtype="bf16", bound="mfma",
+                    kernel="fa_tile_kernel")
+    if name == "cfg4":
+        g = torch.Generator().manual_seed(3)
+        lens = torch.randint(256, 2049, (16,), generator=g).tolist()
+        cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+        T, H, D = int(cu[-1]), 16, 128
+        q, k, v = (seeded((T, H, D), 30 + i, hf).to(dev) for i in range(3))
+        cud = cu.to(dev)
+        mx = max(lens)
+
+        def call():
+            return aten._flash_attention_forward(q, k, v, cud, cud, mx, mx, 0.0, True, False)
+
+        def check():
+            out, lse = call()[:2]
+            b = int(np.argmax(lens))
+            s, e = int(cu[b]), int(cu[b + 1])
+            return _check_heads(q[s:e].transpose(0, 1)[None], k[s:e].transpose(0, 1)[None], v[s:e].transpose(0, 1)[None],
+                                out[s:e].transpose(0, 1)[None], lse[:, s:e][None], True, [(0, 0), (0, H - 1)])
+
+        return dict(call=call, check=check, flops=4096.0 * sum(L * L for L in lens), bytes_kv=2 * T * H * D * 2,
+                    desc=f"varlen packed causal fp16 16 seqs T={T} H={H} D={D}", dtype="fp16", bound="mfma",
+                    kernel="fa_tile_kernel")
+    if name == "cfg5":
+        B, Hq, Hk, Sk, D = 64, 32, 8, 8192, 128
+        q = seeded((B, Hq, 1, D), 4, bf).to(dev)
+        # rotate over 3 distinct K/V sets (6 GiB) so that no step can be served from the 256 MiB Infinity Cache
+        kvs = []
+        k0, v0 = seeded((B, Hk, Sk, D), 5, bf).to(dev), seeded((B, Hk, Sk, D), 6, bf).to(dev)
+        kvs.append((k0, v0))
+        for r in (1, 2):
+            kvs.append((torch.roll(k0, r, dims=0), torch.roll(v0, r, dims=0)))
+        state = {"i": 0}
+
+        def call():
+            kk, vv = kvs[state["i"] % 3]
+            state["i"] += 1
+            return aten._scaled_dot_product_flash_attention(q, kk, vv, 0.0, False, False)
+
+        def check():
+            out, lse = aten._scaled_dot_product_flash_attention(q, k0, v0, 0.0, False, False)[:2]
+            return _check_heads(q, k0, v0, out, lse, False, [(0, 0), (B - 1, Hq - 1)])
+
+        return dict(call=call, check=check, flops=4 * B * Hq * Sk * D, bytes_kv=2 * B * Hk * Sk * D * 2,
+                    desc=f"decode bf16 GQA B={B} Hq={Hq} Hkv={Hk} Sq=1 Skv={Sk} D={D}", dtype="bf16", bound="hbm",
+                    kernel="fa_splitkv_kernel")
+    raise SystemExit(f"unknown config {name}")
+
+
+@torch.no_grad()
+def _check_heads(q, k, v, out, lse, causal, heads):
+    """max-abs error of sampled (batch, head) pairs against fp32 math on the device."""
+    g = q.shape[1] // k.shape[1]
+    Sq, Sk, D = q.shape[2], k.shape[2], q.shape[3]
+    eo = el = 0.0
+    for b, h in heads:
+        s = (q[b, h].float() @ k[b, h // g].float().T) / math.sqrt(D)
+        if causal:
+            r = torch.arange(Sq, device=q.device)[:, None]
+            c = torch.arange(Sk, device=q.device)[None, :]
+            s.masked_fill_(c > r + Sk - Sq, float("-inf"))
+        l = torch.logsumexp(s, -1)
+        o = torch.exp(s - l[:, None]) @ v[b, h // g].float()
+        eo = max(eo, (out[b, h].float() - o).abs().max().item())
+        el = max(el, (lse[b, h] - l).abs().max().item())
+    return eo, el
+
+
+def time_steps(call, steps, warmup):
+    """Exactly `steps` timed calls between two device synchronisations; HIP events on the launch stream give the
+    per-step device time."""
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(steps):
+        call()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per = [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]
+    return wall_ms / steps, float(np.mean(per)), float(np.median(per)), float(np.min(per))
+
+
+def cpu_baseline(budget_s=12.0):
+    """PyTorch's own CPU SDPA (aten::_scaled_dot_product_flash_attention_for_cpu, reached through the oracle package)
+    on a bounded sample of the headline workload: cfg2's shape with fewer (batch, head) pairs."""
+    import oracle
+
+    S, D = 4096, 128
+    threads = torch.get_num_threads()
+    heads = 4
+    q, k, v = (seeded((1, heads, S, D), 1 + i, torch.bfloat16) for i in range(3))
+    t = time.perf_counter()
+    oracle.cpu_sdpa_flash(q, k, v, is_causal=True)
+    first = time.perf_counter() - t
+    # scale the sample towards the time budget (at most the full 128 (batch, head) pairs of cfg2)
+    heads = int(max(4, min(128, 4 * (budget_s / 2) / max(first, 1e-3))))
+    q, k, v = (seeded((1, heads, S, D), 1 + i, torch.bfloat16) for i in range(3))
+    oracle.cpu_sdpa_flash(q, k, v, is_causal=True)  # warm-up
+    runs = []
+    for _ in range(2):
+        t = time.perf_counter()
+        oracle.cpu_sdpa_flash(q, k, v, is_causal=True)
+        runs.append(time.perf_counter() - t)
+    sec = min(runs)
+    flops = 4 * heads * S * S * D / 2
+    return {"value": flops / sec / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"PyTorch CPU SDPA (flash_attention_for_cpu), cfg2 shape, {heads} of 128 (batch, head) pairs, "
+                      f"bf16 causal S=4096 D=128, best of 2, {sec:.2f} s; os.cpu_count()={os.cpu_count()}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path needs no exchange between GPUs); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; there is no CPU path to time", file=sys.stderr)
+        sys.exit(2)
+
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import torch_mlu_amd  # registers the ops; raises if the HIP extension is missing
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    def run(name, steps, warmup):
+        w = make_workload(name, dev)
+        n0 = torch_mlu_amd.launch_count()
+        eo, el = w["check"]()
+        wall, ev_mean, ev_med, ev_min = time_steps(w["call"], steps, warmup)
+        assert torch_mlu_amd.launch_count() >= n0 + steps + warmup, "the registered HIP path did not run"
+        r = {"config": name, "workload": w["desc"], "ms_per_step": wall, "kernel_ms_mean": ev_mean,
+             "kernel_ms_median": ev_med, "kernel_ms_min": ev_min, "tflops": w["flops"] / wall / 1e9,
+             "kv_gbs": w["bytes_kv"] / wall / 1e6, "max_abs_err_out": eo, "max_abs_err_lse": el, "dtype": w["dtype"]}
+        if w["bound"] == "mfma":
+            ach = w["flops"] / ev_mean / 1e9
+            r["roofline"] = {"bound": "mfma", "kernel": w["kernel"], "achieved": ach, "peak": PEAK_MFMA_TFLOPS,
+                             "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_TFLOPS, "traffic": None}
+        else:
+            ach = w["bytes_kv"] / ev_mean / 1e6
+            r["roofline"] = {"bound": "hbm", "kernel": w["kernel"], "achieved": ach, "peak": PEAK_HBM_GBS,
+                             "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None}
+        del w
+        torch.cuda.empty_cache()
+        return r
+
+    main_r = run(args.config, args.steps, args.warmup)
+    extras = []
+    if not args.no_extras:
+        for name in ("cfg2", "cfg3", "cfg4", "cfg5"):
+            if name != args.config:
+                extras.append(run(name, args.steps, args.warmup))
+
+    is_decode = args.config == "cfg5"
+    line = {
+        "metric": "fwd attn TFLOP/s + % MFMA peak (bf16 S=4096 D=128); decode HBM GB/s",
+        "value": main_r["kv_gbs"] if is_decode else main_r["tflops"],
+        "unit": "GB/s" if is_decode else "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_r["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": main_r["dtype"],
+        "data": "synthetic (seeded N(0, 0.5^2), generated on the CPU in fp32 and cast)",
+        "config": {"workload": main_r["workload"], "name": args.config, "entry": "aten::_scaled_dot_product_flash_attention"
+                   if args.config != "cfg4" else "aten::_flash_attention_forward"},
+        "roofline": main_r["roofline"],
+        "parity": {"max_abs_err_out": main_r["max_abs_err_out"], "max_abs_err_lse": main_r["max_abs_err_lse"],
+                   "against": "fp32 math on the device, 2 sampled (batch, head) pairs"},
+        "peaks": {"mfma_tflops": PEAK_MFMA_TFLOPS, "hbm_gbs": PEAK_HBM_GBS,
+                  "device": torch.cuda.get_device_properties(0).gcnArchName,
+                  "cus": torch.cuda.get_device_properties(0).multi_processor_count},
+    }
+    if extras:
+        line["other_configs"] = extras
+        dec = [e for e in extras if e["config"] == "cfg5"]
+        if dec:
+            line["decode"] = {"value": dec[0]["kv_gbs"], "unit": "GB/s", "ms_per_step": dec[0]["ms_per_step"],
+                              "roofline": dec[0]["roofline"]}
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
