@@ -110,6 +110,15 @@ __device__ __forceinline__ void dma16(const unsigned char* gptr, unsigned char* 
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds), "v"(gptr) : "memory", "m0");
 }
 
+// Same, with the global address split into a wavefront-uniform 64-bit base (scalar registers) and a per-lane
+// 32-bit byte offset, and the LDS destination given as a wavefront-uniform LDS byte address.
+__device__ __forceinline__ void dma16s(const unsigned char* sbase, unsigned voff, unsigned lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_wave_base), "v"(voff), "s"(sbase)
+               : "m0");
+}
+
 // Transposed LDS read: within each group of 16 lanes, lane j receives element (j % 4) of the four 8-byte pieces
 // addressed by lanes 4 i + j / 4 (i = 0..3) of the same group.
 __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
@@ -150,6 +159,23 @@ __device__ __forceinline__ int swzV(int row) {
   if constexpr (DP == 64) return ((row >> 1) & 1) << 2;
   return (row & 3) << 2;
 }
+
+template <int N>
+struct IC {
+  static constexpr int value = N;
+};
+
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+// A new row maximum only forces a rescale of the accumulators when it exceeds the one in use by more than this
+// many powers of two; until then probabilities are formed against the older maximum and may reach 2^kLazyLog2,
+// which fp32 sums and fp16/bf16 P operands hold without loss.  The final out = O / l and LSE = m c + log2 l do not
+// depend on which maximum was in use.
+constexpr float kLazyLog2 = 8.0f;
 
 template <typename T, int DP, int MINB>
 __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
@@ -206,36 +232,51 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   const int D = a.head_dim;
   const int row = m0 + 32 * wave + c32;  // this lane's query row (lanes l and l^32 share it)
 
-  // ---- DMA bookkeeping: lane -> (row in instruction block, logical chunk) --------------------------------
-  const int dma_r = wave * RPI + lane / CPR;  // row within tile for instruction 0; instruction i adds 4*RPI*i
-  const int dma_pc = lane % CPR;
-  // head_dim < DP: pad chunks are pointed at chunk 0 (valid memory); they meet zeros of Q / are never stored.
-  // The swizzles only use row bits that the per-instruction row step (4 RPI) leaves alone, except swzK at
+  // ---- DMA bookkeeping ---------------------------------------------------------------------------------
+  // DMA instruction i of this wavefront fills LDS rows dma_r + 4 RPI i (one 1 KiB block).  The global address is
+  // a wavefront-uniform base (tile start + 4 RPI i rows, scalar registers) plus a per-lane byte offset that does
+  // not change from tile to tile, so a full tile costs no vector ALU work; only the last, partial tile clamps
+  // rows per lane.  head_dim < DP: pad chunks are pointed at chunk 0 (valid memory); they meet zeros of Q / are
+  // never stored.  The swizzles only use row bits that the per-instruction row step leaves alone, except swzK at
   // DP == 256 where odd instructions toggle bit 3.
+  const int dma_r = wave * RPI + lane / CPR;
+  const int dma_pc = lane % CPR;
   int lck = dma_pc ^ swzK<DP>(dma_r);
   int lck_odd = (DP == 256) ? (lck ^ 8) : lck;
   int lcv = dma_pc ^ swzV<DP>(dma_r);
   if (lck * 8 >= D) lck = 0;
   if (lck_odd * 8 >= D) lck_odd = 0;
   if (lcv * 8 >= D) lcv = 0;
-  const unsigned char* kp_lane = kp + lck * 16;
-  const unsigned char* kp_lane_odd = kp + lck_odd * 16;
-  const unsigned char* vp_lane = vp + lcv * 16;
   const unsigned k_ss = (unsigned)a.k_ss, v_ss = (unsigned)a.v_ss;
+  const unsigned koff = (unsigned)dma_r * k_ss + lck * 16;
+  const unsigned koff_odd = (unsigned)dma_r * k_ss + lck_odd * 16;
+  const unsigned voff = (unsigned)dma_r * v_ss + lcv * 16;
   const int last_k = Lk - 1;
+  const unsigned lds0 = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + wave * 1024;
 
+  // One DMA instruction of a tile that lies fully inside the sequence: `which` = 0 (K) or 1 (V), block i of tile j
+  // into buffer buf.  Only scalar address arithmetic.  These are issued one at a time between MFMAs so that a
+  // wavefront never sits in the (narrow, CU-shared) vector-memory issue queue with nothing else to do.
+  auto issue_one = [&](int j, int buf, int which, int i) {
+    const unsigned dst = lds0 + (which ? 2 * TILE : 0) + buf * TILE + i * 4096;
+    const unsigned ss = which ? v_ss : k_ss;
+    const unsigned char* base = (which ? vp : kp) + (uint64_t)(unsigned)(j * BN + i * 4 * RPI) * ss;
+    dma16s(base, which ? voff : ((DP == 256 && (i & 1)) ? koff_odd : koff), dst);
+  };
+  // A whole tile at once, rows clamped to the last valid one (first tile, and the partial tile at the end of K).
   auto issue_tile = [&](int j, int buf) {
-    unsigned char* kdst = smem + buf * TILE + wave * 1024;
-    unsigned char* vdst = smem + 2 * TILE + buf * TILE + wave * 1024;
+    const int rmax = last_k - j * BN;  // >= 0: the tile exists
+    const unsigned char* kt = kp + (uint64_t)(unsigned)(j * BN) * k_ss;
+    const unsigned char* vt = vp + (uint64_t)(unsigned)(j * BN) * v_ss;
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const int r = min(j * BN + dma_r + i * 4 * RPI, last_k);
-      dma16(((DP == 256 && (i & 1)) ? kp_lane_odd : kp_lane) + (uint64_t)(unsigned)r * k_ss, kdst + i * 4096);
+      const unsigned r = (unsigned)min(dma_r + i * 4 * RPI, rmax);
+      dma16s(kt, r * k_ss + ((DP == 256 && (i & 1)) ? lck_odd : lck) * 16, lds0 + buf * TILE + i * 4096);
     }
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const int r = min(j * BN + dma_r + i * 4 * RPI, last_k);
-      dma16(vp_lane + (uint64_t)(unsigned)r * v_ss, vdst + i * 4096);
+      const unsigned r = (unsigned)min(dma_r + i * 4 * RPI, rmax);
+      dma16s(vt, r * v_ss + lcv * 16, lds0 + 2 * TILE + buf * TILE + i * 4096);
     }
   };
 
@@ -264,46 +305,67 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
   const float c = a.scale_log2;
+  const float lazy = kLazyLog2 / c;  // threshold in raw-score units
 
-  // per-lane LDS read offsets
-  const int ksw = swzK<DP>(c32);  // same for rows c32 and 32 + c32
+  // ---- per-lane LDS read offsets (bytes from the start of a K / V tile), fixed for the whole kernel ----------
+  // K fragment for k-step ks: rows c32 and 32 + c32 (same swizzle), logical chunk 2 ks + g
+  int kaddr[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) kaddr[ks] = c32 * ROWB + (((2 * ks + g) ^ swzK<DP>(c32)) * 16);
+  // V^T fragment for (mb, t, half): row 16 t + 8 half + 4 g + (L >> 2), logical chunk 4 mb + 2 (G & 1) + ((L & 3) >> 1)
   const int L = lane & 15, G = lane >> 4;
-  // V^T fragment for (mblk, t, half): row 16 t + 8 half + 4 g + (L >> 2), logical chunk 4 mblk + 2 (G & 1) + ((L & 3) >> 1)
   const int v_row = 4 * g + (L >> 2);
-  const int v_lc0 = 2 * (G & 1) + ((L & 3) >> 1);
-  const int v_sw = swzV<DP>(v_row);  // rows differ by multiples of 8 across (t, half): same swizzle
-  const int v_lane_off = v_row * ROWB + (L & 1) * 8;
+  int vaddr[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+    vaddr[mb] = v_row * ROWB + (L & 1) * 8 + (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzV<DP>(v_row)) * 16);
 
   const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
+  const int wave_row_lo = m0 + 32 * wave, wave_row_hi = wave_row_lo + 31;
 
-  for (int j = 0; j < ntiles; ++j) {
-    const int buf = j & 1;
+  auto tile = [&](int j, auto bufc) {
+    constexpr int BUF = decltype(bufc)::value;
     WAIT_VMCNT(0);       // my DMA for tile j has landed
     __syncthreads();     // everyone's has; everyone is done reading the other buffer
-    if (j + 1 < ntiles) issue_tile(j + 1, buf ^ 1);
+    // next tile: fully inside K -> its DMA instructions are interleaved with this tile's MFMAs; partial -> issued here
+    const bool more = j + 1 < ntiles;
+    const bool spread = more && (j + 2) * BN <= Lk && !(a.is_causal && j * BN > wave_row_hi + off);
+    if (more && !spread) issue_tile(j + 1, BUF ^ 1);
 
     // wavefront-uniform skip: every score of this tile is masked for all 32 rows of this wavefront
-    const int wave_row_hi = m0 + 32 * wave + 31;
-    if (a.is_causal && j * BN > wave_row_hi + off) continue;
+    if (a.is_causal && j * BN > wave_row_hi + off) return;
 
-    const unsigned char* kt = smem + buf * TILE;
-    const unsigned char* vt = smem + 2 * TILE + buf * TILE;
+    const unsigned char* kt = smem + BUF * TILE;
+    const unsigned char* vt = smem + 2 * TILE + BUF * TILE;
 
-    // ---- S^T = K Q^T : two 32(kv) x 32(q) blocks ----
+    // ---- S^T = K Q^T : two 32(kv) x 32(q) blocks; K fragments are fetched two k-steps ahead of their MFMAs ----
     f32x16 s0, s1;
 #pragma unroll
     for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; }
+    {
+      s16x8 ka[2][2];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int pc = (2 * ks + g) ^ ksw;
-      const s16x8 a0 = *(const s16x8*)(kt + c32 * ROWB + pc * 16);
-      const s16x8 a1 = *(const s16x8*)(kt + (32 + c32) * ROWB + pc * 16);
-      s0 = Mma<T>::m32(a0, qf[ks], s0);
-      s1 = Mma<T>::m32(a1, qf[ks], s1);
+      for (int ks = 0; ks < 2; ++ks) {
+        ka[ks][0] = *(const s16x8*)(kt + kaddr[ks]);
+        ka[ks][1] = *(const s16x8*)(kt + kaddr[ks] + 32 * ROWB);
+      }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        s0 = Mma<T>::m32(ka[ks & 1][0], qf[ks], s0);
+        s1 = Mma<T>::m32(ka[ks & 1][1], qf[ks], s1);
+        // next tile's K and V: 2 NI DMA instructions spread over the KS k-steps (K block i, then V block i)
+        if (spread) {
+#pragma unroll
+          for (int x = (ks * 2 * NI) / KS; x < ((ks + 1) * 2 * NI) / KS; ++x) issue_one(j + 1, BUF ^ 1, x & 1, x >> 1);
+        }
+        if (ks + 2 < KS) {
+          ka[ks & 1][0] = *(const s16x8*)(kt + kaddr[ks + 2]);
+          ka[ks & 1][1] = *(const s16x8*)(kt + kaddr[ks + 2] + 32 * ROWB);
+        }
+      }
     }
 
     // ---- mask (tail of K, causal diagonal) ----
-    const int wave_row_lo = m0 + 32 * wave;
     const bool need_mask = (j * BN + BN > Lk) || (a.is_causal && j * BN + BN - 1 > wave_row_lo + off);
     if (need_mask) {
       const int lim = min(last_k, causal_row_lim) - j * BN - 4 * g;  // element index e is visible iff e <= lim
@@ -316,54 +378,67 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     }
 
     // ---- online softmax (one lane = one query row x 32 of the 64 columns) ----
-    float mx = fmaxf(s0[0], s1[0]);
+    float mx = max3(s0[0], s0[1], s0[2]);
 #pragma unroll
-    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(s0[v], s1[v]));
+    for (int v = 3; v < 15; v += 2) mx = max3(mx, s0[v], s0[v + 1]);
+    mx = max3(mx, s0[15], s1[0]);
+#pragma unroll
+    for (int v = 1; v < 15; v += 2) mx = max3(mx, s1[v], s1[v + 1]);
+    mx = fmaxf(mx, s1[15]);
     mx = pair_max32(mx);
-    const float m_new = fmaxf(m_run, mx);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = fast_exp2((m_run - m_use) * c);
-    const float mc = m_use * c;
-    m_run = m_new;
+    const bool grow = mx > m_run + lazy;  // first visible tile: m_run = -inf
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float m_new = grow ? mx : m_run;
+      const float alpha = grow ? fast_exp2((m_run - m_new) * c) : 1.0f;  // exp2(-inf) = 0 on the first tile
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
+    }
+    const float mc = (m_run == -INFINITY) ? 0.f : m_run * c;
+
+    // ---- per 16-key chunk t: P = exp2(S c - m c), row sums, P^T as B operand, O^T += V^T P^T.  The V^T fragments
+    //      of chunk t + 1 are fetched while chunk t's MFMAs run. ----
+    auto vfrag = [&](int mb, int t) {
+      const s16x4 lo = lds_read_tr(vt + vaddr[mb] + (16 * t) * ROWB);
+      const s16x4 hi = lds_read_tr(vt + vaddr[mb] + (16 * t + 8) * ROWB);
+      return s16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    s16x8 va[2][MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) va[0][mb] = vfrag(mb, 0);
     float rs = 0.f;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      s0[v] = fast_exp2(s0[v] * c - mc);
-      s1[v] = fast_exp2(s1[v] * c - mc);
-      rs += s0[v] + s1[v];
-    }
-    l_run = l_run * alpha + rs;
-#pragma unroll
-    for (int i = 0; i < MB; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
-
-    // ---- P^T as B operands: k-step t covers kv 16 t .. 16 t + 15 of the tile ----
-    s16x8 pb[4];
-#pragma unroll
     for (int t = 0; t < 4; ++t) {
+      if (t + 1 < 4) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) va[(t + 1) & 1][mb] = vfrag(mb, t + 1);
+      }
       u32x4 w;
 #pragma unroll
       for (int e2 = 0; e2 < 4; ++e2) {
         const int v = 8 * (t & 1) + 2 * e2;
-        w[e2] = (t < 2) ? Mma<T>::pack2(s0[v], s0[v + 1]) : Mma<T>::pack2(s1[v], s1[v + 1]);
+        const float x0 = (t < 2) ? s0[v] : s1[v], x1 = (t < 2) ? s0[v + 1] : s1[v + 1];
+        const float p0 = fast_exp2(x0 * c - mc), p1 = fast_exp2(x1 * c - mc);
+        rs += p0 + p1;
+        w[e2] = Mma<T>::pack2(p0, p1);
       }
-      pb[t] = __builtin_bit_cast(s16x8, w);
+      const s16x8 pb = __builtin_bit_cast(s16x8, w);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) o[mb] = Mma<T>::m32(va[t & 1][mb], pb, o[mb]);
     }
+    l_run += rs;
+  };
 
-    // ---- O^T += V^T P^T ----
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      const int pc = (4 * mb + v_lc0) ^ v_sw;
-      const unsigned char* vbase = vt + v_lane_off + pc * 16;
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const s16x4 lo = lds_read_tr(vbase + (16 * t) * ROWB);
-        const s16x4 hi = lds_read_tr(vbase + (16 * t + 8) * ROWB);
-        const s16x8 av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        o[mb] = Mma<T>::m32(av, pb[t], o[mb]);
-      }
+  {
+    int j = 0;
+    for (; j + 1 < ntiles; j += 2) {
+      tile(j, IC<0>{});
+      tile(j + 1, IC<1>{});
     }
+    if (j < ntiles) tile(j, IC<0>{});
   }
 
   // ---- epilogue ----
