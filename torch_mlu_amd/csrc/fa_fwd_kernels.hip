@@ -62,7 +62,8 @@ struct KArgs {
   int64_t lse_sb, lse_sh, lse_ss;  // element strides
   int32_t batch, heads_q, heads_k, group;
   int32_t seqlen_q, seqlen_k, head_dim;
-  int32_t n_mblk;     // tile kernel: query blocks per sequence
+  int32_t n_mblk;     // tile kernels: workgroups per (sequence, head)
+  int32_t pair;       // tile kernel: a workgroup owns query blocks p and n-1-p of its sequence
   int32_t n_splits;   // split-KV kernel
   int32_t is_causal;
   int32_t neg_scale;  // scale < 0: Q is negated on load and |scale| is used, so that max() tracks the true row max
@@ -202,7 +203,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     const int total = gridDim.x, per = total >> 3;
     if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
   }
-  const int mi = a.n_mblk - 1 - (lid % a.n_mblk);
+  const int pslot = lid % a.n_mblk;  // a.n_mblk: workgroups per (sequence, head)
   const int bh = lid / a.n_mblk;
   const int h = bh % a.heads_q, b = bh / a.heads_q;
   const int hk = h / a.group;
@@ -218,19 +219,18 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     qb = kb = vb = ob = 0;
     lb = 0;
   }
-  const int m0 = mi * BM;
-  if (m0 >= Lq) return;
+  // query blocks owned by this workgroup: paired (causal) -> the heavy block nblk-1-p and the light block p, so that
+  // every workgroup of a sequence has the same number of tiles; unpaired -> block nblk-1-p (heavy blocks first)
+  const int nblk = (Lq + BM - 1) / BM;
+  if (a.pair ? (2 * pslot >= nblk) : (pslot >= nblk)) return;
+  const int blk_first = nblk - 1 - pslot;
+  const int n_own = (DP != 256 && a.pair && blk_first != pslot) ? 2 : 1;  // head_dim 256 never pairs (registers)
   const int off = Lk - Lq;  // causal: col visible iff col <= row + off
-  int n_end = Lk;
-  if (a.is_causal) n_end = min(Lk, m0 + BM + off);
-  if (n_end < 0) n_end = 0;
-  const int ntiles = (n_end + BN - 1) / BN;
 
   const unsigned char* qp = a.q + qb + (int64_t)q0 * a.q_ss + (int64_t)h * a.q_sh;
   const unsigned char* kp = a.k + kb + (int64_t)k0 * a.k_ss + (int64_t)hk * a.k_sh;
   const unsigned char* vp = a.v + vb + (int64_t)k0 * a.v_ss + (int64_t)hk * a.v_sh;
   const int D = a.head_dim;
-  const int row = m0 + 32 * wave + c32;  // this lane's query row (lanes l and l^32 share it)
 
   // ---- DMA bookkeeping ---------------------------------------------------------------------------------
   // DMA instruction i of this wavefront fills LDS rows dma_r + 4 RPI i (one 1 KiB block).  The global address is
@@ -280,6 +280,29 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     }
   };
 
+  // ---- per-lane LDS read offsets (bytes from the start of a K / V tile), fixed for the whole kernel ----------
+  // K fragment for k-step ks: rows c32 and 32 + c32 (same swizzle), logical chunk 2 ks + g
+  int kaddr[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) kaddr[ks] = c32 * ROWB + (((2 * ks + g) ^ swzK<DP>(c32)) * 16);
+  // V^T fragment for (mb, t, half): row 16 t + 8 half + 4 g + (L >> 2), logical chunk 4 mb + 2 (G & 1) + ((L & 3) >> 1)
+  const int L = lane & 15, G = lane >> 4;
+  const int v_row = 4 * g + (L >> 2);
+  int vaddr[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+    vaddr[mb] = v_row * ROWB + (L & 1) * 8 + (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzV<DP>(v_row)) * 16);
+  const float c = a.scale_log2;
+  const float lazy = kLazyLog2 / c;  // threshold in raw-score units
+
+  for (int own = 0; own < n_own; ++own) {
+  const int m0 = (own == 0 ? blk_first : pslot) * BM;
+  int n_end = Lk;
+  if (a.is_causal) n_end = min(Lk, m0 + BM + off);
+  if (n_end < 0) n_end = 0;
+  const int ntiles = (n_end + BN - 1) / BN;
+  const int row = m0 + 32 * wave + c32;  // this lane's query row (lanes l and l^32 share it)
+  if (own) __syncthreads();  // the previous block's last LDS reads are done
   if (ntiles > 0) issue_tile(0, 0);
 
   // ---- Q fragments (B operand): lane (c32, g) holds Q[row][16 ks + 8 g .. +8] -----------------------------
@@ -304,21 +327,6 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
-  const float c = a.scale_log2;
-  const float lazy = kLazyLog2 / c;  // threshold in raw-score units
-
-  // ---- per-lane LDS read offsets (bytes from the start of a K / V tile), fixed for the whole kernel ----------
-  // K fragment for k-step ks: rows c32 and 32 + c32 (same swizzle), logical chunk 2 ks + g
-  int kaddr[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) kaddr[ks] = c32 * ROWB + (((2 * ks + g) ^ swzK<DP>(c32)) * 16);
-  // V^T fragment for (mb, t, half): row 16 t + 8 half + 4 g + (L >> 2), logical chunk 4 mb + 2 (G & 1) + ((L & 3) >> 1)
-  const int L = lane & 15, G = lane >> 4;
-  const int v_row = 4 * g + (L >> 2);
-  int vaddr[MB];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
-    vaddr[mb] = v_row * ROWB + (L & 1) * 8 + (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzV<DP>(v_row)) * 16);
 
   const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
   const int wave_row_lo = m0 + 32 * wave, wave_row_hi = wave_row_lo + 31;
@@ -463,6 +471,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
       a.lse[lb + (int64_t)h * a.lse_sh + (int64_t)(q0 + row) * a.lse_ss] = lse;
     }
   }
+  }  // own
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -852,6 +861,7 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   a.batch = p->batch; a.heads_q = p->heads_q; a.heads_k = p->heads_k; a.group = p->heads_q / p->heads_k;
   a.seqlen_q = p->seqlen_q; a.seqlen_k = p->seqlen_k; a.head_dim = p->head_dim;
   a.n_mblk = (p->seqlen_q + 127) / 128;
+  a.pair = 0;
   a.n_splits = ns;
   a.is_causal = p->is_causal ? 1 : 0;
   a.neg_scale = p->scale < 0.f ? 1 : 0;
@@ -870,13 +880,16 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
 }
 
 template <typename T, int DP, int MINB>
-int launch_tile(const KArgs& a, hipStream_t st) {
+int launch_tile(KArgs a, hipStream_t st) {
   constexpr int lds = 4 * 64 * DP * 2;
   auto kfn = fa_tile_kernel<T, DP, MINB>;
   if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
     (void)hipGetLastError();
     return FA_ERR_LAUNCH;
   }
+  const int nblk = (a.seqlen_q + 127) / 128;
+  a.pair = (DP != 256 && a.is_causal && nblk >= 2 && (int64_t)a.batch * a.heads_q * ((nblk + 1) / 2) >= 1024) ? 1 : 0;
+  a.n_mblk = a.pair ? (nblk + 1) / 2 : nblk;
   const int64_t grid = (int64_t)a.batch * a.heads_q * a.n_mblk;
   if (grid <= 0) return FA_OK;
   if (grid > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
