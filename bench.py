@@ -25,6 +25,14 @@ import torch
 
 PEAK_MFMA_TFLOPS = 2500.0  # dense bf16 / fp16
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same file,
+# each scaled by what the same counter reads for the 1 GiB copy of --config copy1g (2.000 and 1.000); the runs and
+# their commands are recorded under profiles/.  Counters cannot be read from inside a timed run, so these are the
+# recorded values (None: not profiled).
+TRAFFIC_BYTES = {
+    "cfg2": int((521.7 + 130.0) * 2 ** 20),
+    "cfg5": int(2.0022 * 2 ** 30 + 4.25 * 2 ** 20),
+}
 
 
 def seeded(shape, seed, dtype, std=0.5):
@@ -100,6 +108,18 @@ def make_workload(name, dev):
         return dict(call=call, check=check, flops=4 * B * Hq * Sk * D, bytes_kv=2 * B * Hk * Sk * D * 2,
                     desc=f"decode bf16 GQA B={B} Hq={Hq} Hkv={Hk} Sq=1 Skv={Sk} D={D}", dtype="bf16", bound="hbm",
                     kernel="fa_splitkv_kernel")
+    if name == "copy1g":
+        # calibration workload for the HBM traffic counters: a plain 1 GiB device-to-device copy
+        src = torch.zeros(512 * 1024 * 1024, dtype=bf, device=dev)
+        dst = torch.empty_like(src)
+
+        def call():
+            dst.copy_(src)
+            return dst
+
+        return dict(call=call, check=lambda: (0.0, 0.0), flops=0.0, bytes_kv=2.0 * src.numel() * 2,
+                    desc="1 GiB device-to-device copy (counter calibration; bytes = read + written)", dtype="bf16",
+                    bound="hbm", kernel="copy")
     raise SystemExit(f"unknown config {name}")
 
 
@@ -173,7 +193,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "copy1g"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -196,18 +216,18 @@ def main():
         n0 = torch_mlu_amd.launch_count()
         eo, el = w["check"]()
         wall, ev_mean, ev_med, ev_min = time_steps(w["call"], steps, warmup)
-        assert torch_mlu_amd.launch_count() >= n0 + steps + warmup, "the registered HIP path did not run"
+        assert name == "copy1g" or torch_mlu_amd.launch_count() >= n0 + steps + warmup, "the registered HIP path did not run"
         r = {"config": name, "workload": w["desc"], "ms_per_step": wall, "kernel_ms_mean": ev_mean,
              "kernel_ms_median": ev_med, "kernel_ms_min": ev_min, "tflops": w["flops"] / wall / 1e9,
              "kv_gbs": w["bytes_kv"] / wall / 1e6, "max_abs_err_out": eo, "max_abs_err_lse": el, "dtype": w["dtype"]}
         if w["bound"] == "mfma":
             ach = w["flops"] / ev_mean / 1e9
             r["roofline"] = {"bound": "mfma", "kernel": w["kernel"], "achieved": ach, "peak": PEAK_MFMA_TFLOPS,
-                             "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_TFLOPS, "traffic": None}
+                             "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_TFLOPS, "traffic": TRAFFIC_BYTES.get(name)}
         else:
             ach = w["bytes_kv"] / ev_mean / 1e6
             r["roofline"] = {"bound": "hbm", "kernel": w["kernel"], "achieved": ach, "peak": PEAK_HBM_GBS,
-                             "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": None}
+                             "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "traffic": TRAFFIC_BYTES.get(name)}
         del w
         torch.cuda.empty_cache()
         return r
@@ -219,7 +239,7 @@ def main():
             if name != args.config:
                 extras.append(run(name, args.steps, args.warmup))
 
-    is_decode = args.config == "cfg5"
+    is_decode = args.config in ("cfg5", "copy1g")
     line = {
         "metric": "fwd attn TFLOP/s + % MFMA peak (bf16 S=4096 D=128); decode HBM GB/s",
         "value": main_r["kv_gbs"] if is_decode else main_r["tflops"],
