@@ -142,9 +142,16 @@ def _check_heads(q, k, v, out, lse, causal, heads):
     return eo, el
 
 
-def time_steps(call, steps, warmup):
+def time_steps(call, steps, warmup, spin_up_s=0.4):
     """Exactly `steps` timed calls between two device synchronisations; HIP events on the launch stream give the
-    per-step device time."""
+    per-step device time.  Before the `warmup` untimed steps the same call is repeated for `spin_up_s` seconds (also
+    untimed): an idle MI355X sits at a low engine clock and needs a few hundred milliseconds of load to ramp up, which
+    would otherwise be charged to the first timed steps."""
+    t_end = time.perf_counter() + spin_up_s
+    while time.perf_counter() < t_end:
+        for _ in range(10):
+            call()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         call()
     torch.cuda.synchronize()
