@@ -1,0 +1,111 @@
+// Device-side helpers shared by the forward and backward kernels (gfx950 only).
+#ifndef FA_DEVICE_H_
+#define FA_DEVICE_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fa {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+#define LDS_AS __attribute__((address_space(3)))
+#define GLB_AS __attribute__((address_space(1)))
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<__bf16> {
+  static __device__ __forceinline__ f32x16 m32(s16x8 a, s16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16(s16x8 a, s16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ unsigned pack2(float a, float b) {
+    f32x2 f = {a, b};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
+  }
+};
+template <>
+struct Mma<_Float16> {
+  static __device__ __forceinline__ f32x16 m32(s16x8 a, s16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16(s16x8 a, s16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ unsigned pack2(float a, float b) {
+    f32x2 f = {a, b};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f, f16x2));
+  }
+};
+
+// 16-byte global -> LDS DMA.  Lane i of the wavefront writes LDS bytes [lds_wave_base + 16 i, +16); the global
+// address is per lane.  lds_wave_base must be wavefront-uniform.  Written as inline assembly on purpose: the
+// compiler then does not know these loads write LDS, so it does not put a conservative "wait for every
+// outstanding load" in front of the LDS reads of the tile being computed.  Completion is tracked by hand
+// with WAIT_VMCNT (the loads retire in order).
+__device__ __forceinline__ void dma16(const unsigned char* gptr, unsigned char* lds_wave_base) {
+  const unsigned lds = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(LDS_AS unsigned char*)lds_wave_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds), "v"(gptr) : "memory", "m0");
+}
+
+// Same, with the global address split into a wavefront-uniform 64-bit base (scalar registers) and a per-lane
+// 32-bit byte offset, and the LDS destination given as a wavefront-uniform LDS byte address.
+__device__ __forceinline__ void dma16s(const unsigned char* sbase, unsigned voff, unsigned lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_wave_base), "v"(voff), "s"(sbase)
+               : "m0");
+}
+
+// Transposed LDS read: within each group of 16 lanes, lane j receives element (j % 4) of the four 8-byte pieces
+// addressed by lanes 4 i + j / 4 (i = 0..3) of the same group.
+__device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 LDS_AS*)p);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// max over the lane pair (l, l ^ 32)
+__device__ __forceinline__ float pair_max32(float x) {
+  unsigned u = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+}
+__device__ __forceinline__ float pair_sum32(float x) {
+  unsigned u = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+}
+
+#define WAIT_VMCNT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
+
+template <int N>
+struct IC {
+  static constexpr int value = N;
+};
+
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+}  // namespace fa
+
+#endif  // FA_DEVICE_H_

@@ -24,27 +24,12 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fa_device.h"
 #include "fa_fwd.h"
 
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-
-#define LDS_AS __attribute__((address_space(3)))
-#define GLB_AS __attribute__((address_space(1)))
-
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
+using namespace fa;
 
 // Kernel arguments: fa_fwd_params plus what the host derives once.
 struct KArgs {
@@ -72,76 +57,6 @@ struct KArgs {
   float* ws_ml;       // [batch*heads_q*n_splits][2]: m (log2 domain), l
 };
 
-template <typename T>
-struct Mma;
-template <>
-struct Mma<__bf16> {
-  static __device__ __forceinline__ f32x16 m32(s16x8 a, s16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ f32x4 m16(s16x8 a, s16x8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ unsigned pack2(float a, float b) {
-    f32x2 f = {a, b};
-    return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
-  }
-};
-template <>
-struct Mma<_Float16> {
-  static __device__ __forceinline__ f32x16 m32(s16x8 a, s16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ f32x4 m16(s16x8 a, s16x8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ unsigned pack2(float a, float b) {
-    f32x2 f = {a, b};
-    return __builtin_bit_cast(unsigned, __builtin_convertvector(f, f16x2));
-  }
-};
-
-// 16-byte global -> LDS DMA.  Lane i of the wavefront writes LDS bytes [lds_wave_base + 16 i, +16); the global
-// address is per lane.  lds_wave_base must be wavefront-uniform.  Written as inline assembly on purpose: the
-// compiler then does not know these loads write LDS, so it does not put a conservative "wait for every
-// outstanding load" in front of the LDS reads of the tile being computed.  Completion is tracked by hand
-// with WAIT_VMCNT (the loads retire in order).
-__device__ __forceinline__ void dma16(const unsigned char* gptr, unsigned char* lds_wave_base) {
-  const unsigned lds = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(LDS_AS unsigned char*)lds_wave_base);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds), "v"(gptr) : "memory", "m0");
-}
-
-// Same, with the global address split into a wavefront-uniform 64-bit base (scalar registers) and a per-lane
-// 32-bit byte offset, and the LDS destination given as a wavefront-uniform LDS byte address.
-__device__ __forceinline__ void dma16s(const unsigned char* sbase, unsigned voff, unsigned lds_wave_base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :
-               : "s"(lds_wave_base), "v"(voff), "s"(sbase)
-               : "m0");
-}
-
-// Transposed LDS read: within each group of 16 lanes, lane j receives element (j % 4) of the four 8-byte pieces
-// addressed by lanes 4 i + j / 4 (i = 0..3) of the same group.
-__device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
-  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 LDS_AS*)p);
-}
-
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-// max over the lane pair (l, l ^ 32)
-__device__ __forceinline__ float pair_max32(float x) {
-  unsigned u = __builtin_bit_cast(unsigned, x);
-  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
-}
-__device__ __forceinline__ float pair_sum32(float x) {
-  unsigned u = __builtin_bit_cast(unsigned, x);
-  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
-}
-
-#define WAIT_VMCNT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
-
 // ---------------------------------------------------------------------------------------------------------
 // Tile kernel
 // ---------------------------------------------------------------------------------------------------------
@@ -159,17 +74,6 @@ template <int DP>
 __device__ __forceinline__ int swzV(int row) {
   if constexpr (DP == 64) return ((row >> 1) & 1) << 2;
   return (row & 3) << 2;
-}
-
-template <int N>
-struct IC {
-  static constexpr int value = N;
-};
-
-__device__ __forceinline__ float max3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
 }
 
 // A new row maximum only forces a rescale of the accumulators when it exceeds the one in use by more than this
@@ -198,13 +102,22 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   // ---- which (sequence, head, query block): XCD-aware, heavy blocks first -------------------------------
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical ids so that
   // all query blocks of one (sequence, kv head) share that XCD's L2.
+  // Dense: workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical ids so that
+  // all query blocks of one (sequence, kv head) share that XCD's L2.  Packed (ragged lengths, known only on the
+  // device): block-major order instead, i.e. the last (heaviest) blocks of all sequences first and sequences
+  // shorter than that exit at once — longest-processing-time-first without knowing the lengths on the host.
   int lid = blockIdx.x;
-  {
+  int pslot, bh;
+  if (a.cu_q) {
+    const int nbh = a.batch * a.heads_q;
+    pslot = lid / nbh;
+    bh = lid % nbh;
+  } else {
     const int total = gridDim.x, per = total >> 3;
     if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
+    pslot = lid % a.n_mblk;  // a.n_mblk: workgroups per (sequence, head)
+    bh = lid / a.n_mblk;
   }
-  const int pslot = lid % a.n_mblk;  // a.n_mblk: workgroups per (sequence, head)
-  const int bh = lid / a.n_mblk;
   const int h = bh % a.heads_q, b = bh / a.heads_q;
   const int hk = h / a.group;
 
@@ -219,11 +132,12 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     qb = kb = vb = ob = 0;
     lb = 0;
   }
-  // query blocks owned by this workgroup: paired (causal) -> the heavy block nblk-1-p and the light block p, so that
-  // every workgroup of a sequence has the same number of tiles; unpaired -> block nblk-1-p (heavy blocks first)
+  // query blocks owned by this workgroup: paired (causal, dense) -> the heavy block nblk-1-p and the light block p,
+  // so that every workgroup of a sequence has the same number of tiles; unpaired -> one block, heavy blocks first
+  // (packed: counted down from the longest possible sequence so that equal slots mean equal block indices)
   const int nblk = (Lq + BM - 1) / BM;
-  if (a.pair ? (2 * pslot >= nblk) : (pslot >= nblk)) return;
-  const int blk_first = nblk - 1 - pslot;
+  const int blk_first = (a.cu_q ? a.n_mblk : nblk) - 1 - pslot;
+  if (a.pair ? (2 * pslot >= nblk) : (blk_first < 0 || blk_first >= nblk)) return;
   const int n_own = (DP != 256 && a.pair && blk_first != pslot) ? 2 : 1;  // head_dim 256 never pairs (registers)
   const int off = Lk - Lq;  // causal: col visible iff col <= row + off
 
@@ -888,7 +802,7 @@ int launch_tile(KArgs a, hipStream_t st) {
     return FA_ERR_LAUNCH;
   }
   const int nblk = (a.seqlen_q + 127) / 128;
-  a.pair = (DP != 256 && a.is_causal && nblk >= 2 && (int64_t)a.batch * a.heads_q * ((nblk + 1) / 2) >= 1024) ? 1 : 0;
+  a.pair = (DP != 256 && !a.cu_q && a.is_causal && nblk >= 2 && (int64_t)a.batch * a.heads_q * ((nblk + 1) / 2) >= 1024) ? 1 : 0;
   a.n_mblk = a.pair ? (nblk + 1) / 2 : nblk;
   const int64_t grid = (int64_t)a.batch * a.heads_q * a.n_mblk;
   if (grid <= 0) return FA_OK;
