@@ -1,0 +1,87 @@
+/*
+ * fa_bwd.h — C ABI of the MI355X (gfx950) flash-attention backward launcher (same library as fa_fwd.h).
+ *
+ * Replaces the vendor calls torch_mlu's backward launcher `mha_varlen_bwd` makes
+ * (torch_mlu/csrc/aten/operators/cnnl/internal/FlashAttention_internal.cpp:269-483):
+ *
+ *   cnnlSetFlashAttentionBackwardDescriptor + tensor descriptors (:368-447)  -> fa_bwd_params
+ *   cnnlGetFlashAttentionBackwardWorkspaceSize (:430-447)                    -> fa_bwd_workspace_bytes
+ *   cnnlFlashAttentionBackward (:449-480)                                    -> fa_bwd_launch
+ *
+ * Given the forward's inputs, its output and its logsumexp, and the gradient of the output, computes
+ *     P   = exp(scale * Q K^T + mask - LSE)                (recomputed, never stored)
+ *     dV  = P^T dO
+ *     dP  = dO V^T,   delta = rowsum(dO o O),   dS = P o (dP - delta)
+ *     dQ  = scale * dS K,   dK = scale * dS^T Q
+ * with the forward's masking (bottom-right aligned causal) and head grouping (dK, dV of a kv head sum over the
+ * query heads that read it).  Same rules as fa_fwd.h: plain C, device pointers, element strides, no allocation,
+ * no synchronisation, work is only enqueued on the caller's stream.
+ */
+#ifndef FA_BWD_H_
+#define FA_BWD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "fa_fwd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Addressing as in fa_fwd_params: row (b,s,h) of X at X + b*x_stride_b + s*x_stride_s + h*x_stride_h (elements),
+ * head_dim elements contiguous; packed mode (cu_seqlens_q != NULL) ignores *_stride_b and addresses rows by their
+ * packed index.  q, dq, out, dout have heads_q heads; k, v, dk, dv have heads_k heads.  lse is the forward's
+ * logsumexp (natural log), read through the same three strides the forward wrote it with.
+ */
+typedef struct fa_bwd_params {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* out;
+  const void* dout;
+  const float* lse;
+  void* dq;
+  void* dk;
+  void* dv;
+  const int32_t* cu_seqlens_q; /* device int32[batch+1] or NULL */
+  const int32_t* cu_seqlens_k;
+
+  int64_t q_stride_b, q_stride_s, q_stride_h;
+  int64_t k_stride_b, k_stride_s, k_stride_h;
+  int64_t v_stride_b, v_stride_s, v_stride_h;
+  int64_t o_stride_b, o_stride_s, o_stride_h;
+  int64_t do_stride_b, do_stride_s, do_stride_h;
+  int64_t dq_stride_b, dq_stride_s, dq_stride_h;
+  int64_t dk_stride_b, dk_stride_s, dk_stride_h;
+  int64_t dv_stride_b, dv_stride_s, dv_stride_h;
+  int64_t lse_stride_b, lse_stride_h, lse_stride_s;
+
+  int32_t batch;
+  int32_t heads_q;
+  int32_t heads_k;
+  int32_t seqlen_q;  /* dense: rows per sequence; packed: max over sequences */
+  int32_t seqlen_k;
+  int32_t head_dim;  /* multiple of 8, 8..128 */
+  int64_t total_q;   /* packed: rows of q (sizes the delta scratch); dense: ignored */
+
+  float scale;
+  int32_t dtype;     /* FA_DTYPE_* */
+  int32_t is_causal;
+  int32_t reserved;  /* must be 0 */
+} fa_bwd_params;
+
+/* Host-only validation: FA_OK or a negative code (FA_ERR_UNSUPPORTED for head_dim > 128). */
+int fa_bwd_validate(const fa_bwd_params* p);
+
+/* Bytes of device scratch fa_bwd_launch needs (delta = rowsum(dO o O), fp32 per query row and head); 0 if invalid. */
+size_t fa_bwd_workspace_bytes(const fa_bwd_params* p);
+
+/* Enqueue the backward pass on `stream`; `workspace` must hold fa_bwd_workspace_bytes(p) bytes, 16-byte aligned. */
+int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FA_BWD_H_ */

@@ -10,6 +10,8 @@ from .attention_oracle import (  # noqa: F401
     default_atol,
     default_rtol,
     get_tolerances,
+    sdpa_backward_oracle,
     sdpa_oracle,
+    varlen_backward_oracle,
     varlen_oracle,
 )

@@ -133,6 +133,56 @@ def varlen_oracle(q, k, v, cu_seqlens_q, cu_seqlens_k, is_causal: bool = False, 
     return out, lse
 
 
+def sdpa_backward_oracle(q, k, v, dout, is_causal: bool = False, scale: Optional[float] = None, dtype=np.float64
+                         ) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
+    """Gradients of the dense op.  q, dout [B, Hq, Sq, D], k/v [B, Hk, Sk, D] -> (dq, dk, dv) with the inputs' shapes.
+
+    The reference has no backward oracle of its own — its tests differentiate `attention_ref` with autograd
+    (test/torch_ops/test_scaled_dot_product_attention.py:1049-1113) — so this is the closed form of that derivative:
+        P = softmax(scale Q K^T + mask),  dV = P^T dO,  dP = dO V^T,  dS = P o (dP - rowsum(dO o O)),
+        dQ = scale dS K,  dK = scale dS^T Q,
+    with dK, dV of a kv head summed over the query heads that read it (the "(h g)" repeat at :119-120 differentiated).
+    Pinned in tests/test_oracle.py against torch.autograd on PyTorch's float64 math SDPA."""
+    q, k, v, dout = _np(q, dtype), _np(k, dtype), _np(v, dtype), _np(dout, dtype)
+    B, Hq, Sq, D = q.shape
+    Hk, Sk = k.shape[1], k.shape[2]
+    g = Hq // Hk
+    sc = (1.0 / math.sqrt(D)) if scale is None else float(scale)
+    out, p, _ = attention_ref(q.transpose(0, 2, 1, 3), k.transpose(0, 2, 1, 3), v.transpose(0, 2, 1, 3), scale=scale,
+                              causal=is_causal, dtype=dtype)      # out [B,Hq,Sq,D], p [B,Hq,Sq,Sk]
+    kr = np.repeat(k, g, axis=1)
+    vr = np.repeat(v, g, axis=1)
+    dv_r = np.matmul(p.transpose(0, 1, 3, 2), dout)                 # [B,Hq,Sk,D]
+    dp = np.matmul(dout, vr.transpose(0, 1, 3, 2))                  # [B,Hq,Sq,Sk]
+    delta = (dout * out).sum(axis=-1, keepdims=True)
+    ds = p * (dp - delta)
+    dq = sc * np.matmul(ds, kr)
+    dk_r = sc * np.matmul(ds.transpose(0, 1, 3, 2), q)
+    dk = dk_r.reshape(B, Hk, g, Sk, D).sum(axis=2)
+    dv = dv_r.reshape(B, Hk, g, Sk, D).sum(axis=2)
+    return dq, dk, dv
+
+
+def varlen_backward_oracle(q, k, v, dout, cu_seqlens_q, cu_seqlens_k, is_causal: bool = False,
+                           scale: Optional[float] = None, dtype=np.float64):
+    """Packed layout: q, dout [Tq, Hq, D], k/v [Tk, Hk, D] -> (dq, dk, dv); every sequence independently."""
+    q, k, v, dout = _np(q, dtype), _np(k, dtype), _np(v, dtype), _np(dout, dtype)
+    cq = np.asarray(cu_seqlens_q.cpu() if hasattr(cu_seqlens_q, "cpu") else cu_seqlens_q, dtype=np.int64)
+    ck = np.asarray(cu_seqlens_k.cpu() if hasattr(cu_seqlens_k, "cpu") else cu_seqlens_k, dtype=np.int64)
+    dq, dk, dv = np.zeros_like(q), np.zeros_like(k), np.zeros_like(v)
+    for b in range(len(cq) - 1):
+        q0, q1, k0, k1 = cq[b], cq[b + 1], ck[b], ck[b + 1]
+        if q1 <= q0 or k1 <= k0:
+            continue
+        a, bb, cc = sdpa_backward_oracle(q[q0:q1].transpose(1, 0, 2)[None], k[k0:k1].transpose(1, 0, 2)[None],
+                                         v[k0:k1].transpose(1, 0, 2)[None], dout[q0:q1].transpose(1, 0, 2)[None],
+                                         is_causal=is_causal, scale=scale, dtype=dtype)
+        dq[q0:q1] = a[0].transpose(1, 0, 2)
+        dk[k0:k1] = bb[0].transpose(1, 0, 2)
+        dv[k0:k1] = cc[0].transpose(1, 0, 2)
+    return dq, dk, dv
+
+
 def get_tolerances(true_value, computed_value, dtype_name: str, fudge_factor: Optional[float] = 2.0
                    ) -> Tuple[float, float]:
     """Restates test_scaled_dot_product_attention.py:166-204: the allowed error is `fudge_factor` times the error

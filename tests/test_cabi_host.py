@@ -1,4 +1,4 @@
-"""Host-only checks of the C ABI (include/fa_fwd.h / libfa_fwd.so): the library loads, exports every declared
+"""Host-only checks of the C ABI (include/fa_fwd.h, include/fa_bwd.h / libfa_fwd.so): the library loads, exports every declared
 symbol, and its argument validation / planning — which never touch the GPU — return the documented codes."""
 import ctypes
 import os
@@ -12,9 +12,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "fa_fwd.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(fa_fwd_[a-z_]+)\s*\(", text)))
+    syms = set()
+    for header in ("fa_fwd.h", "fa_bwd.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        syms |= set(re.findall(r"\b(fa_(?:fwd|bwd)_[a-z_]+)\s*\(", text))
+    return sorted(syms)
 
 
 def test_library_exports_every_declared_symbol():
@@ -124,3 +127,63 @@ def test_plan_decode_uses_splitkv_and_sizes_workspace():
     # wide GQA groups (> 16 query heads per kv head) fall back to the tile kernel
     p = _good(batch=1, heads_q=32, heads_k=1, seqlen_q=1, seqlen_k=4096)
     assert _plan(p)[1] == capi.FA_KERNEL_TILE
+
+
+# ---- backward entry points ------------------------------------------------------------------------------------------
+def _good_bwd(**over):
+    p = capi.FaBwdParams()
+    p.q, p.k, p.v, p.out, p.dout, p.lse = 0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000
+    p.dq, p.dk, p.dv = 0x7000, 0x8000, 0x9000
+    B, Hq, Hk, Sq, Sk, D = 2, 8, 2, 128, 256, 128
+    for n, (S, H) in dict(q=(Sq, Hq), o=(Sq, Hq), do=(Sq, Hq), dq=(Sq, Hq), k=(Sk, Hk), v=(Sk, Hk), dk=(Sk, Hk),
+                          dv=(Sk, Hk)).items():
+        setattr(p, n + "_stride_b", S * H * D)
+        setattr(p, n + "_stride_s", H * D)
+        setattr(p, n + "_stride_h", D)
+    p.lse_stride_b, p.lse_stride_h, p.lse_stride_s = Hq * Sq, Sq, 1
+    p.batch, p.heads_q, p.heads_k, p.seqlen_q, p.seqlen_k, p.head_dim = B, Hq, Hk, Sq, Sk, D
+    p.total_q = 0
+    p.scale, p.dtype, p.is_causal, p.reserved = 0.088, capi.FA_DTYPE_BF16, 1, 0
+    for k, v in over.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_bwd_validate_accepts_good_params_and_sizes_delta_scratch():
+    L = capi.lib()
+    p = _good_bwd()
+    assert L.fa_bwd_validate(ctypes.byref(p)) == capi.FA_OK
+    assert L.fa_bwd_workspace_bytes(ctypes.byref(p)) == 2 * 128 * 8 * 4      # fp32 per (batch, row, query head)
+    packed = _good_bwd(cu_seqlens_q=0xa000, cu_seqlens_k=0xb000, total_q=200)
+    assert L.fa_bwd_validate(ctypes.byref(packed)) == capi.FA_OK
+    assert L.fa_bwd_workspace_bytes(ctypes.byref(packed)) == 200 * 8 * 4
+
+
+@pytest.mark.parametrize("over,rc", [
+    (dict(dout=None), capi.FA_ERR_BAD_ARG),
+    (dict(dk=None), capi.FA_ERR_BAD_ARG),
+    (dict(lse=None), capi.FA_ERR_BAD_ARG),
+    (dict(dv=0x9004), capi.FA_ERR_BAD_ARG),
+    (dict(do_stride_s=1028), capi.FA_ERR_BAD_ARG),
+    (dict(batch=0), capi.FA_ERR_BAD_ARG),
+    (dict(reserved=3), capi.FA_ERR_BAD_ARG),
+    (dict(cu_seqlens_k=0xb000), capi.FA_ERR_BAD_ARG),
+    (dict(head_dim=136), capi.FA_ERR_UNSUPPORTED),      # the reference's backward stops at 128 as well
+    (dict(head_dim=100), capi.FA_ERR_UNSUPPORTED),
+    (dict(dtype=3), capi.FA_ERR_UNSUPPORTED),
+    (dict(heads_k=3), capi.FA_ERR_UNSUPPORTED),
+])
+def test_bwd_validate_rejects(over, rc):
+    L = capi.lib()
+    p = _good_bwd(**over)
+    assert L.fa_bwd_validate(ctypes.byref(p)) == rc
+    assert L.fa_bwd_workspace_bytes(ctypes.byref(p)) == 0
+    assert L.fa_bwd_launch(ctypes.byref(p), None, 0, None) == rc     # refused before anything is enqueued
+
+
+def test_bwd_null_and_short_workspace():
+    L = capi.lib()
+    assert L.fa_bwd_validate(None) == capi.FA_ERR_BAD_ARG
+    p = _good_bwd()
+    assert L.fa_bwd_launch(ctypes.byref(p), 0x10000, 16, None) == capi.FA_ERR_BAD_ARG
+    assert L.fa_bwd_launch(ctypes.byref(p), None, 1 << 20, None) == capi.FA_ERR_BAD_ARG

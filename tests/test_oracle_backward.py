@@ -1,0 +1,153 @@
+"""Pins the backward oracle (oracle.sdpa_backward_oracle / varlen_backward_oracle) — against torch.autograd on
+float64 math attention (library routine), against central finite differences of the forward oracle (brute force),
+and against closed forms and invariants that a dropped delta term, a wrong sign, a missing scale or a transposed
+operand would break.  Runs without a GPU."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests._util import seeded
+
+
+def _autograd_ref(q, k, v, dout, causal, scale):
+    """d/d(q,k,v) of softmax(scale q k^T + bottom-right causal mask) v, float64, written with plain torch ops."""
+    q, k, v = (t.double().clone().requires_grad_() for t in (q, k, v))
+    B, Hq, Sq, D = q.shape
+    Hk, Sk = k.shape[1], k.shape[2]
+    kr = k.repeat_interleave(Hq // Hk, dim=1)
+    vr = v.repeat_interleave(Hq // Hk, dim=1)
+    s = torch.matmul(q, kr.transpose(-1, -2)) * (1.0 / math.sqrt(D) if scale is None else scale)
+    if causal:
+        i = torch.arange(Sq)[:, None]
+        j = torch.arange(Sk)[None, :]
+        s = s.masked_fill(j > i + (Sk - Sq), float("-inf"))
+    out = torch.matmul(torch.softmax(s, dim=-1), vr)
+    out.backward(dout.double())
+    return q.grad.numpy(), k.grad.numpy(), v.grad.numpy()
+
+
+def _inputs(B, Hq, Hk, Sq, Sk, D, seed):
+    return (seeded((B, Hq, Sq, D), seed, torch.float32), seeded((B, Hk, Sk, D), seed + 1, torch.float32),
+            seeded((B, Hk, Sk, D), seed + 2, torch.float32), seeded((B, Hq, Sq, D), seed + 3, torch.float32))
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(1, 1, 1, 8, 8, 16), (2, 4, 2, 33, 47, 32), (1, 6, 1, 40, 40, 64),
+                                   (2, 2, 2, 17, 64, 8)])
+@pytest.mark.parametrize("scale", [None, 0.3, -0.2])
+def test_backward_oracle_vs_autograd_float64(shape, causal, scale):
+    q, k, v, do = _inputs(*shape, seed=10)
+    got = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=causal, scale=scale)
+    want = _autograd_ref(q, k, v, do, causal, scale)
+    for g, w in zip(got, want):
+        assert g.shape == w.shape
+        assert np.abs(g - w).max() < 1e-12
+
+
+def test_backward_oracle_vs_finite_differences():
+    """Central differences of the forward oracle's <out, dout>: no shared derivative code at all."""
+    B, Hq, Hk, Sq, Sk, D = 1, 2, 1, 3, 5, 4
+    q, k, v, do = (t.double().numpy() for t in _inputs(B, Hq, Hk, Sq, Sk, D, seed=77))
+    dq, dk, dv = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True, scale=0.7)
+
+    def f(q_, k_, v_):
+        out, _ = oracle.sdpa_oracle(q_, k_, v_, is_causal=True, scale=0.7)
+        return float((out * do).sum())
+
+    h = 1e-6
+    for x, g, pos in ((q, dq, 0), (k, dk, 1), (v, dv, 2)):
+        num = np.zeros_like(x)
+        for idx in np.ndindex(*x.shape):
+            xp, xm = x.copy(), x.copy()
+            xp[idx] += h
+            xm[idx] -= h
+            args_p, args_m = [q, k, v], [q, k, v]
+            args_p[pos], args_m[pos] = xp, xm
+            num[idx] = (f(*args_p) - f(*args_m)) / (2 * h)
+        assert np.abs(num - g).max() < 1e-8
+
+
+def test_zero_query_closed_form():
+    """q = 0: P is uniform over the visible keys, so dV[j] = sum over the rows that see j of dO[i]/n_i, dK = 0 (it is
+    multiplied by q), and dQ = scale * sum_j P_ij (dP_ij - delta_i) K_j with delta_i = mean_j dP_ij."""
+    B, H, Sq, Sk, D = 1, 1, 4, 6, 8
+    _, k, v, do = (t.double().numpy() for t in _inputs(B, H, H, Sq, Sk, D, seed=5))
+    q = np.zeros((B, H, Sq, D))
+    dq, dk, dv = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True, scale=0.5)
+    assert np.abs(dk).max() == 0.0
+    want_dv = np.zeros_like(v)
+    want_dq = np.zeros_like(q)
+    for i in range(Sq):
+        n = i + (Sk - Sq) + 1
+        want_dv[0, 0, :n] += do[0, 0, i] / n
+        dp = v[0, 0, :n] @ do[0, 0, i]
+        want_dq[0, 0, i] = 0.5 * ((dp - dp.mean()) / n) @ k[0, 0, :n]
+    assert np.abs(dv - want_dv).max() < 1e-14
+    assert np.abs(dq - want_dq).max() < 1e-14
+
+
+def test_invariants_of_the_softmax_jacobian():
+    """(1) <dQ, Q> == <dK, K> (both are scale * <dS, Q K^T>); (2) adding a constant vector c to every value row adds c
+    to every output row, so dQ and dK do not change; (3) dV summed over keys equals dO summed over rows, per head
+    group (P's rows sum to one)."""
+    q, k, v, do = (t.double().numpy() for t in _inputs(2, 4, 2, 19, 23, 16, seed=31))
+    dq, dk, dv = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=False)
+    assert abs((dq * q).sum() - (dk * k).sum()) < 1e-11
+    dq2, dk2, dv2 = oracle.sdpa_backward_oracle(q, k, v + 3.25, do, is_causal=False)
+    assert np.abs(dq2 - dq).max() < 1e-12 and np.abs(dk2 - dk).max() < 1e-12 and np.abs(dv2 - dv).max() < 1e-12
+    want = do.reshape(2, 2, 2, 19, 16).sum(axis=(2, 3))
+    assert np.abs(dv.sum(axis=2) - want).max() < 1e-12
+
+
+def test_scale_enters_once_and_sign_flips():
+    """Scaling q by a and the scale by 1/a leaves S unchanged: dK is unchanged and dQ shrinks by a."""
+    q, k, v, do = (t.double().numpy() for t in _inputs(1, 2, 2, 9, 11, 8, seed=3))
+    dq, dk, dv = oracle.sdpa_backward_oracle(q, k, v, do, scale=0.4)
+    dq2, dk2, dv2 = oracle.sdpa_backward_oracle(q * -2.0, k, v, do, scale=-0.2)
+    assert np.abs(dq2 * -2.0 - dq).max() < 1e-13
+    assert np.abs(dk2 - dk).max() < 1e-13 and np.abs(dv2 - dv).max() < 1e-13
+
+
+def test_rows_without_visible_keys_have_zero_gradient():
+    """Causal with Sq > Sk: the first Sq - Sk rows see no key, their output is 0 and nothing flows through them."""
+    q, k, v, do = (t.double().numpy() for t in _inputs(1, 2, 1, 7, 3, 8, seed=8))
+    dq, dk, dv = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True)
+    assert np.abs(dq[:, :, :4]).max() == 0.0
+    assert all(np.isfinite(x).all() for x in (dq, dk, dv))
+    # the visible part is an ordinary 3x3 causal problem
+    dq3, dk3, dv3 = oracle.sdpa_backward_oracle(q[:, :, 4:], k, v, do[:, :, 4:], is_causal=True)
+    assert np.abs(dq[:, :, 4:] - dq3).max() < 1e-14
+    assert np.abs(dk - dk3).max() < 1e-14 and np.abs(dv - dv3).max() < 1e-14
+
+
+def test_gqa_gradient_is_the_sum_over_the_group():
+    q, k, v, do = (t.double().numpy() for t in _inputs(1, 6, 2, 10, 12, 8, seed=12))
+    dq, dk, dv = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True)
+    kr, vr = np.repeat(k, 3, axis=1), np.repeat(v, 3, axis=1)
+    dq_m, dk_m, dv_m = oracle.sdpa_backward_oracle(q, kr, vr, do, is_causal=True)
+    assert np.abs(dq - dq_m).max() < 1e-14
+    assert np.abs(dk - dk_m.reshape(1, 2, 3, 12, 8).sum(2)).max() < 1e-13
+    assert np.abs(dv - dv_m.reshape(1, 2, 3, 12, 8).sum(2)).max() < 1e-13
+
+
+def test_packed_backward_equals_per_sequence_dense():
+    lens_q, lens_k = [5, 0, 9, 3], [7, 4, 9, 6]
+    cu_q, cu_k = np.concatenate([[0], np.cumsum(lens_q)]), np.concatenate([[0], np.cumsum(lens_k)])
+    Hq, Hk, D = 4, 2, 8
+    q = seeded((int(cu_q[-1]), Hq, D), 1, torch.float32).double().numpy()
+    k = seeded((int(cu_k[-1]), Hk, D), 2, torch.float32).double().numpy()
+    v = seeded((int(cu_k[-1]), Hk, D), 3, torch.float32).double().numpy()
+    do = seeded((int(cu_q[-1]), Hq, D), 4, torch.float32).double().numpy()
+    dq, dk, dv = oracle.varlen_backward_oracle(q, k, v, do, cu_q, cu_k, is_causal=True)
+    for b in range(4):
+        qs, ks = slice(cu_q[b], cu_q[b + 1]), slice(cu_k[b], cu_k[b + 1])
+        if lens_q[b] == 0:
+            assert np.abs(dk[ks]).max() == 0.0 and np.abs(dv[ks]).max() == 0.0   # keys nobody reads
+            continue
+        w = _autograd_ref(*(torch.from_numpy(x).transpose(0, 1)[None] for x in (q[qs], k[ks], v[ks], do[qs])),
+                          True, None)
+        for g, r in zip((dq[qs], dk[ks], dv[ks]), w):
+            assert np.abs(g - r[0].transpose(1, 0, 2)).max() < 1e-12

@@ -33,11 +33,13 @@ def _run(cmd, **kw):
 
 
 def build_kernels(verbose: bool = False) -> str:
-    """hipcc: csrc/fa_fwd_kernels.hip -> lib/libfa_fwd.so (the C ABI of include/fa_fwd.h)."""
+    """hipcc: csrc/fa_fwd_kernels.hip + csrc/fa_bwd_kernels.hip -> lib/libfa_fwd.so (the C ABI of include/fa_fwd.h and
+    include/fa_bwd.h)."""
     os.makedirs(LIBDIR, exist_ok=True)
     out = os.path.join(LIBDIR, "libfa_fwd.so")
     tmp = out + ".tmp"
-    log = _run([HIPCC, *HIP_FLAGS, "-shared", f"-I{INCLUDE}", os.path.join(CSRC, "fa_fwd_kernels.hip"), "-o", tmp])
+    srcs = [os.path.join(CSRC, f) for f in ("fa_fwd_kernels.hip", "fa_bwd_kernels.hip") if os.path.exists(os.path.join(CSRC, f))]
+    log = _run([HIPCC, *HIP_FLAGS, "-shared", f"-I{INCLUDE}", f"-I{CSRC}", *srcs, "-o", tmp])
     os.replace(tmp, out)
     if verbose and log.strip():
         print(log)

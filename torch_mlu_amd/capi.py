@@ -40,6 +40,9 @@ EXPORTED_SYMBOLS = (
     "fa_fwd_workspace_bytes",
     "fa_fwd_launch",
     "fa_fwd_plan",
+    "fa_bwd_validate",
+    "fa_bwd_workspace_bytes",
+    "fa_bwd_launch",
 )
 
 
@@ -74,6 +77,20 @@ class FaFwdParams(ctypes.Structure):
     ]
 
 
+class FaBwdParams(ctypes.Structure):
+    """Mirror of `struct fa_bwd_params` (include/fa_bwd.h)."""
+
+    _fields_ = (
+        [(n, ctypes.c_void_p) for n in ("q", "k", "v", "out", "dout", "lse", "dq", "dk", "dv", "cu_seqlens_q",
+                                        "cu_seqlens_k")]
+        + [(f"{t}_stride_{d}", ctypes.c_int64) for t in ("q", "k", "v", "o", "do", "dq", "dk", "dv") for d in "bsh"]
+        + [("lse_stride_b", ctypes.c_int64), ("lse_stride_h", ctypes.c_int64), ("lse_stride_s", ctypes.c_int64)]
+        + [(n, ctypes.c_int32) for n in ("batch", "heads_q", "heads_k", "seqlen_q", "seqlen_k", "head_dim")]
+        + [("total_q", ctypes.c_int64), ("scale", ctypes.c_float)]
+        + [(n, ctypes.c_int32) for n in ("dtype", "is_causal", "reserved")]
+    )
+
+
 _lib = None
 
 
@@ -99,6 +116,12 @@ def lib() -> ctypes.CDLL:
         L.fa_fwd_plan.restype = ctypes.c_int
         L.fa_fwd_plan.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.POINTER(ctypes.c_int32),
                                   ctypes.POINTER(ctypes.c_int32)]
+        L.fa_bwd_validate.restype = ctypes.c_int
+        L.fa_bwd_validate.argtypes = [ctypes.POINTER(FaBwdParams)]
+        L.fa_bwd_workspace_bytes.restype = ctypes.c_size_t
+        L.fa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(FaBwdParams)]
+        L.fa_bwd_launch.restype = ctypes.c_int
+        L.fa_bwd_launch.argtypes = [ctypes.POINTER(FaBwdParams), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         _lib = L
     return _lib
 
@@ -205,3 +228,77 @@ def fa_forward_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seql
                     kernel=kernel, num_splits=num_splits)
     launch(p, q.device)
     return out, lse
+
+
+def _set_strides(p, name, t, packed):
+    if packed:
+        setattr(p, f"{name}_stride_b", 0)
+        setattr(p, f"{name}_stride_s", t.stride(0))
+        setattr(p, f"{name}_stride_h", t.stride(1))
+    else:
+        setattr(p, f"{name}_stride_b", t.stride(0))
+        setattr(p, f"{name}_stride_s", t.stride(1))
+        setattr(p, f"{name}_stride_h", t.stride(2))
+
+
+def fa_backward_dense(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
+                      lse: torch.Tensor, *, is_causal: bool = False, scale: Optional[float] = None
+                      ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """All of dout, q, out [B, Hq, Sq, D] and k, v [B, Hk, Sk, D] (any strides, contiguous last dim), lse [B, Hq, Sq]
+    -> (dq, dk, dv) stored [B, S, H, D] and returned as [B, H, S, D] views, like the reference's dense wrapper
+    (torch_mlu/csrc/aten/operators/cnnl/transformers/attention.cpp:297-302)."""
+    B, Hq, Sq, D = q.shape
+    Hk, Sk = k.shape[1], k.shape[2]
+    dq = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+    dk = torch.empty((B, Sk, Hk, D), dtype=q.dtype, device=q.device)
+    dv = torch.empty((B, Sk, Hk, D), dtype=q.dtype, device=q.device)
+    p = FaBwdParams()
+    views = {"q": q.transpose(1, 2), "k": k.transpose(1, 2), "v": v.transpose(1, 2), "o": out.transpose(1, 2),
+             "do": dout.transpose(1, 2), "dq": dq, "dk": dk, "dv": dv}
+    p.q, p.k, p.v, p.out, p.dout = (views[n].data_ptr() for n in ("q", "k", "v", "o", "do"))
+    p.lse, p.dq, p.dk, p.dv = lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    p.cu_seqlens_q = None
+    p.cu_seqlens_k = None
+    for n, t in views.items():
+        _set_strides(p, n, t, False)
+    p.lse_stride_b, p.lse_stride_h, p.lse_stride_s = lse.stride(0), lse.stride(1), lse.stride(2)
+    p.batch, p.heads_q, p.heads_k, p.seqlen_q, p.seqlen_k, p.head_dim = B, Hq, Hk, Sq, Sk, D
+    p.total_q = 0
+    p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
+    p.dtype, p.is_causal, p.reserved = _dtype_code(q.dtype), 1 if is_causal else 0, 0
+    _launch_bwd(p, q.device)
+    return dq.transpose(1, 2), dk.transpose(1, 2), dv.transpose(1, 2)
+
+
+def fa_backward_packed(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, max_seqlen_k: int, *,
+                       is_causal: bool = False, scale: Optional[float] = None):
+    """Packed: dout, q, out [Tq, Hq, D], k, v [Tk, Hk, D], lse [Hq, Tq] -> (dq, dk, dv) with the inputs' shapes."""
+    Tq, Hq, D = q.shape
+    dq, dk, dv = torch.empty_like(q, memory_format=torch.contiguous_format), torch.empty_like(
+        k, memory_format=torch.contiguous_format), torch.empty_like(v, memory_format=torch.contiguous_format)
+    p = FaBwdParams()
+    views = {"q": q, "k": k, "v": v, "o": out, "do": dout, "dq": dq, "dk": dk, "dv": dv}
+    p.q, p.k, p.v, p.out, p.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr()
+    p.lse, p.dq, p.dk, p.dv = lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    p.cu_seqlens_q, p.cu_seqlens_k = cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr()
+    for n, t in views.items():
+        _set_strides(p, n, t, True)
+    p.lse_stride_b, p.lse_stride_h, p.lse_stride_s = 0, lse.stride(0), lse.stride(1)
+    p.batch, p.heads_q, p.heads_k = cu_seqlens_q.numel() - 1, Hq, k.shape[1]
+    p.seqlen_q, p.seqlen_k, p.head_dim, p.total_q = max_seqlen_q, max_seqlen_k, D, Tq
+    p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
+    p.dtype, p.is_causal, p.reserved = _dtype_code(q.dtype), 1 if is_causal else 0, 0
+    _launch_bwd(p, q.device)
+    return dq, dk, dv
+
+
+def _launch_bwd(p: FaBwdParams, device: torch.device) -> None:
+    L = lib()
+    rc = L.fa_bwd_validate(ctypes.byref(p))
+    if rc != FA_OK:
+        raise FaFwdError(rc)
+    need = L.fa_bwd_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    rc = L.fa_bwd_launch(ctypes.byref(p), ws.data_ptr(), need, torch.cuda.current_stream(device).cuda_stream)
+    if rc != FA_OK:
+        raise FaFwdError(rc)

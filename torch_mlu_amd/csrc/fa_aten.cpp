@@ -31,6 +31,7 @@
 #include <mutex>
 #include <tuple>
 
+#include "fa_bwd.h"
 #include "fa_fwd.h"
 
 namespace torch_mlu_amd {
@@ -278,6 +279,122 @@ scaled_dot_product_flash_attention(const at::Tensor& query, const at::Tensor& ke
                          philox_offset, debug_attn_mask);
 }
 
+// ---- _flash_attention_backward --------------------------------------------------------------------------------
+// cnnl__flash_attention_backward, attention.cpp:305-348, and the checks of mha_varlen_bwd
+// (FlashAttention_internal.cpp:288-366).  3-D inputs: packed [T, H, D] with cum_seq (the reference's only mode);
+// 4-D inputs: dense [B, S, H, D] views (cum_seq ignored), which is how the dense wrapper below calls it.
+std::tuple<at::Tensor, at::Tensor, at::Tensor> flash_attention_backward(
+    const at::Tensor& grad_out, const at::Tensor& query, const at::Tensor& key, const at::Tensor& value,
+    const at::Tensor& out, const at::Tensor& logsumexp, const at::Tensor& cum_seq_q, const at::Tensor& cum_seq_k,
+    int64_t max_q, int64_t max_k, double dropout_p, bool is_causal, const at::Tensor& philox_seed,
+    const at::Tensor& philox_offset, std::optional<double> scale, std::optional<int64_t> window_size_left,
+    std::optional<int64_t> window_size_right) {
+  (void)philox_seed;
+  (void)philox_offset;
+  TORCH_CHECK(dropout_p == 0.0, "flash attention backward: dropout_p > 0 is not supported by this build");
+  TORCH_CHECK(!window_size_left.has_value() || *window_size_left < 0, "flash attention backward: sliding window is not supported");
+  TORCH_CHECK(!window_size_right.has_value() || *window_size_right < 0 || (is_causal && *window_size_right == 0),
+              "flash attention backward: sliding window is not supported");
+  const bool packed = query.dim() == 3;
+  if (packed) TORCH_CHECK(cum_seq_q.defined() && cum_seq_k.defined(), "packed inputs need cum_seq_q and cum_seq_k");
+  Packed pk{packed ? &cum_seq_q : nullptr, packed ? &cum_seq_k : nullptr, max_q, max_k};
+  check_inputs(query, key, value, packed ? &pk : nullptr, /*require_device=*/true);
+  TORCH_CHECK(grad_out.scalar_type() == query.scalar_type(), "query and dout must have the same dtype");
+  TORCH_CHECK(out.scalar_type() == query.scalar_type(), "query and out must have the same dtype");
+  TORCH_CHECK(grad_out.sizes() == query.sizes() && out.sizes() == query.sizes(), "dout and out must have the shape of query");
+  TORCH_CHECK(logsumexp.scalar_type() == at::kFloat && logsumexp.is_cuda(), "logsumexp must be a float32 tensor on the device");
+  TORCH_CHECK(query.size(-1) <= 128, "FlashAttention backward only supports head dimension at most 128 in this build");
+
+  const c10::OptionalDeviceGuard guard(query.device());
+  const float softmax_scale = resolve_scale(query, scale);
+  auto fix = [](const at::Tensor& t) { return t.stride(-1) == 1 ? aligned_or_copy(t) : t.contiguous(); };
+  const at::Tensor q = aligned_or_copy(query), k = aligned_or_copy(key), v = aligned_or_copy(value);
+  const at::Tensor dout = fix(grad_out), o = fix(out);  // the reference makes both contiguous (attention.cpp:324-325)
+  at::Tensor dq = at::empty(q.sizes(), q.options());
+  at::Tensor dk = at::empty(k.sizes(), k.options());
+  at::Tensor dv = at::empty(v.sizes(), v.options());
+
+  const int64_t batch = packed ? cum_seq_q.numel() - 1 : q.size(0);
+  const int64_t heads = q.size(-2);
+  const int64_t seqlen_q = packed ? max_q : q.size(1);
+  const int64_t seqlen_k = packed ? max_k : k.size(1);
+  const int64_t total_q = packed ? q.size(0) : batch * seqlen_q;
+  if (packed) {
+    TORCH_CHECK(logsumexp.dim() == 2 && logsumexp.size(0) == heads && logsumexp.size(1) == total_q,
+                "logsumexp must have shape (num_heads, total_q)");
+  } else {
+    TORCH_CHECK(logsumexp.dim() == 3 && logsumexp.size(0) == batch && logsumexp.size(1) == heads &&
+                    logsumexp.size(2) >= seqlen_q,
+                "logsumexp must have shape (batch_size, num_heads, seqlen_q)");
+  }
+
+  fa_bwd_params p{};
+  p.q = q.data_ptr(); p.k = k.data_ptr(); p.v = v.data_ptr(); p.out = o.data_ptr(); p.dout = dout.data_ptr();
+  p.lse = logsumexp.data_ptr<float>();
+  p.dq = dq.data_ptr(); p.dk = dk.data_ptr(); p.dv = dv.data_ptr();
+  p.cu_seqlens_q = packed ? cum_seq_q.data_ptr<int32_t>() : nullptr;
+  p.cu_seqlens_k = packed ? cum_seq_k.data_ptr<int32_t>() : nullptr;
+  fill_strides(q, packed, p.q_stride_b, p.q_stride_s, p.q_stride_h);
+  fill_strides(k, packed, p.k_stride_b, p.k_stride_s, p.k_stride_h);
+  fill_strides(v, packed, p.v_stride_b, p.v_stride_s, p.v_stride_h);
+  fill_strides(o, packed, p.o_stride_b, p.o_stride_s, p.o_stride_h);
+  fill_strides(dout, packed, p.do_stride_b, p.do_stride_s, p.do_stride_h);
+  fill_strides(dq, packed, p.dq_stride_b, p.dq_stride_s, p.dq_stride_h);
+  fill_strides(dk, packed, p.dk_stride_b, p.dk_stride_s, p.dk_stride_h);
+  fill_strides(dv, packed, p.dv_stride_b, p.dv_stride_s, p.dv_stride_h);
+  if (packed) {
+    p.lse_stride_b = 0; p.lse_stride_h = logsumexp.stride(0); p.lse_stride_s = logsumexp.stride(1);
+  } else {
+    p.lse_stride_b = logsumexp.stride(0); p.lse_stride_h = logsumexp.stride(1); p.lse_stride_s = logsumexp.stride(2);
+  }
+  p.batch = static_cast<int32_t>(batch);
+  p.heads_q = static_cast<int32_t>(heads);
+  p.heads_k = static_cast<int32_t>(k.size(-2));
+  p.seqlen_q = static_cast<int32_t>(seqlen_q);
+  p.seqlen_k = static_cast<int32_t>(seqlen_k);
+  p.head_dim = static_cast<int32_t>(q.size(-1));
+  p.total_q = total_q;
+  p.scale = softmax_scale;
+  p.dtype = q.scalar_type() == at::kBFloat16 ? FA_DTYPE_BF16 : FA_DTYPE_FP16;
+  p.is_causal = is_causal ? 1 : 0;
+
+  if (total_q == 0 || k.numel() == 0) {
+    dq.zero_(); dk.zero_(); dv.zero_();
+    return std::make_tuple(dq, dk, dv);
+  }
+  const size_t ws_bytes = fa_bwd_workspace_bytes(&p);
+  at::Tensor ws = at::empty({static_cast<int64_t>(ws_bytes > 0 ? ws_bytes : 16)}, q.options().dtype(at::kByte));
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
+  const int rc = fa_bwd_launch(&p, ws.data_ptr(), ws_bytes, stream);
+  TORCH_CHECK(rc == FA_OK, "fa_bwd_launch failed: ", fa_fwd_error_string(rc), " (rc=", rc, ")");
+  g_launches.fetch_add(1, std::memory_order_relaxed);
+  return std::make_tuple(dq, dk, dv);
+}
+
+// ---- _scaled_dot_product_flash_attention_backward -------------------------------------------------------------
+// cnnl__scaled_dot_product_flash_attention_backward, attention.cpp:205-303 — without its contiguous copies.
+std::tuple<at::Tensor, at::Tensor, at::Tensor> scaled_dot_product_flash_attention_backward(
+    const at::Tensor& grad_out, const at::Tensor& query, const at::Tensor& key, const at::Tensor& value,
+    const at::Tensor& out, const at::Tensor& logsumexp, const at::Tensor& cum_seq_q, const at::Tensor& cum_seq_k,
+    int64_t max_q, int64_t max_k, double dropout_p, bool is_causal, const at::Tensor& philox_seed,
+    const at::Tensor& philox_offset, std::optional<double> scale) {
+  if (!grad_out.defined()) return std::make_tuple(at::Tensor{}, at::Tensor{}, at::Tensor{});  // attention.cpp:222-224
+  TORCH_CHECK(query.dim() == 4 && key.dim() == 4 && value.dim() == 4 && grad_out.dim() == 4,
+              "query, key, value and grad_out must be 4-dimensional (batch, num_heads, seq_len, head_dim)");
+  TORCH_CHECK(query.size(0) == grad_out.size(0) && query.size(0) == key.size(0) && query.size(0) == value.size(0),
+              "query, key, value and grad_out must have the same batch size");
+  TORCH_CHECK(key.size(2) == value.size(2), "Key and Value must have the same sequence length");
+  TORCH_CHECK(query.size(2) == grad_out.size(2) && query.size(1) == grad_out.size(1), "grad_out must have the shape of query");
+  TORCH_CHECK(query.size(3) == key.size(3) && value.size(3) == grad_out.size(3),
+              "query, key, value and grad_out must have the same head dimension");
+  auto [grad_q, grad_k, grad_v] = at::_flash_attention_backward(
+      grad_out.transpose(1, 2), query.transpose(1, 2), key.transpose(1, 2), value.transpose(1, 2),
+      out.transpose(1, 2), logsumexp, cum_seq_q, cum_seq_k, max_q, max_k, dropout_p, is_causal, philox_seed,
+      philox_offset, scale, std::nullopt, std::nullopt);
+  // [B,S,H,D] storage returned as [B,H,S,D] views (attention.cpp:297-302)
+  return std::make_tuple(grad_q.transpose(1, 2), grad_k.transpose(1, 2), grad_v.transpose(1, 2));
+}
+
 // ---- test hooks -----------------------------------------------------------------------------------------------
 int64_t launch_count() { return g_launches.load(std::memory_order_relaxed); }
 
@@ -298,6 +415,9 @@ void validate_flash_inputs(const at::Tensor& query, const at::Tensor& key, const
 TORCH_LIBRARY_IMPL(aten, CUDA, m) {
   m.impl("_scaled_dot_product_flash_attention", TORCH_FN(torch_mlu_amd::scaled_dot_product_flash_attention));
   m.impl("_flash_attention_forward", TORCH_FN(torch_mlu_amd::flash_attention_forward));
+  m.impl("_scaled_dot_product_flash_attention_backward",
+         TORCH_FN(torch_mlu_amd::scaled_dot_product_flash_attention_backward));
+  m.impl("_flash_attention_backward", TORCH_FN(torch_mlu_amd::flash_attention_backward));
 }
 
 TORCH_LIBRARY(torch_mlu_amd, m) {

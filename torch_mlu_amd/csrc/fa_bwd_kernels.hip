@@ -1,0 +1,594 @@
+// Flash-attention backward for MI355X (gfx950): HIP kernels and the C-ABI launcher declared in include/fa_bwd.h.
+//
+// Replaces the vendor call cnnlFlashAttentionBackward that torch_mlu's launcher makes
+// (torch_mlu/csrc/aten/operators/cnnl/internal/FlashAttention_internal.cpp:449-480) and its descriptor / workspace
+// plumbing (:368-447).
+//
+// Two kernels, no atomics, deterministic:
+//   fa_bwd_dq_kernel   — one workgroup = 128 query rows of one (sequence, head), loops over K/V tiles of 64 rows.
+//                        Per lane one query row (as in the forward): S^T = K Q^T, dP^T = V dO^T,
+//                        P^T = exp2(S^T c - LSE), dS^T = P^T o (dP^T - delta), dQ^T += K^T dS^T.
+//                        Also computes delta = rowsum(dO o O) for its rows and stores it for the second kernel.
+//   fa_bwd_dkv_kernel  — one workgroup = 128 key rows of one (sequence, kv head), loops over the query heads of the
+//                        GQA group and over Q/dO tiles of 64 rows.  Per lane one key row: S = Q K^T, dP = dO V^T,
+//                        P, dS as above, dV^T += dO^T P, dK^T += Q^T dS.
+// Both stream their tiles through LDS by global->LDS DMA with one XOR swizzle that is conflict-free for row reads
+// (ds_read_b128, MFMA A operand) and for transposed reads (ds_read_b64_tr_b16) of the same tile.
+// S and dP are recomputed in each kernel (7 matrix products per tile pair instead of 5) in exchange for not needing
+// fp32 atomics on dQ.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fa_bwd.h"
+#include "fa_device.h"
+
+namespace {
+
+using namespace fa;
+
+struct BArgs {
+  const unsigned char* q;
+  const unsigned char* k;
+  const unsigned char* v;
+  const unsigned char* o;
+  const unsigned char* dout;
+  const float* lse;
+  unsigned char* dq;
+  unsigned char* dk;
+  unsigned char* dv;
+  float* delta;  // dense [B][Hq][Sq], packed [Hq][total_q]
+  const int32_t* cu_q;
+  const int32_t* cu_k;
+  int64_t q_sb, q_ss, q_sh;  // byte strides
+  int64_t k_sb, k_ss, k_sh;
+  int64_t v_sb, v_ss, v_sh;
+  int64_t o_sb, o_ss, o_sh;
+  int64_t do_sb, do_ss, do_sh;
+  int64_t dq_sb, dq_ss, dq_sh;
+  int64_t dk_sb, dk_ss, dk_sh;
+  int64_t dv_sb, dv_ss, dv_sh;
+  int64_t lse_sb, lse_sh, lse_ss;  // element strides
+  int64_t dl_sb, dl_sh;            // delta strides (elements); row stride is 1
+  int32_t batch, heads_q, heads_k, group;
+  int32_t seqlen_q, seqlen_k, head_dim;
+  int32_t n_qblk, n_kblk;
+  int32_t is_causal;
+  float scale;       // signed softmax scale
+  float scale_log2;  // scale * log2(e), signed
+};
+
+// One swizzle for tiles that are read both by rows (16 lanes = 16 consecutive rows, same logical chunk) and
+// transposed (a half-wave = 4 consecutive rows x 4 consecutive chunks): physical chunk = logical ^ swzU(row).
+template <int DP>
+__device__ __forceinline__ int swzU(int row) {
+  if constexpr (DP == 64) return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+  return ((row & 3) << 2) | ((row >> 2) & 3);
+}
+
+template <typename T, int DP>
+struct TileIO {
+  static constexpr int CPR = DP / 8;
+  static constexpr int ROWB = DP * 2;
+  static constexpr int TILE = 64 * ROWB;
+  static constexpr int NI = TILE / 1024 / 4;
+  static constexpr int RPI = 64 / CPR;
+  static constexpr int KS = DP / 16;
+  static constexpr int MB = DP / 32;
+};
+
+// ---------------------------------------------------------------------------------------------------------
+// dQ kernel
+// ---------------------------------------------------------------------------------------------------------
+template <typename T, int DP>
+__global__ void __launch_bounds__(256, 1) fa_bwd_dq_kernel(const BArgs a) {
+  using IO = TileIO<T, DP>;
+  constexpr int CPR = IO::CPR, ROWB = IO::ROWB, TILE = IO::TILE, NI = IO::NI, RPI = IO::RPI, KS = IO::KS, MB = IO::MB;
+  constexpr int BM = 128, BN = 64;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // K0 K1 V0 V1
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 5, c32 = lane & 31;
+
+  const int lid = blockIdx.x;
+  const int mi = a.n_qblk - 1 - (lid % a.n_qblk);
+  const int bh = lid / a.n_qblk;
+  const int h = bh % a.heads_q, b = bh / a.heads_q;
+  const int hk = h / a.group;
+
+  int q0 = 0, k0 = 0, Lq = a.seqlen_q, Lk = a.seqlen_k;
+  int64_t qb = (int64_t)b * a.q_sb, kb = (int64_t)b * a.k_sb, vb = (int64_t)b * a.v_sb, ob = (int64_t)b * a.o_sb;
+  int64_t dob = (int64_t)b * a.do_sb, dqb = (int64_t)b * a.dq_sb;
+  int64_t lb = (int64_t)b * a.lse_sb, dlb = (int64_t)b * a.dl_sb;
+  if (a.cu_q) {
+    q0 = a.cu_q[b];
+    Lq = a.cu_q[b + 1] - q0;
+    k0 = a.cu_k[b];
+    Lk = a.cu_k[b + 1] - k0;
+    qb = kb = vb = ob = dob = dqb = 0;
+    lb = dlb = 0;
+  }
+  const int m0 = mi * BM;
+  if (m0 >= Lq) return;
+  const int off = Lk - Lq;
+  int n_end = Lk;
+  if (a.is_causal) n_end = min(Lk, m0 + BM + off);
+  if (n_end < 0) n_end = 0;
+  const int ntiles = (n_end + BN - 1) / BN;
+  const int D = a.head_dim;
+  const int row = m0 + 32 * wave + c32;
+  const int wave_row_lo = m0 + 32 * wave, wave_row_hi = wave_row_lo + 31;
+  const int last_k = Lk - 1;
+
+  const unsigned char* kp = a.k + kb + (int64_t)k0 * a.k_ss + (int64_t)hk * a.k_sh;
+  const unsigned char* vp = a.v + vb + (int64_t)k0 * a.v_ss + (int64_t)hk * a.v_sh;
+
+  // ---- DMA: rows clamped to the last valid one, logical chunk un-swizzled on the global side ----
+  const int dma_r = wave * RPI + lane / CPR;
+  int lc = (lane % CPR) ^ swzU<DP>(dma_r);  // invariant under the per-instruction row step (multiple of 16)
+  if (lc * 8 >= D) lc = 0;
+  const unsigned k_ss = (unsigned)a.k_ss, v_ss = (unsigned)a.v_ss;
+  const unsigned lds0 = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + wave * 1024;
+  auto issue_tile = [&](int j, int buf) {
+    const int rmax = last_k - j * BN;
+    const unsigned char* kt = kp + (uint64_t)(unsigned)(j * BN) * k_ss;
+    const unsigned char* vt = vp + (uint64_t)(unsigned)(j * BN) * v_ss;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      dma16s(kt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * k_ss + lc * 16, lds0 + buf * TILE + i * 4096);
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      dma16s(vt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * v_ss + lc * 16, lds0 + 2 * TILE + buf * TILE + i * 4096);
+  };
+  if (ntiles > 0) issue_tile(0, 0);
+
+  // ---- per-row operands: Q and dO fragments (B operands), delta, LSE ----
+  s16x8 qf[KS], dof[KS];
+  float delta = 0.f;
+  {
+    const int qr = min(row, Lq - 1);
+    const unsigned char* qrow = a.q + qb + (int64_t)(q0 + qr) * a.q_ss + (int64_t)h * a.q_sh;
+    const unsigned char* dorow = a.dout + dob + (int64_t)(q0 + qr) * a.do_ss + (int64_t)h * a.do_sh;
+    const unsigned char* orow = a.o + ob + (int64_t)(q0 + qr) * a.o_ss + (int64_t)h * a.o_sh;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int ch = 2 * ks + g;
+      u32x4 x = {0, 0, 0, 0}, y = {0, 0, 0, 0}, z = {0, 0, 0, 0};
+      if (ch * 8 < D) {
+        x = *(const u32x4*)(qrow + ch * 16);
+        y = *(const u32x4*)(dorow + ch * 16);
+        z = *(const u32x4*)(orow + ch * 16);
+      }
+      qf[ks] = __builtin_bit_cast(s16x8, x);
+      dof[ks] = __builtin_bit_cast(s16x8, y);
+      typedef T T8 __attribute__((ext_vector_type(8)));
+      const T8 dv8 = __builtin_bit_cast(T8, y), ov8 = __builtin_bit_cast(T8, z);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) delta += (float)dv8[e] * (float)ov8[e];
+    }
+    delta = pair_sum32(delta);
+  }
+  const float lse2 = (row < Lq) ? a.lse[lb + (int64_t)h * a.lse_sh + (int64_t)(q0 + row) * a.lse_ss] * kLog2e : INFINITY;
+  if (row < Lq && g == 0) a.delta[dlb + (int64_t)h * a.dl_sh + (q0 + row)] = delta;
+
+  f32x16 acc[MB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+  const float c = a.scale_log2;
+
+  int kaddr[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) kaddr[ks] = c32 * ROWB + (((2 * ks + g) ^ swzU<DP>(c32)) * 16);
+  const int L = lane & 15, G = lane >> 4;
+  const int t_row = 4 * g + (L >> 2);
+  int taddr[2][MB];  // transposed-fragment addresses, [half][mb]: rows t_row (+8)
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      taddr[hf][mb] = (t_row + 8 * hf) * ROWB + (L & 1) * 8 +
+                      (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzU<DP>(t_row + 8 * hf)) * 16);
+  const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
+
+  for (int j = 0; j < ntiles; ++j) {
+    const int buf = j & 1;
+    WAIT_VMCNT(0);
+    __syncthreads();
+    if (j + 1 < ntiles) issue_tile(j + 1, buf ^ 1);
+    if (a.is_causal && j * BN > wave_row_hi + off) continue;  // fully masked for this wavefront
+
+    const unsigned char* kt = smem + buf * TILE;
+    const unsigned char* vt = smem + 2 * TILE + buf * TILE;
+    f32x16 s0, s1, p0, p1;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; p0[v] = 0.f; p1[v] = 0.f; }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const s16x8 k0f = *(const s16x8*)(kt + kaddr[ks]);
+      const s16x8 k1f = *(const s16x8*)(kt + kaddr[ks] + 32 * ROWB);
+      const s16x8 v0f = *(const s16x8*)(vt + kaddr[ks]);
+      const s16x8 v1f = *(const s16x8*)(vt + kaddr[ks] + 32 * ROWB);
+      s0 = Mma<T>::m32(k0f, qf[ks], s0);
+      s1 = Mma<T>::m32(k1f, qf[ks], s1);
+      p0 = Mma<T>::m32(v0f, dof[ks], p0);
+      p1 = Mma<T>::m32(v1f, dof[ks], p1);
+    }
+    // P^T = exp2(S^T c - LSE), dS^T = P^T (dP^T - delta); masked positions contribute nothing
+    const bool need_mask = (j * BN + BN > Lk) || (a.is_causal && j * BN + BN - 1 > wave_row_lo + off);
+    const int lim = need_mask ? min(last_k, causal_row_lim) - j * BN - 4 * g : 0x7fffffff;
+    s16x8 dsb[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      u32x4 w;
+#pragma unroll
+      for (int e2 = 0; e2 < 4; ++e2) {
+        float ds[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int v = 8 * (t & 1) + 2 * e2 + u;
+          const int e = 32 * (t >> 1) + 8 * (v >> 2) + (v & 3);
+          const float sv = (t < 2) ? s0[v] : s1[v], dpv = (t < 2) ? p0[v] : p1[v];
+          const float p = (e <= lim) ? fast_exp2(sv * c - lse2) : 0.f;
+          ds[u] = p * (dpv - delta);
+        }
+        w[e2] = Mma<T>::pack2(ds[0], ds[1]);
+      }
+      dsb[t] = __builtin_bit_cast(s16x8, w);
+    }
+    // dQ^T += K^T dS^T
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const s16x4 lo = lds_read_tr(kt + taddr[0][mb] + (16 * t) * ROWB);
+        const s16x4 hi = lds_read_tr(kt + taddr[1][mb] + (16 * t) * ROWB);
+        const s16x8 av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        acc[mb] = Mma<T>::m32(av, dsb[t], acc[mb]);
+      }
+  }
+
+  if (row < Lq) {
+    unsigned char* orow = a.dq + dqb + (int64_t)(q0 + row) * a.dq_ss + (int64_t)h * a.dq_sh;
+    const float sc = a.scale;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const int d = 32 * mb + 8 * v4 + 4 * g;
+        if (d < D) {
+          u32x2 w;
+          w[0] = Mma<T>::pack2(acc[mb][4 * v4 + 0] * sc, acc[mb][4 * v4 + 1] * sc);
+          w[1] = Mma<T>::pack2(acc[mb][4 * v4 + 2] * sc, acc[mb][4 * v4 + 3] * sc);
+          *(u32x2*)(orow + d * 2) = w;
+        }
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// dK / dV kernel
+// ---------------------------------------------------------------------------------------------------------
+template <typename T, int DP>
+__global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
+  using IO = TileIO<T, DP>;
+  constexpr int CPR = IO::CPR, ROWB = IO::ROWB, TILE = IO::TILE, NI = IO::NI, RPI = IO::RPI, KS = IO::KS, MB = IO::MB;
+  constexpr int BKV = 128, BQ = 64;
+  constexpr int VEC = 4 * TILE;  // Q0 Q1 dO0 dO1 | lse[2][64] delta[2][64]
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 5, c32 = lane & 31;
+
+  const int lid = blockIdx.x;
+  const int ni = lid % a.n_kblk;
+  const int bhk = lid / a.n_kblk;
+  const int hk = bhk % a.heads_k, b = bhk / a.heads_k;
+
+  int q0 = 0, k0 = 0, Lq = a.seqlen_q, Lk = a.seqlen_k;
+  int64_t qb = (int64_t)b * a.q_sb, kb = (int64_t)b * a.k_sb, vb = (int64_t)b * a.v_sb, dob = (int64_t)b * a.do_sb;
+  int64_t dkb = (int64_t)b * a.dk_sb, dvb = (int64_t)b * a.dv_sb;
+  int64_t lb = (int64_t)b * a.lse_sb, dlb = (int64_t)b * a.dl_sb;
+  if (a.cu_q) {
+    q0 = a.cu_q[b];
+    Lq = a.cu_q[b + 1] - q0;
+    k0 = a.cu_k[b];
+    Lk = a.cu_k[b + 1] - k0;
+    qb = kb = vb = dob = dkb = dvb = 0;
+    lb = dlb = 0;
+  }
+  const int n0 = ni * BKV;
+  if (n0 >= Lk) return;
+  const int off = Lk - Lq;
+  const int D = a.head_dim;
+  const int kvrow = n0 + 32 * wave + c32;            // this lane's key row
+  const int wave_kv_lo = n0 + 32 * wave;
+  // query tiles that can see this key block: rows q with q + off >= n0
+  int jq_begin = 0;
+  if (a.is_causal) jq_begin = max(0, n0 - off) / BQ;
+  const int jq_end = (Lq + BQ - 1) / BQ;
+  const int nq = max(0, jq_end - jq_begin);
+  const int niter = nq * a.group;  // flattened (query head of the group, query tile)
+
+  // ---- K and V fragments of my key row (B operands) ----
+  s16x8 kf[KS], vf[KS];
+  {
+    const int kr = min(kvrow, Lk - 1);
+    const unsigned char* krow = a.k + kb + (int64_t)(k0 + kr) * a.k_ss + (int64_t)hk * a.k_sh;
+    const unsigned char* vrow = a.v + vb + (int64_t)(k0 + kr) * a.v_ss + (int64_t)hk * a.v_sh;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int ch = 2 * ks + g;
+      u32x4 x = {0, 0, 0, 0}, y = {0, 0, 0, 0};
+      if (ch * 8 < D) {
+        x = *(const u32x4*)(krow + ch * 16);
+        y = *(const u32x4*)(vrow + ch * 16);
+      }
+      kf[ks] = __builtin_bit_cast(s16x8, x);
+      vf[ks] = __builtin_bit_cast(s16x8, y);
+    }
+  }
+
+  // ---- DMA of a (query head, query tile): Q rows, dO rows, LSE and delta of the 64 rows ----
+  const int dma_r = wave * RPI + lane / CPR;
+  int lc = (lane % CPR) ^ swzU<DP>(dma_r);
+  if (lc * 8 >= D) lc = 0;
+  const unsigned q_ss = (unsigned)a.q_ss, do_ss = (unsigned)a.do_ss;
+  const unsigned lds0 = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + wave * 1024;
+  const unsigned ldsv = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + VEC;
+  auto issue_iter = [&](int it, int buf) {
+    const int hq = hk * a.group + it / nq;
+    const int jq = jq_begin + it % nq;
+    const int rmax = Lq - 1 - jq * BQ;
+    const unsigned char* qt = a.q + qb + (int64_t)(q0 + jq * BQ) * a.q_ss + (int64_t)hq * a.q_sh;
+    const unsigned char* dt = a.dout + dob + (int64_t)(q0 + jq * BQ) * a.do_ss + (int64_t)hq * a.do_sh;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      dma16s(qt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * q_ss + lc * 16, lds0 + buf * TILE + i * 4096);
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      dma16s(dt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * do_ss + lc * 16, lds0 + 2 * TILE + buf * TILE + i * 4096);
+    if (wave < 2) {  // wavefront 0: LSE of the 64 rows, wavefront 1: delta (4 bytes per lane)
+      const int r = min(lane, rmax);
+      const float* src = (wave == 0)
+                             ? a.lse + lb + (int64_t)hq * a.lse_sh + (int64_t)(q0 + jq * BQ + r) * a.lse_ss
+                             : a.delta + dlb + (int64_t)hq * a.dl_sh + (q0 + jq * BQ + r);
+      const unsigned dst = ldsv + (wave * 2 + buf) * 256;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(dst), "v"(src) : "m0");
+    }
+  };
+  if (niter > 0) issue_iter(0, 0);
+
+  f32x16 dk[MB], dv[MB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { dk[i][v] = 0.f; dv[i][v] = 0.f; }
+  const float c = a.scale_log2;
+
+  int kaddr[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) kaddr[ks] = c32 * ROWB + (((2 * ks + g) ^ swzU<DP>(c32)) * 16);
+  const int L = lane & 15, G = lane >> 4;
+  const int t_row = 4 * g + (L >> 2);
+  int taddr[2][MB];
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      taddr[hf][mb] = (t_row + 8 * hf) * ROWB + (L & 1) * 8 +
+                      (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzU<DP>(t_row + 8 * hf)) * 16);
+
+  for (int it = 0; it < niter; ++it) {
+    const int buf = it & 1;
+    WAIT_VMCNT(0);
+    __syncthreads();
+    if (it + 1 < niter) issue_iter(it + 1, buf ^ 1);
+    const int jq = jq_begin + it % nq;
+    const int qlo = jq * BQ;
+    // every (q, kv) of this tile masked for this wavefront: q + off < kv for all pairs
+    if (a.is_causal && qlo + BQ - 1 + off < wave_kv_lo) continue;
+
+    const unsigned char* qt = smem + buf * TILE;
+    const unsigned char* dt = smem + 2 * TILE + buf * TILE;
+    const float* lse_t = (const float*)(smem + VEC + (0 * 2 + buf) * 256);
+    const float* del_t = (const float*)(smem + VEC + (1 * 2 + buf) * 256);
+    const bool need_mask = (qlo + BQ > Lq) || (a.is_causal && qlo + off < wave_kv_lo + 31) || (wave_kv_lo + 32 > Lk);
+
+#pragma unroll
+    for (int qbk = 0; qbk < 2; ++qbk) {  // two blocks of 32 query rows
+      f32x16 s, dp;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const s16x8 qa = *(const s16x8*)(qt + kaddr[ks] + qbk * 32 * ROWB);
+        const s16x8 da = *(const s16x8*)(dt + kaddr[ks] + qbk * 32 * ROWB);
+        s = Mma<T>::m32(qa, kf[ks], s);
+        dp = Mma<T>::m32(da, vf[ks], dp);
+      }
+      // register v of this lane <-> query row qlo + 32 qbk + 8 (v >> 2) + 4 g + (v & 3), key row kvrow
+      s16x8 pb[2], dsb[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        u32x4 wp, wd;
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          const int v = 8 * t + 2 * e2;          // v, v + 1: consecutive query rows
+          const int ql = 32 * qbk + 8 * (v >> 2) + 4 * g + (v & 3);
+          const float l0 = lse_t[ql] * kLog2e, l1 = lse_t[ql + 1] * kLog2e;
+          const float d0 = del_t[ql], d1 = del_t[ql + 1];
+          float p0 = fast_exp2(s[v] * c - l0), p1 = fast_exp2(s[v + 1] * c - l1);
+          if (need_mask) {
+            const int qa0 = qlo + ql;
+            const bool ok0 = (qa0 < Lq) && (kvrow < Lk) && (!a.is_causal || kvrow <= qa0 + off);
+            const bool ok1 = (qa0 + 1 < Lq) && (kvrow < Lk) && (!a.is_causal || kvrow <= qa0 + 1 + off);
+            p0 = ok0 ? p0 : 0.f;
+            p1 = ok1 ? p1 : 0.f;
+          }
+          wp[e2] = Mma<T>::pack2(p0, p1);
+          wd[e2] = Mma<T>::pack2(p0 * (dp[v] - d0), p1 * (dp[v + 1] - d1));
+        }
+        pb[t] = __builtin_bit_cast(s16x8, wp);
+        dsb[t] = __builtin_bit_cast(s16x8, wd);
+      }
+      // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 32 query rows of this block: chunks 2 qbk, 2 qbk + 1)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          const int ro = (32 * qbk + 16 * t) * ROWB;
+          const s16x4 dlo = lds_read_tr(dt + taddr[0][mb] + ro);
+          const s16x4 dhi = lds_read_tr(dt + taddr[1][mb] + ro);
+          const s16x8 dav = {dlo[0], dlo[1], dlo[2], dlo[3], dhi[0], dhi[1], dhi[2], dhi[3]};
+          dv[mb] = Mma<T>::m32(dav, pb[t], dv[mb]);
+          const s16x4 qlo4 = lds_read_tr(qt + taddr[0][mb] + ro);
+          const s16x4 qhi4 = lds_read_tr(qt + taddr[1][mb] + ro);
+          const s16x8 qav = {qlo4[0], qlo4[1], qlo4[2], qlo4[3], qhi4[0], qhi4[1], qhi4[2], qhi4[3]};
+          dk[mb] = Mma<T>::m32(qav, dsb[t], dk[mb]);
+        }
+    }
+  }
+
+  if (kvrow < Lk) {
+    unsigned char* krow = a.dk + dkb + (int64_t)(k0 + kvrow) * a.dk_ss + (int64_t)hk * a.dk_sh;
+    unsigned char* vrow = a.dv + dvb + (int64_t)(k0 + kvrow) * a.dv_ss + (int64_t)hk * a.dv_sh;
+    const float sc = a.scale;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const int d = 32 * mb + 8 * v4 + 4 * g;
+        if (d < D) {
+          u32x2 w;
+          w[0] = Mma<T>::pack2(dk[mb][4 * v4 + 0] * sc, dk[mb][4 * v4 + 1] * sc);
+          w[1] = Mma<T>::pack2(dk[mb][4 * v4 + 2] * sc, dk[mb][4 * v4 + 3] * sc);
+          *(u32x2*)(krow + d * 2) = w;
+          w[0] = Mma<T>::pack2(dv[mb][4 * v4 + 0], dv[mb][4 * v4 + 1]);
+          w[1] = Mma<T>::pack2(dv[mb][4 * v4 + 2], dv[mb][4 * v4 + 3]);
+          *(u32x2*)(vrow + d * 2) = w;
+        }
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------------------------
+int bwd_validate(const fa_bwd_params* p) {
+  if (!p) return FA_ERR_BAD_ARG;
+  if (!p->q || !p->k || !p->v || !p->out || !p->dout || !p->lse || !p->dq || !p->dk || !p->dv) return FA_ERR_BAD_ARG;
+  if ((p->cu_seqlens_q == nullptr) != (p->cu_seqlens_k == nullptr)) return FA_ERR_BAD_ARG;
+  if (p->batch <= 0 || p->heads_q <= 0 || p->heads_k <= 0) return FA_ERR_BAD_ARG;
+  if (p->seqlen_q < 0 || p->seqlen_k < 0 || p->head_dim <= 0) return FA_ERR_BAD_ARG;
+  if (p->reserved != 0) return FA_ERR_BAD_ARG;
+  if (p->cu_seqlens_q && p->total_q < 0) return FA_ERR_BAD_ARG;
+  if (p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_UNSUPPORTED;
+  if (p->head_dim > 128 || (p->head_dim & 7)) return FA_ERR_UNSUPPORTED;
+  if (p->heads_q % p->heads_k) return FA_ERR_UNSUPPORTED;
+  const uintptr_t al = (uintptr_t)p->q | (uintptr_t)p->k | (uintptr_t)p->v | (uintptr_t)p->out | (uintptr_t)p->dout |
+                       (uintptr_t)p->dq | (uintptr_t)p->dk | (uintptr_t)p->dv;
+  if (al & 15) return FA_ERR_BAD_ARG;
+  if ((uintptr_t)p->lse & 3) return FA_ERR_BAD_ARG;
+  const int64_t st[] = {p->q_stride_s,  p->q_stride_h,  p->k_stride_s,  p->k_stride_h,  p->v_stride_s,  p->v_stride_h,
+                        p->o_stride_s,  p->o_stride_h,  p->do_stride_s, p->do_stride_h, p->dq_stride_s, p->dq_stride_h,
+                        p->dk_stride_s, p->dk_stride_h, p->dv_stride_s, p->dv_stride_h};
+  for (int64_t s : st)
+    if (s < 0 || (s & 7)) return FA_ERR_BAD_ARG;
+  if (!p->cu_seqlens_q) {
+    const int64_t sb[] = {p->q_stride_b,  p->k_stride_b,  p->v_stride_b,  p->o_stride_b,
+                          p->do_stride_b, p->dq_stride_b, p->dk_stride_b, p->dv_stride_b};
+    for (int64_t s : sb)
+      if (s < 0 || (s & 7)) return FA_ERR_BAD_ARG;
+  }
+  if (p->lse_stride_h < 0 || p->lse_stride_s < 0) return FA_ERR_BAD_ARG;
+  if (p->k_stride_s * 2 > 0x7fffffffLL || p->v_stride_s * 2 > 0x7fffffffLL || p->q_stride_s * 2 > 0x7fffffffLL ||
+      p->do_stride_s * 2 > 0x7fffffffLL)
+    return FA_ERR_UNSUPPORTED;
+  return FA_OK;
+}
+
+size_t bwd_ws_bytes(const fa_bwd_params* p) {
+  const size_t rows = p->cu_seqlens_q ? (size_t)p->total_q : (size_t)p->batch * p->seqlen_q;
+  return (rows * p->heads_q * 4 + 15) & ~(size_t)15;
+}
+
+template <typename T, int DP>
+int bwd_launch(const BArgs& a, hipStream_t st) {
+  constexpr int lds_dq = 4 * 64 * DP * 2;
+  constexpr int lds_dkv = 4 * 64 * DP * 2 + 4 * 256;
+  auto kq = fa_bwd_dq_kernel<T, DP>;
+  auto kkv = fa_bwd_dkv_kernel<T, DP>;
+  if (hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dq) != hipSuccess ||
+      hipFuncSetAttribute((const void*)kkv, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv) != hipSuccess) {
+    (void)hipGetLastError();
+    return FA_ERR_LAUNCH;
+  }
+  const int64_t gq = (int64_t)a.batch * a.heads_q * a.n_qblk;
+  const int64_t gk = (int64_t)a.batch * a.heads_k * a.n_kblk;
+  if (gq > 0x7fffffffLL || gk > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
+  if (gq > 0) {
+    hipLaunchKernelGGL(kq, dim3((unsigned)gq), dim3(256), lds_dq, st, a);
+    if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
+  }
+  if (gk > 0) {
+    hipLaunchKernelGGL(kkv, dim3((unsigned)gk), dim3(256), lds_dkv, st, a);
+    if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
+  }
+  return FA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fa_bwd_validate(const fa_bwd_params* p) { return bwd_validate(p); }
+
+size_t fa_bwd_workspace_bytes(const fa_bwd_params* p) {
+  if (bwd_validate(p) != FA_OK) return 0;
+  return bwd_ws_bytes(p);
+}
+
+int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = bwd_validate(p);
+  if (rc != FA_OK) return rc;
+  const size_t need = bwd_ws_bytes(p);
+  if (need > 0 && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15))) return FA_ERR_BAD_ARG;
+  BArgs a;
+  a.q = (const unsigned char*)p->q; a.k = (const unsigned char*)p->k; a.v = (const unsigned char*)p->v;
+  a.o = (const unsigned char*)p->out; a.dout = (const unsigned char*)p->dout; a.lse = p->lse;
+  a.dq = (unsigned char*)p->dq; a.dk = (unsigned char*)p->dk; a.dv = (unsigned char*)p->dv;
+  a.delta = (float*)workspace;
+  a.cu_q = p->cu_seqlens_q; a.cu_k = p->cu_seqlens_k;
+  a.q_sb = p->q_stride_b * 2; a.q_ss = p->q_stride_s * 2; a.q_sh = p->q_stride_h * 2;
+  a.k_sb = p->k_stride_b * 2; a.k_ss = p->k_stride_s * 2; a.k_sh = p->k_stride_h * 2;
+  a.v_sb = p->v_stride_b * 2; a.v_ss = p->v_stride_s * 2; a.v_sh = p->v_stride_h * 2;
+  a.o_sb = p->o_stride_b * 2; a.o_ss = p->o_stride_s * 2; a.o_sh = p->o_stride_h * 2;
+  a.do_sb = p->do_stride_b * 2; a.do_ss = p->do_stride_s * 2; a.do_sh = p->do_stride_h * 2;
+  a.dq_sb = p->dq_stride_b * 2; a.dq_ss = p->dq_stride_s * 2; a.dq_sh = p->dq_stride_h * 2;
+  a.dk_sb = p->dk_stride_b * 2; a.dk_ss = p->dk_stride_s * 2; a.dk_sh = p->dk_stride_h * 2;
+  a.dv_sb = p->dv_stride_b * 2; a.dv_ss = p->dv_stride_s * 2; a.dv_sh = p->dv_stride_h * 2;
+  a.lse_sb = p->lse_stride_b; a.lse_sh = p->lse_stride_h; a.lse_ss = p->lse_stride_s;
+  if (p->cu_seqlens_q) {
+    a.dl_sb = 0; a.dl_sh = p->total_q;
+  } else {
+    a.dl_sb = (int64_t)p->heads_q * p->seqlen_q; a.dl_sh = p->seqlen_q;
+  }
+  a.batch = p->batch; a.heads_q = p->heads_q; a.heads_k = p->heads_k; a.group = p->heads_q / p->heads_k;
+  a.seqlen_q = p->seqlen_q; a.seqlen_k = p->seqlen_k; a.head_dim = p->head_dim;
+  a.n_qblk = (p->seqlen_q + 127) / 128;
+  a.n_kblk = (p->seqlen_k + 127) / 128;
+  a.is_causal = p->is_causal ? 1 : 0;
+  a.scale = p->scale;
+  a.scale_log2 = p->scale * kLog2e;
+  hipStream_t st = (hipStream_t)stream;
+  const int dp = p->head_dim <= 64 ? 64 : 128;
+  if (p->dtype == FA_DTYPE_BF16) return dp == 64 ? bwd_launch<__bf16, 64>(a, st) : bwd_launch<__bf16, 128>(a, st);
+  return dp == 64 ? bwd_launch<_Float16, 64>(a, st) : bwd_launch<_Float16, 128>(a, st);
+}
+
+}  // extern "C"
