@@ -51,7 +51,7 @@ struct BArgs {
   int64_t dl_sb, dl_sh;            // delta strides (elements); row stride is 1
   int32_t batch, heads_q, heads_k, group;
   int32_t seqlen_q, seqlen_k, head_dim;
-  int32_t n_qblk, n_kblk;
+  int32_t n_qslot, n_kslot;  // workgroups per (sequence, head) of the dQ kernel / per (sequence, kv head) of the dK/dV kernel
   int32_t is_causal;
   float scale;       // signed softmax scale
   float scale_log2;  // scale * log2(e), signed
@@ -80,7 +80,7 @@ struct TileIO {
 // dQ kernel
 // ---------------------------------------------------------------------------------------------------------
 template <typename T, int DP>
-__global__ void __launch_bounds__(256, 1) fa_bwd_dq_kernel(const BArgs a) {
+__global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
   using IO = TileIO<T, DP>;
   constexpr int CPR = IO::CPR, ROWB = IO::ROWB, TILE = IO::TILE, NI = IO::NI, RPI = IO::RPI, KS = IO::KS, MB = IO::MB;
   constexpr int BM = 128, BN = 64;
@@ -91,9 +91,21 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dq_kernel(const BArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5, c32 = lane & 31;
 
-  const int lid = blockIdx.x;
-  const int mi = a.n_qblk - 1 - (lid % a.n_qblk);
-  const int bh = lid / a.n_qblk;
+  // Workgroups are dealt round-robin to the 8 XCDs and dispatched in order: dense problems give each XCD a contiguous
+  // range of logical ids (all query blocks of a head share one L2, and no XCD gets only the heavy blocks); packed
+  // problems go block-major, heaviest block index first, and sequences shorter than that exit at once.
+  int lid = blockIdx.x;
+  int pslot, bh;
+  if (a.cu_q) {
+    const int nbh = a.batch * a.heads_q;
+    pslot = lid / nbh;
+    bh = lid % nbh;
+  } else {
+    const int per = gridDim.x >> 3;
+    if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
+    pslot = lid % a.n_qslot;
+    bh = lid / a.n_qslot;
+  }
   const int h = bh % a.heads_q, b = bh / a.heads_q;
   const int hk = h / a.group;
 
@@ -109,16 +121,12 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dq_kernel(const BArgs a) {
     qb = kb = vb = ob = dob = dqb = 0;
     lb = dlb = 0;
   }
-  const int m0 = mi * BM;
-  if (m0 >= Lq) return;
+  // heaviest (last) query block first; packed: counted down from the longest possible sequence
+  const int nblk = (Lq + BM - 1) / BM;
+  const int blk_first = (a.cu_q ? a.n_qslot : nblk) - 1 - pslot;
+  if (blk_first < 0 || blk_first >= nblk) return;
   const int off = Lk - Lq;
-  int n_end = Lk;
-  if (a.is_causal) n_end = min(Lk, m0 + BM + off);
-  if (n_end < 0) n_end = 0;
-  const int ntiles = (n_end + BN - 1) / BN;
   const int D = a.head_dim;
-  const int row = m0 + 32 * wave + c32;
-  const int wave_row_lo = m0 + 32 * wave, wave_row_hi = wave_row_lo + 31;
   const int last_k = Lk - 1;
 
   const unsigned char* kp = a.k + kb + (int64_t)k0 * a.k_ss + (int64_t)hk * a.k_sh;
@@ -141,6 +149,28 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dq_kernel(const BArgs a) {
     for (int i = 0; i < NI; ++i)
       dma16s(vt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * v_ss + lc * 16, lds0 + 2 * TILE + buf * TILE + i * 4096);
   };
+
+  const float c = a.scale_log2;
+  int kaddr[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) kaddr[ks] = c32 * ROWB + (((2 * ks + g) ^ swzU<DP>(c32)) * 16);
+  const int L = lane & 15, G = lane >> 4;
+  const int t_row = 4 * g + (L >> 2);
+  int taddr[2][MB];  // transposed-fragment addresses, [half][mb]: rows t_row (+8)
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      taddr[hf][mb] = (t_row + 8 * hf) * ROWB + (L & 1) * 8 +
+                      (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzU<DP>(t_row + 8 * hf)) * 16);
+
+  const int m0 = blk_first * BM;
+  int n_end = Lk;
+  if (a.is_causal) n_end = min(Lk, m0 + BM + off);
+  if (n_end < 0) n_end = 0;
+  const int ntiles = (n_end + BN - 1) / BN;
+  const int row = m0 + 32 * wave + c32;
+  const int wave_row_lo = m0 + 32 * wave, wave_row_hi = wave_row_lo + 31;
   if (ntiles > 0) issue_tile(0, 0);
 
   // ---- per-row operands: Q and dO fragments (B operands), delta, LSE ----
@@ -169,7 +199,8 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dq_kernel(const BArgs a) {
     }
     delta = pair_sum32(delta);
   }
-  const float lse2 = (row < Lq) ? a.lse[lb + (int64_t)h * a.lse_sh + (int64_t)(q0 + row) * a.lse_ss] * kLog2e : INFINITY;
+  const float lse2 =
+      (row < Lq) ? a.lse[lb + (int64_t)h * a.lse_sh + (int64_t)(q0 + row) * a.lse_ss] * kLog2e : INFINITY;
   if (row < Lq && g == 0) a.delta[dlb + (int64_t)h * a.dl_sh + (q0 + row)] = delta;
 
   f32x16 acc[MB];
@@ -177,20 +208,6 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dq_kernel(const BArgs a) {
   for (int i = 0; i < MB; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
-  const float c = a.scale_log2;
-
-  int kaddr[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) kaddr[ks] = c32 * ROWB + (((2 * ks + g) ^ swzU<DP>(c32)) * 16);
-  const int L = lane & 15, G = lane >> 4;
-  const int t_row = 4 * g + (L >> 2);
-  int taddr[2][MB];  // transposed-fragment addresses, [half][mb]: rows t_row (+8)
-#pragma unroll
-  for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-      taddr[hf][mb] = (t_row + 8 * hf) * ROWB + (L & 1) * 8 +
-                      (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzU<DP>(t_row + 8 * hf)) * 16);
   const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
 
   for (int j = 0; j < ntiles; ++j) {
@@ -284,9 +301,20 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5, c32 = lane & 31;
 
-  const int lid = blockIdx.x;
-  const int ni = lid % a.n_kblk;
-  const int bhk = lid / a.n_kblk;
+  // Same dispatch-order reasoning as the dQ kernel.  Causal: the first key blocks are the heavy ones (every query
+  // row sees them) and they come first.
+  int lid = blockIdx.x;
+  int pslot, bhk;
+  if (a.cu_q) {
+    const int nbh = a.batch * a.heads_k;
+    pslot = lid / nbh;
+    bhk = lid % nbh;
+  } else {
+    const int per = gridDim.x >> 3;
+    if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
+    pslot = lid % a.n_kslot;
+    bhk = lid / a.n_kslot;
+  }
   const int hk = bhk % a.heads_k, b = bhk / a.heads_k;
 
   int q0 = 0, k0 = 0, Lq = a.seqlen_q, Lk = a.seqlen_k;
@@ -301,11 +329,33 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
     qb = kb = vb = dob = dkb = dvb = 0;
     lb = dlb = 0;
   }
-  const int n0 = ni * BKV;
-  if (n0 >= Lk) return;
+  if (pslot * BKV >= Lk) return;
   const int off = Lk - Lq;
   const int D = a.head_dim;
-  const int kvrow = n0 + 32 * wave + c32;            // this lane's key row
+
+  const int dma_r = wave * RPI + lane / CPR;
+  int lc = (lane % CPR) ^ swzU<DP>(dma_r);
+  if (lc * 8 >= D) lc = 0;
+  const unsigned q_ss = (unsigned)a.q_ss, do_ss = (unsigned)a.do_ss;
+  const unsigned lds0 = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + wave * 1024;
+  const unsigned ldsv = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + VEC;
+  const float c = a.scale_log2;
+
+  int kaddr[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) kaddr[ks] = c32 * ROWB + (((2 * ks + g) ^ swzU<DP>(c32)) * 16);
+  const int L = lane & 15, G = lane >> 4;
+  const int t_row = 4 * g + (L >> 2);
+  int taddr[2][MB];
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      taddr[hf][mb] = (t_row + 8 * hf) * ROWB + (L & 1) * 8 +
+                      (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzU<DP>(t_row + 8 * hf)) * 16);
+
+  const int n0 = pslot * BKV;
+  const int kvrow = n0 + 32 * wave + c32;  // this lane's key row
   const int wave_kv_lo = n0 + 32 * wave;
   // query tiles that can see this key block: rows q with q + off >= n0
   int jq_begin = 0;
@@ -334,12 +384,6 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
   }
 
   // ---- DMA of a (query head, query tile): Q rows, dO rows, LSE and delta of the 64 rows ----
-  const int dma_r = wave * RPI + lane / CPR;
-  int lc = (lane % CPR) ^ swzU<DP>(dma_r);
-  if (lc * 8 >= D) lc = 0;
-  const unsigned q_ss = (unsigned)a.q_ss, do_ss = (unsigned)a.do_ss;
-  const unsigned lds0 = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + wave * 1024;
-  const unsigned ldsv = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + VEC;
   auto issue_iter = [&](int it, int buf) {
     const int hq = hk * a.group + it / nq;
     const int jq = jq_begin + it % nq;
@@ -351,7 +395,8 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
       dma16s(qt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * q_ss + lc * 16, lds0 + buf * TILE + i * 4096);
 #pragma unroll
     for (int i = 0; i < NI; ++i)
-      dma16s(dt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * do_ss + lc * 16, lds0 + 2 * TILE + buf * TILE + i * 4096);
+      dma16s(dt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * do_ss + lc * 16,
+             lds0 + 2 * TILE + buf * TILE + i * 4096);
     if (wave < 2) {  // wavefront 0: LSE of the 64 rows, wavefront 1: delta (4 bytes per lane)
       const int r = min(lane, rmax);
       const float* src = (wave == 0)
@@ -368,20 +413,6 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
   for (int i = 0; i < MB; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) { dk[i][v] = 0.f; dv[i][v] = 0.f; }
-  const float c = a.scale_log2;
-
-  int kaddr[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) kaddr[ks] = c32 * ROWB + (((2 * ks + g) ^ swzU<DP>(c32)) * 16);
-  const int L = lane & 15, G = lane >> 4;
-  const int t_row = 4 * g + (L >> 2);
-  int taddr[2][MB];
-#pragma unroll
-  for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-      taddr[hf][mb] = (t_row + 8 * hf) * ROWB + (L & 1) * 8 +
-                      (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzU<DP>(t_row + 8 * hf)) * 16);
 
   for (int it = 0; it < niter; ++it) {
     const int buf = it & 1;
@@ -397,7 +428,8 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
     const unsigned char* dt = smem + 2 * TILE + buf * TILE;
     const float* lse_t = (const float*)(smem + VEC + (0 * 2 + buf) * 256);
     const float* del_t = (const float*)(smem + VEC + (1 * 2 + buf) * 256);
-    const bool need_mask = (qlo + BQ > Lq) || (a.is_causal && qlo + off < wave_kv_lo + 31) || (wave_kv_lo + 32 > Lk);
+    const bool need_mask =
+        (qlo + BQ > Lq) || (a.is_causal && qlo + off < wave_kv_lo + 31) || (wave_kv_lo + 32 > Lk);
 
 #pragma unroll
     for (int qbk = 0; qbk < 2; ++qbk) {  // two blocks of 32 query rows
@@ -418,7 +450,7 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
         u32x4 wp, wd;
 #pragma unroll
         for (int e2 = 0; e2 < 4; ++e2) {
-          const int v = 8 * t + 2 * e2;          // v, v + 1: consecutive query rows
+          const int v = 8 * t + 2 * e2;  // v, v + 1: consecutive query rows
           const int ql = 32 * qbk + 8 * (v >> 2) + 4 * g + (v & 3);
           const float l0 = lse_t[ql] * kLog2e, l1 = lse_t[ql + 1] * kLog2e;
           const float d0 = del_t[ql], d1 = del_t[ql + 1];
@@ -436,7 +468,7 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
         pb[t] = __builtin_bit_cast(s16x8, wp);
         dsb[t] = __builtin_bit_cast(s16x8, wd);
       }
-      // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 32 query rows of this block: chunks 2 qbk, 2 qbk + 1)
+      // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 32 query rows of this block)
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -528,8 +560,8 @@ int bwd_launch(const BArgs& a, hipStream_t st) {
     (void)hipGetLastError();
     return FA_ERR_LAUNCH;
   }
-  const int64_t gq = (int64_t)a.batch * a.heads_q * a.n_qblk;
-  const int64_t gk = (int64_t)a.batch * a.heads_k * a.n_kblk;
+  const int64_t gq = (int64_t)a.batch * a.heads_q * a.n_qslot;
+  const int64_t gk = (int64_t)a.batch * a.heads_k * a.n_kslot;
   if (gq > 0x7fffffffLL || gk > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
   if (gq > 0) {
     hipLaunchKernelGGL(kq, dim3((unsigned)gq), dim3(256), lds_dq, st, a);
@@ -580,9 +612,9 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   }
   a.batch = p->batch; a.heads_q = p->heads_q; a.heads_k = p->heads_k; a.group = p->heads_q / p->heads_k;
   a.seqlen_q = p->seqlen_q; a.seqlen_k = p->seqlen_k; a.head_dim = p->head_dim;
-  a.n_qblk = (p->seqlen_q + 127) / 128;
-  a.n_kblk = (p->seqlen_k + 127) / 128;
   a.is_causal = p->is_causal ? 1 : 0;
+  a.n_qslot = (p->seqlen_q + 127) / 128;
+  a.n_kslot = (p->seqlen_k + 127) / 128;
   a.scale = p->scale;
   a.scale_log2 = p->scale * kLog2e;
   hipStream_t st = (hipStream_t)stream;
