@@ -288,8 +288,14 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
 // ---------------------------------------------------------------------------------------------------------
 // dK / dV kernel
 // ---------------------------------------------------------------------------------------------------------
-template <typename T, int DP>
-__global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
+// WHAT selects the outputs: kDK (S, dP, dS, dK), kDV (S, P, dV) or both.  With head_dim 128 both accumulators do not
+// fit the 256 registers that two wavefronts per SIMD leave, so dK and dV run as two launches (S is recomputed once
+// more); with head_dim <= 64 one launch produces both.
+constexpr int kDK = 1, kDV = 2;
+
+template <typename T, int DP, int WHAT>
+__global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
+  constexpr bool DO_K = (WHAT & kDK) != 0, DO_V = (WHAT & kDV) != 0;
   using IO = TileIO<T, DP>;
   constexpr int CPR = IO::CPR, ROWB = IO::ROWB, TILE = IO::TILE, NI = IO::NI, RPI = IO::RPI, KS = IO::KS, MB = IO::MB;
   constexpr int BKV = 128, BQ = 64;
@@ -376,7 +382,7 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
       u32x4 x = {0, 0, 0, 0}, y = {0, 0, 0, 0};
       if (ch * 8 < D) {
         x = *(const u32x4*)(krow + ch * 16);
-        y = *(const u32x4*)(vrow + ch * 16);
+        if constexpr (DO_K) y = *(const u32x4*)(vrow + ch * 16);
       }
       kf[ks] = __builtin_bit_cast(s16x8, x);
       vf[ks] = __builtin_bit_cast(s16x8, y);
@@ -397,7 +403,7 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
     for (int i = 0; i < NI; ++i)
       dma16s(dt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * do_ss + lc * 16,
              lds0 + 2 * TILE + buf * TILE + i * 4096);
-    if (wave < 2) {  // wavefront 0: LSE of the 64 rows, wavefront 1: delta (4 bytes per lane)
+    if (wave < (DO_K ? 2 : 1)) {  // wavefront 0: LSE of the 64 rows, wavefront 1: delta (4 bytes per lane)
       const int r = min(lane, rmax);
       const float* src = (wave == 0)
                              ? a.lse + lb + (int64_t)hq * a.lse_sh + (int64_t)(q0 + jq * BQ + r) * a.lse_ss
@@ -439,9 +445,11 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const s16x8 qa = *(const s16x8*)(qt + kaddr[ks] + qbk * 32 * ROWB);
-        const s16x8 da = *(const s16x8*)(dt + kaddr[ks] + qbk * 32 * ROWB);
         s = Mma<T>::m32(qa, kf[ks], s);
-        dp = Mma<T>::m32(da, vf[ks], dp);
+        if constexpr (DO_K) {
+          const s16x8 da = *(const s16x8*)(dt + kaddr[ks] + qbk * 32 * ROWB);
+          dp = Mma<T>::m32(da, vf[ks], dp);
+        }
       }
       // register v of this lane <-> query row qlo + 32 qbk + 8 (v >> 2) + 4 g + (v & 3), key row kvrow
       s16x8 pb[2], dsb[2];
@@ -453,7 +461,7 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
           const int v = 8 * t + 2 * e2;  // v, v + 1: consecutive query rows
           const int ql = 32 * qbk + 8 * (v >> 2) + 4 * g + (v & 3);
           const float l0 = lse_t[ql] * kLog2e, l1 = lse_t[ql + 1] * kLog2e;
-          const float d0 = del_t[ql], d1 = del_t[ql + 1];
+          const float d0 = DO_K ? del_t[ql] : 0.f, d1 = DO_K ? del_t[ql + 1] : 0.f;
           float p0 = fast_exp2(s[v] * c - l0), p1 = fast_exp2(s[v + 1] * c - l1);
           if (need_mask) {
             const int qa0 = qlo + ql;
@@ -462,8 +470,8 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
             p0 = ok0 ? p0 : 0.f;
             p1 = ok1 ? p1 : 0.f;
           }
-          wp[e2] = Mma<T>::pack2(p0, p1);
-          wd[e2] = Mma<T>::pack2(p0 * (dp[v] - d0), p1 * (dp[v + 1] - d1));
+          if constexpr (DO_V) wp[e2] = Mma<T>::pack2(p0, p1);
+          if constexpr (DO_K) wd[e2] = Mma<T>::pack2(p0 * (dp[v] - d0), p1 * (dp[v + 1] - d1));
         }
         pb[t] = __builtin_bit_cast(s16x8, wp);
         dsb[t] = __builtin_bit_cast(s16x8, wd);
@@ -474,14 +482,18 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
           const int ro = (32 * qbk + 16 * t) * ROWB;
-          const s16x4 dlo = lds_read_tr(dt + taddr[0][mb] + ro);
-          const s16x4 dhi = lds_read_tr(dt + taddr[1][mb] + ro);
-          const s16x8 dav = {dlo[0], dlo[1], dlo[2], dlo[3], dhi[0], dhi[1], dhi[2], dhi[3]};
-          dv[mb] = Mma<T>::m32(dav, pb[t], dv[mb]);
-          const s16x4 qlo4 = lds_read_tr(qt + taddr[0][mb] + ro);
-          const s16x4 qhi4 = lds_read_tr(qt + taddr[1][mb] + ro);
-          const s16x8 qav = {qlo4[0], qlo4[1], qlo4[2], qlo4[3], qhi4[0], qhi4[1], qhi4[2], qhi4[3]};
-          dk[mb] = Mma<T>::m32(qav, dsb[t], dk[mb]);
+          if constexpr (DO_V) {
+            const s16x4 dlo = lds_read_tr(dt + taddr[0][mb] + ro);
+            const s16x4 dhi = lds_read_tr(dt + taddr[1][mb] + ro);
+            const s16x8 dav = {dlo[0], dlo[1], dlo[2], dlo[3], dhi[0], dhi[1], dhi[2], dhi[3]};
+            dv[mb] = Mma<T>::m32(dav, pb[t], dv[mb]);
+          }
+          if constexpr (DO_K) {
+            const s16x4 qlo4 = lds_read_tr(qt + taddr[0][mb] + ro);
+            const s16x4 qhi4 = lds_read_tr(qt + taddr[1][mb] + ro);
+            const s16x8 qav = {qlo4[0], qlo4[1], qlo4[2], qlo4[3], qhi4[0], qhi4[1], qhi4[2], qhi4[3]};
+            dk[mb] = Mma<T>::m32(qav, dsb[t], dk[mb]);
+          }
         }
     }
   }
@@ -497,12 +509,16 @@ __global__ void __launch_bounds__(256, 1) fa_bwd_dkv_kernel(const BArgs a) {
         const int d = 32 * mb + 8 * v4 + 4 * g;
         if (d < D) {
           u32x2 w;
-          w[0] = Mma<T>::pack2(dk[mb][4 * v4 + 0] * sc, dk[mb][4 * v4 + 1] * sc);
-          w[1] = Mma<T>::pack2(dk[mb][4 * v4 + 2] * sc, dk[mb][4 * v4 + 3] * sc);
-          *(u32x2*)(krow + d * 2) = w;
-          w[0] = Mma<T>::pack2(dv[mb][4 * v4 + 0], dv[mb][4 * v4 + 1]);
-          w[1] = Mma<T>::pack2(dv[mb][4 * v4 + 2], dv[mb][4 * v4 + 3]);
-          *(u32x2*)(vrow + d * 2) = w;
+          if constexpr (DO_K) {
+            w[0] = Mma<T>::pack2(dk[mb][4 * v4 + 0] * sc, dk[mb][4 * v4 + 1] * sc);
+            w[1] = Mma<T>::pack2(dk[mb][4 * v4 + 2] * sc, dk[mb][4 * v4 + 3] * sc);
+            *(u32x2*)(krow + d * 2) = w;
+          }
+          if constexpr (DO_V) {
+            w[0] = Mma<T>::pack2(dv[mb][4 * v4 + 0], dv[mb][4 * v4 + 1]);
+            w[1] = Mma<T>::pack2(dv[mb][4 * v4 + 2], dv[mb][4 * v4 + 3]);
+            *(u32x2*)(vrow + d * 2) = w;
+          }
         }
       }
   }
@@ -553,10 +569,13 @@ template <typename T, int DP>
 int bwd_launch(const BArgs& a, hipStream_t st) {
   constexpr int lds_dq = 4 * 64 * DP * 2;
   constexpr int lds_dkv = 4 * 64 * DP * 2 + 4 * 256;
+  constexpr bool split = DP > 64;  // head_dim 128: dK and dV as two launches
   auto kq = fa_bwd_dq_kernel<T, DP>;
-  auto kkv = fa_bwd_dkv_kernel<T, DP>;
+  auto kkv = fa_bwd_dkv_kernel<T, DP, split ? kDK : (kDK | kDV)>;
+  auto kv2 = fa_bwd_dkv_kernel<T, DP, kDV>;
   if (hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dq) != hipSuccess ||
-      hipFuncSetAttribute((const void*)kkv, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv) != hipSuccess) {
+      hipFuncSetAttribute((const void*)kkv, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv) != hipSuccess ||
+      (split && hipFuncSetAttribute((const void*)kv2, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv) != hipSuccess)) {
     (void)hipGetLastError();
     return FA_ERR_LAUNCH;
   }
@@ -570,6 +589,10 @@ int bwd_launch(const BArgs& a, hipStream_t st) {
   if (gk > 0) {
     hipLaunchKernelGGL(kkv, dim3((unsigned)gk), dim3(256), lds_dkv, st, a);
     if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
+    if (split) {
+      hipLaunchKernelGGL(kv2, dim3((unsigned)gk), dim3(256), lds_dkv, st, a);
+      if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
+    }
   }
   return FA_OK;
 }
