@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the flash-attention forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd] [--no-extras] [--no-cpu-baseline]
 
 A "step" is one call of the registered op on one batch of seeded synthetic input that is already resident in HBM.
 The headline workload is BASELINE.json configs[1] (causal prefill, bf16 MHA, B=4 H=32 S=4096 D=128); the other
@@ -30,8 +30,9 @@ PEAK_HBM_GBS = 8000.0
 # their commands are recorded under profiles/.  Counters cannot be read from inside a timed run, so these are the
 # recorded values (None: not profiled).
 TRAFFIC_BYTES = {
-    "cfg2": int((521.7 + 130.0) * 2 ** 20),
-    "cfg5": int(2.0022 * 2 ** 30 + 4.25 * 2 ** 20),
+    "cfg2": int((522.1 + 130.0) * 2 ** 20),
+    "cfg5": int(2.0021 * 2 ** 30 + 4.25 * 2 ** 20),
+    "cfg2_bwd": int((1701.8 + 386.1) * 2 ** 20),  # the three launches of one backward together
 }
 
 
@@ -63,6 +64,23 @@ def make_workload(name, dev):
         return dict(call=call, check=check, flops=4 * B * Hq * S * S * D / 2, bytes_kv=2 * B * Hk * S * D * 2,
                     desc=f"causal prefill bf16 B={B} Hq={Hq} Hkv={Hk} S={S} D={D}", dtype="bf16", bound="mfma",
                     kernel="fa_tile_kernel")
+    if name == "cfg2_bwd":
+        # the backward of the headline workload (same shape and inputs, plus a seeded dOut); FLOPs are the five matrix
+        # products of the algorithm (2.5 x the forward's), although the two-kernel design executes eight
+        B, H, S, D = 4, 32, 4096, 128
+        q, k, v, do = (seeded((B, H, S, D), 1 + i, bf).to(dev) for i in range(4))
+        out, lse, cq, ck, mq, mk, ps, po, _ = aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False)
+
+        def call():
+            return aten._scaled_dot_product_flash_attention_backward(do, q, k, v, out, lse, cq, ck, mq, mk, 0.0, True,
+                                                                     ps, po)
+
+        def check():
+            return _check_grads(q, k, v, do, call(), [(0, 0), (B - 1, H - 1)])
+
+        return dict(call=call, check=check, flops=10 * B * H * S * S * D / 2, bytes_kv=2 * B * H * S * D * 2,
+                    desc=f"backward of causal prefill bf16 B={B} H={H} S={S} D={D}", dtype="bf16", bound="mfma",
+                    kernel="fa_bwd_dq_kernel + fa_bwd_dkv_kernel<dK> + fa_bwd_dkv_kernel<dV>")
     if name == "cfg4":
         g = torch.Generator().manual_seed(3)
         lens = torch.randint(256, 2049, (16,), generator=g).tolist()
@@ -142,6 +160,24 @@ def _check_heads(q, k, v, out, lse, causal, heads):
     return eo, el
 
 
+def _check_grads(q, k, v, do, grads, heads):
+    """max-abs error of dQ / of dK and dV on sampled (batch, head) pairs against autograd through fp32 math on the
+    device (causal, MHA).  Returned in the (out, lse) slots of the bench record: (dQ error, max of dK and dV error)."""
+    Sq, Sk, D = q.shape[2], k.shape[2], q.shape[3]
+    r = torch.arange(Sq, device=q.device)[:, None]
+    c = torch.arange(Sk, device=q.device)[None, :]
+    eq = ekv = 0.0
+    for b, h in heads:
+        qq, kk, vv = (t[b, h].float().clone().requires_grad_() for t in (q, k, v))
+        s = (qq @ kk.T) / math.sqrt(D)
+        s = s.masked_fill(c > r + Sk - Sq, float("-inf"))
+        (torch.softmax(s, -1) @ vv).backward(do[b, h].float())
+        eq = max(eq, (grads[0][b, h].float() - qq.grad).abs().max().item())
+        ekv = max(ekv, (grads[1][b, h].float() - kk.grad).abs().max().item(),
+                  (grads[2][b, h].float() - vv.grad).abs().max().item())
+    return eq, ekv
+
+
 def time_steps(call, steps, warmup, spin_up_s=0.4):
     """Exactly `steps` timed calls between two device synchronisations; HIP events on the launch stream give the
     per-step device time.  Before the `warmup` untimed steps the same call is repeated for `spin_up_s` seconds (also
@@ -200,7 +236,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "copy1g"])
+    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "copy1g"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -227,6 +263,9 @@ def main():
         r = {"config": name, "workload": w["desc"], "ms_per_step": wall, "kernel_ms_mean": ev_mean,
              "kernel_ms_median": ev_med, "kernel_ms_min": ev_min, "tflops": w["flops"] / wall / 1e9,
              "kv_gbs": w["bytes_kv"] / wall / 1e6, "max_abs_err_out": eo, "max_abs_err_lse": el, "dtype": w["dtype"]}
+        if name.endswith("_bwd"):
+            r["max_abs_err_dq"], r["max_abs_err_dkv"] = r.pop("max_abs_err_out"), r.pop("max_abs_err_lse")
+            del r["kv_gbs"]
         if w["bound"] == "mfma":
             ach = w["flops"] / ev_mean / 1e9
             r["roofline"] = {"bound": "mfma", "kernel": w["kernel"], "achieved": ach, "peak": PEAK_MFMA_TFLOPS,
@@ -242,14 +281,14 @@ def main():
     main_r = run(args.config, args.steps, args.warmup)
     extras = []
     if not args.no_extras:
-        for name in ("cfg2", "cfg3", "cfg4", "cfg5"):
+        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd"):
             if name != args.config:
                 extras.append(run(name, args.steps, args.warmup))
 
     is_decode = args.config in ("cfg5", "copy1g")
     line = {
         "metric": "fwd attn TFLOP/s + % MFMA peak (bf16 S=4096 D=128); decode HBM GB/s",
-        "value": main_r["kv_gbs"] if is_decode else main_r["tflops"],
+        "value": main_r.get("kv_gbs") if is_decode else main_r["tflops"],
         "unit": "GB/s" if is_decode else "TFLOP/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -260,11 +299,13 @@ def main():
         "vs_baseline": None,
         "dtype": main_r["dtype"],
         "data": "synthetic (seeded N(0, 0.5^2), generated on the CPU in fp32 and cast)",
-        "config": {"workload": main_r["workload"], "name": args.config, "entry": "aten::_scaled_dot_product_flash_attention"
-                   if args.config != "cfg4" else "aten::_flash_attention_forward"},
+        "config": {"workload": main_r["workload"], "name": args.config,
+                   "entry": {"cfg4": "aten::_flash_attention_forward",
+                             "cfg2_bwd": "aten::_scaled_dot_product_flash_attention_backward"}.get(
+                                 args.config, "aten::_scaled_dot_product_flash_attention")},
         "roofline": main_r["roofline"],
-        "parity": {"max_abs_err_out": main_r["max_abs_err_out"], "max_abs_err_lse": main_r["max_abs_err_lse"],
-                   "against": "fp32 math on the device, 2 sampled (batch, head) pairs"},
+        "parity": dict({k: v for k, v in main_r.items() if k.startswith("max_abs_err")},
+                       against="fp32 math on the device, 2 sampled (batch, head) pairs"),
         "peaks": {"mfma_tflops": PEAK_MFMA_TFLOPS, "hbm_gbs": PEAK_HBM_GBS,
                   "device": torch.cuda.get_device_properties(0).gcnArchName,
                   "cus": torch.cuda.get_device_properties(0).multi_processor_count},
