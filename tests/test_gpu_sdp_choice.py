@@ -1,0 +1,115 @@
+"""The backend selector on the GPU: plain F.scaled_dot_product_attention (no backend forced) reaches this build's
+kernels for the inputs they take, is left to PyTorch's other backends otherwise, and the error paths of the reference's
+TestSDPAThrowException (test/torch_ops/test_scaled_dot_product_attention.py:243-420) behave the same."""
+import math
+import warnings
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+import torch_mlu_amd
+from tests._util import OUT_TOL, out_close, seeded
+from torch_mlu_amd.backends import SDPBackend, sdp_kernel
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF, HF = torch.bfloat16, torch.float16
+
+
+def _qkv(B, Hq, Hk, Sq, Sk, D, dtype, seed=0):
+    return (seeded((B, Hq, Sq, D), seed, dtype), seeded((B, Hk, Sk, D), seed + 1, dtype),
+            seeded((B, Hk, Sk, D), seed + 2, dtype))
+
+
+def test_plain_sdpa_reaches_this_builds_kernels():
+    cases = [dict(shape=(2, 4, 4, 200, 200, 128), causal=True, gqa=False, dtype=BF),
+             dict(shape=(2, 8, 2, 130, 130, 64), causal=False, gqa=True, dtype=HF),
+             dict(shape=(4, 8, 2, 1, 900, 128), causal=False, gqa=True, dtype=BF),      # decode -> split-KV
+             dict(shape=(1, 2, 2, 70, 300, 256), causal=False, gqa=False, dtype=HF)]    # head_dim 256, rectangular
+    for c in cases:
+        q, k, v = _qkv(*c["shape"], c["dtype"])
+        qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+        assert torch._fused_sdp_choice(qd, kd, vd, None, 0.0, c["causal"], enable_gqa=c["gqa"]) == SDPBackend.FLASH_ATTENTION
+        n0 = torch_mlu_amd.launch_count()
+        out = F.scaled_dot_product_attention(qd, kd, vd, is_causal=c["causal"], enable_gqa=c["gqa"])
+        assert torch_mlu_amd.launch_count() == n0 + 1, c
+        ref, _ = oracle.sdpa_oracle(q, k, v, is_causal=c["causal"])
+        out_close(out.float().cpu().numpy(), ref, c["dtype"])
+
+
+def test_training_through_plain_sdpa():
+    q, k, v = _qkv(2, 4, 4, 160, 160, 64, HF, seed=5)
+    qd, kd, vd = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    n0 = torch_mlu_amd.launch_count()
+    F.scaled_dot_product_attention(qd, kd, vd, is_causal=True).sum().backward()
+    assert torch_mlu_amd.launch_count() == n0 + 2
+    want = oracle.sdpa_backward_oracle(q, k, v, torch.ones_like(q), is_causal=True)
+    for t, w in zip((qd, kd, vd), want):
+        assert np.abs(t.grad.float().cpu().numpy() - w).max() <= 2 * 2.0 ** -11 * max(np.abs(w).max(), 0.25)
+
+
+def test_inputs_the_flash_kernels_do_not_take_go_elsewhere_and_stay_correct():
+    """Non-square causal (F.sdpa's mask is top-left aligned, the flash kernels' bottom-right), an attn_mask, fp32
+    inputs, and head_dim 256 with a gradient: the selector must not pick flash, and the answer is F.sdpa's."""
+    q, k, v = _qkv(1, 2, 2, 40, 72, 64, HF, seed=9)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    n0 = torch_mlu_amd.launch_count()
+    assert torch._fused_sdp_choice(qd, kd, vd, None, 0.0, True) != SDPBackend.FLASH_ATTENTION
+    out = F.scaled_dot_product_attention(qd, kd, vd, is_causal=True)
+    s = (q.double() @ k.double().transpose(-1, -2)) / math.sqrt(64)
+    s = s.masked_fill(~torch.ones(40, 72, dtype=torch.bool).tril(), float("-inf"))          # top-left
+    want = torch.softmax(s, -1) @ v.double()
+    assert (out.double().cpu() - want).abs().max().item() <= OUT_TOL[HF]
+    mask = torch.zeros(40, 72, dtype=HF, device=DEV)
+    assert torch._fused_sdp_choice(qd, kd, vd, mask) != SDPBackend.FLASH_ATTENTION
+    assert torch._fused_sdp_choice(qd.float(), kd.float(), vd.float()) != SDPBackend.FLASH_ATTENTION
+    q256 = torch.randn(1, 2, 16, 256, dtype=HF, device=DEV, requires_grad=True)
+    assert torch._fused_sdp_choice(q256, q256.detach(), q256.detach()) != SDPBackend.FLASH_ATTENTION
+    assert torch._fused_sdp_choice(q256.detach(), q256.detach(), q256.detach()) == SDPBackend.FLASH_ATTENTION
+    assert torch_mlu_amd.launch_count() == n0
+    # the selector leaves the user's flags as they were
+    assert torch.backends.cuda.flash_sdp_enabled()
+
+
+def test_no_backend_exception():
+    q, k, v = (torch.randn(2, 3, 4, device=DEV, dtype=HF) for _ in range(3))
+    with sdp_kernel(enable_flash=False, enable_math=False, enable_mem_efficient=False):
+        prev = torch.backends.cuda.cudnn_sdp_enabled()
+        torch.backends.cuda.enable_cudnn_sdp(False)
+        try:
+            with pytest.raises(RuntimeError, match="No viable backend for scaled_dot_product_attention was found."):
+                torch._fused_sdp_choice(q, k, v)
+            with pytest.raises(RuntimeError, match="No viable backend for scaled_dot_product_attention was found."):
+                F.scaled_dot_product_attention(q, k, v)
+        finally:
+            torch.backends.cuda.enable_cudnn_sdp(prev)
+
+
+@pytest.mark.parametrize("build,msg", [
+    (lambda: [torch.randn(2, 3, 8, device=DEV, dtype=HF) for _ in range(3)] + [None],
+     "Both fused kernels requires query, key and value to be 4 dimensional"),
+    (lambda: [torch.randn(1, 16, 64, 64, device=DEV, dtype=HF)] + [torch.randn(2, 16, 64, 64, device=DEV, dtype=HF)
+                                                                  for _ in range(2)] + [None],
+     "For dense inputs, both fused kernels require query, key and value to have the same batch_size and num_heads."),
+    (lambda: [torch.randn(2, 2, 3, 16, device=DEV, dtype=HF) for _ in range(3)] + [torch.ones(2, 2, 3, 3, device=DEV,
+                                                                                             dtype=HF)],
+     "Flash Attention does not support non-null attn_mask."),
+    (lambda: [torch.randn(2, 2, 0, 128, device=DEV, dtype=HF) for _ in range(3)] + [None],
+     "Both fused kernels do not support zero seq_len_q or seq_len_kv."),
+    (lambda: [torch.randn(2, 16, 64, 64, device=DEV, dtype=torch.float32) for _ in range(3)] + [None],
+     "Expected query, key and value to all be of dtype"),
+])
+def test_flash_only_refusals_warn_and_raise(build, msg):
+    q, k, v, mask = build()
+    with sdp_kernel(enable_flash=True, enable_math=False, enable_mem_efficient=False):
+        prev = torch.backends.cuda.cudnn_sdp_enabled()
+        torch.backends.cuda.enable_cudnn_sdp(False)
+        try:
+            with pytest.warns(UserWarning, match=msg):
+                with pytest.raises(RuntimeError, match="No available kernel"):
+                    F.scaled_dot_product_attention(q, k, v, mask, 0.0, False)
+        finally:
+            torch.backends.cuda.enable_cudnn_sdp(prev)

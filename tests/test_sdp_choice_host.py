@@ -1,0 +1,75 @@
+"""Host-only checks of the SDPA backend selector's input constraints (csrc/fa_sdp_choice.cpp), which restate
+torch_mlu/csrc/aten/operators/cnnl/transformers/sdp_utils.h:99-472 and are exercised by the reference's
+TestSDPAThrowException (test/torch_ops/test_scaled_dot_product_attention.py:243-420).  CPU tensors are enough: every
+constraint is checked before the device one."""
+import pytest
+import torch
+
+import torch_mlu_amd  # noqa: F401
+
+reason = torch.ops.torch_mlu_amd._flash_refusal_reason
+HF = torch.float16
+
+
+def _qkv(size, dtype=HF, size_k=None):
+    return torch.randn(size, dtype=dtype), torch.randn(size_k or size, dtype=dtype), torch.randn(size_k or size, dtype=dtype)
+
+
+def test_good_inputs_reach_the_device_check_last():
+    q, k, v = _qkv((2, 4, 16, 64))
+    assert "HIP device" in reason(q, k, v)
+    assert "HIP device" in reason(q, k, v, None, 0.0, True)
+
+
+@pytest.mark.parametrize("build,msg", [
+    (lambda: _qkv((2, 3, 8)), "Both fused kernels requires query, key and value to be 4 dimensional"),
+    (lambda: (torch.randn(1, 16, 32, 64, dtype=HF),) + _qkv((2, 16, 32, 64))[1:],
+     "For dense inputs, both fused kernels require query, key and value to have the same batch_size and num_heads."),
+    (lambda: _qkv((2, 8, 16, 64), size_k=(2, 2, 16, 64)), "same batch_size and num_heads"),     # GQA without enable_gqa
+    (lambda: _qkv((2, 2, 3, 9), size_k=(2, 2, 3, 10)), "Flash attention requires q,k,v to have the same last dimension"),
+    (lambda: _qkv((2, 2, 3, 12)), "divisible by 8"),
+    (lambda: _qkv((2, 2, 3, 264)), "at most 256"),
+    (lambda: _qkv((2, 2, 0, 128)), "Both fused kernels do not support zero seq_len_q or seq_len_kv."),
+    (lambda: _qkv((2, 16, 32, 64), dtype=torch.float32), "Expected query, key and value to all be of dtype"),
+    (lambda: _qkv((2, 16, 32, 64), dtype=torch.float64), "Expected query, key and value to all be of dtype"),
+])
+def test_constraint_messages(build, msg):
+    q, k, v = build()
+    assert msg in reason(q, k, v)
+
+
+def test_last_dim_stride():
+    q, k, v = _qkv((2, 2, 8, 128))
+    q = q.as_strided((2, 2, 8, 128), [2, 2, 2, 2])
+    assert "Both fused kernels require the last dimension of the input to have stride 1." in reason(q, k, v)
+
+
+def test_attn_mask_dropout_and_non_square_causal():
+    q, k, v = _qkv((2, 2, 3, 16))
+    assert "Flash Attention does not support non-null attn_mask." in reason(q, k, v, torch.ones(2, 2, 3, 3, dtype=HF))
+    assert "dropout" in reason(q, k, v, None, 0.1)
+    q2, k2, v2 = _qkv((2, 2, 3, 16), size_k=(2, 2, 7, 16))
+    assert "top-left" in reason(q2, k2, v2, None, 0.0, True)
+    assert "HIP device" in reason(q2, k2, v2, None, 0.0, False)
+
+
+def test_gqa_needs_the_flag_and_a_whole_group():
+    q, k, v = _qkv((2, 8, 16, 64), size_k=(2, 2, 16, 64))
+    assert "HIP device" in reason(q, k, v, None, 0.0, False, True)
+    q, k, v = _qkv((2, 8, 16, 64), size_k=(2, 3, 16, 64))
+    assert "multiple of the number of key/value heads" in reason(q, k, v, None, 0.0, False, True)
+
+
+def test_backward_head_dim_limit_only_when_a_gradient_is_required():
+    q, k, v = _qkv((1, 2, 16, 256))
+    assert "HIP device" in reason(q, k, v)
+    q.requires_grad_()
+    assert "at most 128 when a gradient is required" in reason(q, k, v)
+    with torch.no_grad():
+        assert "HIP device" in reason(q, k, v)
+
+
+def test_runtime_disabled():
+    q, k, v = _qkv((2, 4, 16, 64))
+    with torch_mlu_amd.backends.sdp_kernel(enable_flash=False, enable_math=True, enable_mem_efficient=True):
+        assert "Flash attention has been runtime disabled." in reason(q, k, v)

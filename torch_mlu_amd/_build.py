@@ -47,7 +47,8 @@ def build_kernels(verbose: bool = False) -> str:
 
 
 def build_aten(verbose: bool = False) -> str:
-    """g++: csrc/fa_aten.cpp -> lib/libfa_aten.so (registers the two aten ops; links libfa_fwd.so by $ORIGIN)."""
+    """g++: csrc/fa_aten.cpp + csrc/fa_sdp_choice.cpp -> lib/libfa_aten.so (registers the forward and backward aten ops
+    and the SDPA backend selector; links libfa_fwd.so by $ORIGIN)."""
     import torch
     from torch.utils import cpp_extension as ce
 
@@ -60,7 +61,7 @@ def build_aten(verbose: bool = False) -> str:
     cmd = [
         "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
         "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
-        *inc, os.path.join(CSRC, "fa_aten.cpp"), "-o", tmp,
+        *inc, os.path.join(CSRC, "fa_aten.cpp"), os.path.join(CSRC, "fa_sdp_choice.cpp"), "-o", tmp,
         f"-L{LIBDIR}", "-lfa_fwd", f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
         "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}", "-Wl,--no-as-needed",
     ]
