@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FA_FWD_ABI_VERSION 1
+#define FA_FWD_ABI_VERSION 2
 
 /* element types accepted for q/k/v/out (FlashAttention_internal.cpp:73-80 allows exactly these two) */
 #define FA_DTYPE_FP16 0
@@ -36,6 +36,12 @@ extern "C" {
 #define FA_ERR_UNSUPPORTED (-2) /* shape or dtype outside the supported envelope */
 #define FA_ERR_LAUNCH (-3)      /* the HIP runtime refused the launch (hipGetLastError != hipSuccess) */
 
+/* is_causal values */
+#define FA_MASK_NONE 0
+#define FA_MASK_CAUSAL_BOTTOM_RIGHT 1 /* col <= row + Lk - Lq: the flash entry points (reference oracle, construct_local_mask) */
+#define FA_MASK_CAUSAL_TOP_LEFT 2     /* col <= row: the mem-efficient entry points (CustomMaskType::CausalFromTopLeft,
+                                         attention.cpp:368-370) */
+
 /* kernel selection */
 #define FA_KERNEL_AUTO 0     /* split-KV kernel when seqlen_q == 1 and heads_q/heads_k <= 16, else the tile kernel */
 #define FA_KERNEL_TILE 1     /* MFMA tile (prefill) kernel */
@@ -44,9 +50,11 @@ extern "C" {
 /*
  * One attention-forward problem:  for every sequence b and query head h
  *     S   = scale * Q[b,h] K[b,h/(heads_q/heads_k)]^T      (fp32 accumulate)
- *     S   = -inf where is_causal and col > row + Lk_b - Lq_b (bottom-right aligned)
+ *     S  += bias[b,h]                                      (optional additive bias, mem-efficient entry points)
+ *     S   = -inf where is_causal and col > row + Lk_b - Lq_b (bottom-right aligned; FA_MASK_CAUSAL_TOP_LEFT: col > row)
  *     LSE = ln sum_j exp(S[:,j]),   out = softmax_row(S) V
- * which is what cnnlFlashAttentionForward_v2 is asked to compute (FlashAttention_internal.cpp:147-161,231-258).
+ * which is what cnnlFlashAttentionForward_v2 is asked to compute (FlashAttention_internal.cpp:147-161,231-258; with
+ * the bias descriptor of the mem-efficient launcher, :585-590,659-686).
  *
  * Addressing (all strides are in ELEMENTS, row (b,s,h) of X starts at X + b*x_stride_b + s*x_stride_s + h*x_stride_h,
  * the head_dim elements of a row are contiguous — the "contiguous last dimension" the reference demands at :101-108):
@@ -57,7 +65,12 @@ extern "C" {
  *          are only ever read on the device.
  * LSE element (b,h,s) is written at lse + b*lse_stride_b + h*lse_stride_h + s*lse_stride_s; in packed mode s is the
  * packed row index and lse_stride_b is ignored (the reference's kernel-side buffer is [heads_q, total_q], :129).
- * Rows with no visible key (possible only when is_causal and Lk < Lq, or Lk == 0) get out = 0 and LSE = +inf.
+ * Rows with no visible key (is_causal and Lk < Lq, Lk == 0, or a bias row that is -inf throughout) get out = 0 and
+ * LSE = +inf.
+ * bias (optional, dense mode only, same dtype as q): element (b,h,row,col) at bias + b*bias_stride_b + h*bias_stride_h
+ * + row*bias_stride_q + col; columns contiguous; stride 0 broadcasts over batch or heads (or rows); the base pointer
+ * and all three strides must keep 4-element groups 8-byte aligned (multiples of 4 elements).  A problem with a bias
+ * always runs the tile kernel.
  */
 typedef struct fa_fwd_params {
   const void* q;   /* device, 16-byte aligned */
@@ -83,10 +96,13 @@ typedef struct fa_fwd_params {
 
   float scale;       /* softmax scale, already resolved (attention.cpp:174-175 passes it as float) */
   int32_t dtype;     /* FA_DTYPE_* */
-  int32_t is_causal; /* 0/1 */
+  int32_t is_causal; /* FA_MASK_* (0 / 1 keep their old meaning) */
   int32_t kernel;    /* FA_KERNEL_* */
   int32_t num_splits; /* split-KV only: 0 = choose, else 1..FA_MAX_SPLITS */
   int32_t reserved;  /* must be 0 */
+
+  const void* bias;  /* device or NULL */
+  int64_t bias_stride_b, bias_stride_h, bias_stride_q;
 } fa_fwd_params;
 
 #define FA_MAX_SPLITS 64

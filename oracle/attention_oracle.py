@@ -55,12 +55,18 @@ def construct_local_mask(seqlen_q: int, seqlen_k: int, window_size=(-1, -1)) -> 
     return np.logical_or(col > np.minimum(row + sk - sq + window_size[1], sk), col < row + sk - sq - window_size[0])
 
 
-def attention_ref(q, k, v, scale: Optional[float] = None, causal: bool = False, dtype=np.float64
-                  ) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
+def attention_ref(q, k, v, scale: Optional[float] = None, causal: bool = False, dtype=np.float64,
+                  attn_bias=None, causal_top_left: bool = False) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
     """q [B, Sq, Hq, D], k/v [B, Sk, Hk, D]  (the reference oracle's layout, :94-97).
 
     Returns (output [B, Hq, Sq, D], attention [B, Hq, Sq, Sk], lse [B, Hq, Sq]) — the first two are what the
     reference's `attention_ref` returns (:103-105, :161); lse is added.
+
+    Two additions for the mem-efficient entry points, which the reference's `attention_ref` does not cover (its tests
+    compare those against the math backend): `attn_bias`, added to the scaled scores (broadcastable to
+    [B, Hq, Sq, Sk]; what the bias descriptor of mem_eff_fwd means, FlashAttention_internal.cpp:585-590), and
+    `causal_top_left`, the mask col > row of CustomMaskType::CausalFromTopLeft (attention.cpp:368-370) instead of the
+    bottom-right aligned one.  Both are pinned in tests/test_oracle.py against PyTorch's float64 math SDPA.
     """
     q, k, v = _np(q, dtype), _np(k, dtype), _np(v, dtype)
     B, Sq, Hq, D = q.shape
@@ -76,9 +82,14 @@ def attention_ref(q, k, v, scale: Optional[float] = None, causal: bool = False, 
     kh = np.ascontiguousarray(k.transpose(0, 2, 3, 1))   # [B,H,D,Sk]
     vh = np.ascontiguousarray(v.transpose(0, 2, 1, 3))   # [B,H,Sk,D]
     scores = np.matmul(qh, kh)                           # einsum("bthd,bshd->bhts")
+    if attn_bias is not None:
+        scores = scores + np.broadcast_to(_np(attn_bias, dtype), scores.shape)
     masked_rows = None
     if window[0] >= 0 or window[1] >= 0:
-        mask = construct_local_mask(Sq, Sk, window)
+        if causal_top_left:
+            mask = np.arange(Sk, dtype=np.int64)[None, :] > np.arange(Sq, dtype=np.int64)[:, None]
+        else:
+            mask = construct_local_mask(Sq, Sk, window)
         scores = np.where(mask[None, None], -np.inf, scores)
         masked_rows = mask.all(axis=-1)
     with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
@@ -95,8 +106,8 @@ def attention_ref(q, k, v, scale: Optional[float] = None, causal: bool = False, 
     return output, attention, lse
 
 
-def sdpa_oracle(q, k, v, is_causal: bool = False, scale: Optional[float] = None, dtype=np.float64
-                ) -> Tuple[np.ndarray, np.ndarray]:
+def sdpa_oracle(q, k, v, is_causal: bool = False, scale: Optional[float] = None, dtype=np.float64, attn_bias=None,
+                causal_top_left: bool = False) -> Tuple[np.ndarray, np.ndarray]:
     """Dense op layout: q [B, Hq, Sq, D], k/v [B, Hk, Sk, D] -> (out [B, Hq, Sq, D], lse [B, Hq, Sq]).
 
     The [B,H,S,D] -> [B,S,H,D] transposes are the ones the reference's dense wrapper makes
@@ -104,7 +115,8 @@ def sdpa_oracle(q, k, v, is_causal: bool = False, scale: Optional[float] = None,
     """
     q, k, v = _np(q, dtype), _np(k, dtype), _np(v, dtype)
     out, _, lse = attention_ref(q.transpose(0, 2, 1, 3), k.transpose(0, 2, 1, 3), v.transpose(0, 2, 1, 3),
-                                scale=scale, causal=is_causal, dtype=dtype)
+                                scale=scale, causal=is_causal, dtype=dtype, attn_bias=attn_bias,
+                                causal_top_left=causal_top_left)
     return out, lse
 
 

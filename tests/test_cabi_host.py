@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_version_and_error_strings():
     L = capi.lib()
-    assert L.fa_fwd_version() == 1
+    assert L.fa_fwd_version() == 2
     assert capi.error_string(0) == "ok"
     for rc in (-1, -2, -3, -99):
         assert capi.error_string(rc)
@@ -187,3 +187,28 @@ def test_bwd_null_and_short_workspace():
     p = _good_bwd()
     assert L.fa_bwd_launch(ctypes.byref(p), 0x10000, 16, None) == capi.FA_ERR_BAD_ARG
     assert L.fa_bwd_launch(ctypes.byref(p), None, 1 << 20, None) == capi.FA_ERR_BAD_ARG
+
+
+# ---- additive bias and mask alignment ------------------------------------------------------------------------------
+def test_bias_and_mask_mode_validation_and_plan():
+    L = capi.lib()
+    good = _good(bias=0x7000, bias_stride_b=0, bias_stride_h=128 * 256, bias_stride_q=256, is_causal=0)
+    assert L.fa_fwd_validate(ctypes.byref(good)) == capi.FA_OK
+    for over, rc in ((dict(bias=0x7004), capi.FA_ERR_BAD_ARG),                 # 4-key groups must be 8-byte aligned
+                     (dict(bias_stride_q=258), capi.FA_ERR_BAD_ARG),
+                     (dict(bias_stride_h=-4), capi.FA_ERR_BAD_ARG),
+                     (dict(cu_seqlens_q=0x6000, cu_seqlens_k=0x6100), capi.FA_ERR_UNSUPPORTED),   # packed + bias
+                     (dict(kernel=capi.FA_KERNEL_SPLITKV, seqlen_q=1), capi.FA_ERR_UNSUPPORTED),
+                     (dict(is_causal=3), capi.FA_ERR_BAD_ARG)):
+        p = _good(**{**dict(bias=0x7000, bias_stride_b=0, bias_stride_h=128 * 256, bias_stride_q=256), **over})
+        assert L.fa_fwd_validate(ctypes.byref(p)) == rc, over
+    # a single query row with a bias, or with a top-left causal mask, runs the tile kernel
+    kern, ns = ctypes.c_int32(), ctypes.c_int32()
+    dec = _good(seqlen_q=1, seqlen_k=4096, is_causal=0)
+    assert L.fa_fwd_plan(ctypes.byref(dec), ctypes.byref(kern), ctypes.byref(ns)) == 0 and kern.value == capi.FA_KERNEL_SPLITKV
+    dec.bias, dec.bias_stride_q = 0x7000, 4096
+    assert L.fa_fwd_plan(ctypes.byref(dec), ctypes.byref(kern), ctypes.byref(ns)) == 0 and kern.value == capi.FA_KERNEL_TILE
+    tl = _good(seqlen_q=1, seqlen_k=4096, is_causal=capi.FA_MASK_CAUSAL_TOP_LEFT)
+    assert L.fa_fwd_plan(ctypes.byref(tl), ctypes.byref(kern), ctypes.byref(ns)) == 0 and kern.value == capi.FA_KERNEL_TILE
+    tl.kernel = capi.FA_KERNEL_SPLITKV
+    assert L.fa_fwd_validate(ctypes.byref(tl)) == capi.FA_ERR_UNSUPPORTED

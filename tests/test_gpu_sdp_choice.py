@@ -51,27 +51,52 @@ def test_training_through_plain_sdpa():
         assert np.abs(t.grad.float().cpu().numpy() - w).max() <= 2 * 2.0 ** -11 * max(np.abs(w).max(), 0.25)
 
 
-def test_inputs_the_flash_kernels_do_not_take_go_elsewhere_and_stay_correct():
-    """Non-square causal (F.sdpa's mask is top-left aligned, the flash kernels' bottom-right), an attn_mask, fp32
-    inputs, and head_dim 256 with a gradient: the selector must not pick flash, and the answer is F.sdpa's."""
+def test_what_flash_cannot_take_goes_to_mem_efficient_or_elsewhere_and_stays_correct():
+    """Non-square causal (F.sdpa's mask is top-left aligned, the flash kernels' bottom-right) and an attn_mask go to
+    this build's mem-efficient entry point; fp32 inputs and head_dim 256 with a gradient are left to PyTorch."""
     q, k, v = _qkv(1, 2, 2, 40, 72, 64, HF, seed=9)
     qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
     n0 = torch_mlu_amd.launch_count()
-    assert torch._fused_sdp_choice(qd, kd, vd, None, 0.0, True) != SDPBackend.FLASH_ATTENTION
+    assert torch._fused_sdp_choice(qd, kd, vd, None, 0.0, True) == SDPBackend.EFFICIENT_ATTENTION
     out = F.scaled_dot_product_attention(qd, kd, vd, is_causal=True)
+    assert torch_mlu_amd.launch_count() == n0 + 1
     s = (q.double() @ k.double().transpose(-1, -2)) / math.sqrt(64)
     s = s.masked_fill(~torch.ones(40, 72, dtype=torch.bool).tril(), float("-inf"))          # top-left
     want = torch.softmax(s, -1) @ v.double()
     assert (out.double().cpu() - want).abs().max().item() <= OUT_TOL[HF]
     mask = torch.zeros(40, 72, dtype=HF, device=DEV)
-    assert torch._fused_sdp_choice(qd, kd, vd, mask) != SDPBackend.FLASH_ATTENTION
-    assert torch._fused_sdp_choice(qd.float(), kd.float(), vd.float()) != SDPBackend.FLASH_ATTENTION
+    assert torch._fused_sdp_choice(qd, kd, vd, mask) == SDPBackend.EFFICIENT_ATTENTION
+    fused = (SDPBackend.FLASH_ATTENTION, SDPBackend.EFFICIENT_ATTENTION)
+    assert torch._fused_sdp_choice(qd.float(), kd.float(), vd.float()) not in fused
     q256 = torch.randn(1, 2, 16, 256, dtype=HF, device=DEV, requires_grad=True)
-    assert torch._fused_sdp_choice(q256, q256.detach(), q256.detach()) != SDPBackend.FLASH_ATTENTION
+    assert torch._fused_sdp_choice(q256, q256.detach(), q256.detach()) not in fused
     assert torch._fused_sdp_choice(q256.detach(), q256.detach(), q256.detach()) == SDPBackend.FLASH_ATTENTION
-    assert torch_mlu_amd.launch_count() == n0
+    assert torch_mlu_amd.launch_count() == n0 + 1
     # the selector leaves the user's flags as they were
-    assert torch.backends.cuda.flash_sdp_enabled()
+    assert torch.backends.cuda.flash_sdp_enabled() and torch.backends.cuda.mem_efficient_sdp_enabled()
+
+
+def test_attn_mask_through_plain_sdpa():
+    """Float and boolean masks, broadcast shapes, GQA: one launch of this build's kernel each, answer = the oracle's."""
+    B, Hq, Hk, Sq, Sk, D = 2, 4, 2, 150, 203, 64
+    q, k, v = _qkv(B, Hq, Hk, Sq, Sk, D, BF, seed=21)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    g = torch.Generator().manual_seed(3)
+    for mshape in ((B, Hq, Sq, Sk), (B, 1, Sq, Sk), (1, 1, Sq, Sk), (Sq, Sk), (B, 1, 1, Sk)):
+        fmask = (torch.randn(mshape, generator=g) * 2).to(BF)
+        bmask = torch.rand(mshape, generator=g) > 0.3
+        for m in (fmask, bmask):
+            n0 = torch_mlu_amd.launch_count()
+            out = F.scaled_dot_product_attention(qd, kd, vd, attn_mask=m.to(DEV), enable_gqa=True)
+            assert torch_mlu_amd.launch_count() == n0 + 1, (mshape, m.dtype)
+            bias = m.float() if m.dtype != torch.bool else torch.zeros(mshape).masked_fill(~m, float("-inf"))
+            ref, _ = oracle.sdpa_oracle(q, k, v, attn_bias=bias.double().numpy())
+            dead = ~np.isfinite(bias.double().numpy()).any(-1)          # rows that see nothing: this build gives 0
+            got = out.float().cpu().numpy()
+            assert np.isfinite(got).all()
+            out_close(got, ref, BF)
+            if dead.any():
+                assert np.abs(got[np.broadcast_to(dead[..., None], got.shape[:-1] + (1,))[..., 0]]).max() == 0.0
 
 
 def test_no_backend_exception():

@@ -244,3 +244,69 @@ def test_tolerance_rule_restatement():
     assert math.isclose(rtol, 2 * 1.6e-2)
     atol, rtol = oracle.get_tolerances(t, t + 0.5, "float16", fudge_factor=None)
     assert math.isclose(atol, 0.5)
+
+
+# ---- additive bias and top-left causal (mem-efficient entry points) ----------------------------------------------
+@pytest.mark.parametrize("shape", [(2, 3, 3, 17, 29, 16), (1, 4, 2, 33, 12, 8)])
+@pytest.mark.parametrize("bias_shape", ["full", "head_broadcast", "row_broadcast"])
+def test_bias_oracle_vs_torch_math_float64(shape, bias_shape):
+    B, Hq, Hk, Sq, Sk, D = shape
+    q, k, v = seeded((B, Hq, Sq, D), 50, torch.float64), seeded((B, Hk, Sk, D), 51, torch.float64), seeded(
+        (B, Hk, Sk, D), 52, torch.float64)
+    bshape = {"full": (B, Hq, Sq, Sk), "head_broadcast": (B, 1, Sq, Sk), "row_broadcast": (1, 1, 1, Sk)}[bias_shape]
+    bias = seeded(bshape, 53, torch.float64, std=2.0)
+    out, lse = oracle.sdpa_oracle(q, k, v, attn_bias=bias, scale=0.37)
+    g = Hq // Hk
+    with torch.nn.attention.sdpa_kernel(torch.nn.attention.SDPBackend.MATH):
+        ref = F.scaled_dot_product_attention(q, k.repeat_interleave(g, 1), v.repeat_interleave(g, 1), attn_mask=bias,
+                                             scale=0.37)
+    assert np.abs(out - ref.numpy()).max() < 1e-12
+    s = torch.matmul(q, k.repeat_interleave(g, 1).transpose(-1, -2)) * 0.37 + bias
+    assert np.abs(lse - torch.logsumexp(s, -1).numpy()).max() < 1e-12
+
+
+def test_boolean_mask_as_minus_inf_bias_and_fully_masked_rows():
+    q, k, v = (seeded((1, 2, 6, 8), 60 + i, torch.float64) for i in range(3))
+    keep = torch.rand(1, 1, 6, 6, generator=torch.Generator().manual_seed(1)) > 0.4
+    keep[0, 0, 2] = False                                   # one row sees nothing
+    bias = torch.zeros(1, 1, 6, 6, dtype=torch.float64).masked_fill(~keep, float("-inf"))
+    out, lse = oracle.sdpa_oracle(q, k, v, attn_bias=bias)
+    for i in range(6):
+        cols = keep[0, 0, i].nonzero()[:, 0]
+        if len(cols) == 0:
+            assert np.abs(out[:, :, i]).max() == 0.0 and np.isposinf(lse[:, :, i]).all()
+            continue
+        o2, l2 = oracle.sdpa_oracle(q[:, :, i:i + 1], k[:, :, cols], v[:, :, cols])     # same as dropping those keys
+        assert np.abs(out[:, :, i:i + 1] - o2).max() < 1e-13 and np.abs(lse[:, :, i:i + 1] - l2).max() < 1e-13
+
+
+def test_bias_closed_forms():
+    """q = 0 and bias = ln w: out = sum_j w_j v_j / sum_j w_j, LSE = ln sum_j w_j.  A bias constant along a row changes
+    nothing but the LSE (by that constant)."""
+    k, v = seeded((1, 1, 9, 4), 70, torch.float64), seeded((1, 1, 9, 4), 71, torch.float64)
+    w = torch.rand(5, 9, dtype=torch.float64, generator=torch.Generator().manual_seed(2)) + 0.1
+    out, lse = oracle.sdpa_oracle(torch.zeros(1, 1, 5, 4, dtype=torch.float64), k, v, attn_bias=torch.log(w)[None, None])
+    assert np.abs(out[0, 0] - ((w @ v[0, 0]) / w.sum(-1, keepdim=True)).numpy()).max() < 1e-13
+    assert np.abs(lse[0, 0] - torch.log(w.sum(-1)).numpy()).max() < 1e-13
+    q = seeded((1, 1, 5, 4), 72, torch.float64)
+    o0, l0 = oracle.sdpa_oracle(q, k, v)
+    rowc = torch.arange(5, dtype=torch.float64)[None, None, :, None] * 1.5
+    o1, l1 = oracle.sdpa_oracle(q, k, v, attn_bias=rowc.expand(1, 1, 5, 9))
+    assert np.abs(o1 - o0).max() < 1e-13 and np.abs(l1 - l0 - rowc[..., 0].numpy()).max() < 1e-13
+
+
+@pytest.mark.parametrize("sq,sk", [(5, 9), (9, 5), (7, 7), (1, 4)])
+def test_top_left_causal_vs_torch_math(sq, sk):
+    """F.scaled_dot_product_attention(is_causal=True) is defined with a top-left aligned mask (tril of ones(L, S))."""
+    q, k, v = seeded((2, 2, sq, 8), 80, torch.float64), seeded((2, 2, sk, 8), 81, torch.float64), seeded(
+        (2, 2, sk, 8), 82, torch.float64)
+    out, lse = oracle.sdpa_oracle(q, k, v, is_causal=True, causal_top_left=True)
+    with torch.nn.attention.sdpa_kernel(torch.nn.attention.SDPBackend.MATH):
+        ref = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+    assert np.abs(out - ref.numpy()).max() < 1e-12
+    if sq == sk:
+        o2, l2 = oracle.sdpa_oracle(q, k, v, is_causal=True)
+        assert np.abs(out - o2).max() == 0.0 and np.abs(lse - l2).max() == 0.0
+    if sq <= sk:    # row i sees i + 1 keys whatever sk is
+        o3, l3 = oracle.sdpa_oracle(q, k[:, :, :sq], v[:, :, :sq], is_causal=True)
+        assert np.abs(out - o3).max() < 1e-13

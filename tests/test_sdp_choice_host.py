@@ -73,3 +73,24 @@ def test_runtime_disabled():
     q, k, v = _qkv((2, 4, 16, 64))
     with torch_mlu_amd.backends.sdp_kernel(enable_flash=False, enable_math=True, enable_mem_efficient=True):
         assert "Flash attention has been runtime disabled." in reason(q, k, v)
+
+
+# ---- this build's mem-efficient entry point ------------------------------------------------------------------------
+mem_reason = torch.ops.torch_mlu_amd._mem_efficient_refusal_reason
+
+
+def test_mem_efficient_constraints():
+    q, k, v = _qkv((2, 4, 16, 64))
+    mask = torch.zeros(16, 16, dtype=HF)
+    assert "HIP device" in mem_reason(q, k, v, mask)                       # everything else passes
+    assert "HIP device" in mem_reason(q, k, v, torch.ones(16, 16, dtype=torch.bool))
+    q2, k2, v2 = _qkv((2, 4, 16, 64), size_k=(2, 4, 40, 64))
+    assert "HIP device" in mem_reason(q2, k2, v2, None, 0.0, True)         # non-square causal is fine here (top-left)
+    assert "boolean mask or have the dtype of query" in mem_reason(q, k, v, torch.zeros(16, 16))
+    assert "dropout" in mem_reason(q, k, v, None, 0.1)
+    assert "Mem efficient attention requires query.size(-1)==key.size(-1)==value.size(-1)" in mem_reason(*_qkv((2, 2, 3, 12)))
+    assert "4 dimensional" in mem_reason(*_qkv((2, 3, 8)))
+    assert "no backward" in mem_reason(q.clone().requires_grad_(), k, v)
+    assert "no backward" in mem_reason(q, k, v, mask.clone().requires_grad_())
+    with torch_mlu_amd.backends.sdp_kernel(enable_flash=True, enable_math=True, enable_mem_efficient=False):
+        assert "Memory Efficient attention has been runtime disabled." in mem_reason(q, k, v)

@@ -27,6 +27,7 @@ FA_OK = 0
 FA_ERR_BAD_ARG = -1
 FA_ERR_UNSUPPORTED = -2
 FA_ERR_LAUNCH = -3
+FA_MASK_NONE, FA_MASK_CAUSAL_BOTTOM_RIGHT, FA_MASK_CAUSAL_TOP_LEFT = 0, 1, 2
 FA_KERNEL_AUTO = 0
 FA_KERNEL_TILE = 1
 FA_KERNEL_SPLITKV = 2
@@ -74,6 +75,8 @@ class FaFwdParams(ctypes.Structure):
         ("kernel", ctypes.c_int32),
         ("num_splits", ctypes.c_int32),
         ("reserved", ctypes.c_int32),
+        ("bias", ctypes.c_void_p),
+        ("bias_stride_b", ctypes.c_int64), ("bias_stride_h", ctypes.c_int64), ("bias_stride_q", ctypes.c_int64),
     ]
 
 
@@ -147,8 +150,10 @@ def _dtype_code(dt: torch.dtype) -> int:
 def make_params(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor, *,
                 cu_seqlens_q: Optional[torch.Tensor] = None, cu_seqlens_k: Optional[torch.Tensor] = None,
                 max_seqlen_q: int = 0, max_seqlen_k: int = 0, scale: Optional[float] = None,
-                is_causal: bool = False, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0) -> FaFwdParams:
-    """Fill a params struct.
+                is_causal=False, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
+                bias: Optional[torch.Tensor] = None) -> FaFwdParams:
+    """Fill a params struct.  `is_causal`: False / True (bottom-right aligned) or one of the FA_MASK_* codes; `bias`:
+    a [B, Hq, Sq, Sk] view (dense mode; stride 0 where broadcast) of the inputs' dtype.
 
     Dense: q/out are [B, Sq, Hq, D] *views* (any strides with a contiguous last dim), k/v [B, Sk, Hk, D],
     lse [B, Hq, Sq].  Packed: q/out [Tq, Hq, D], k/v [Tk, Hk, D], lse [Hq, Tq], cu_seqlens int32 [B+1].
@@ -183,10 +188,15 @@ def make_params(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Te
     # (torch_mlu/csrc/aten/operators/cnnl/transformers/sdp_utils.h:40-47, attention.cpp:174-175)
     p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
     p.dtype = _dtype_code(q.dtype)
-    p.is_causal = 1 if is_causal else 0
+    p.is_causal = int(is_causal)
     p.kernel = kernel
     p.num_splits = num_splits
     p.reserved = 0
+    if bias is not None:
+        p.bias = bias.data_ptr()
+        p.bias_stride_b, p.bias_stride_h, p.bias_stride_q = bias.stride(0), bias.stride(1), bias.stride(2)
+    else:
+        p.bias = None
     return p
 
 
@@ -201,16 +211,19 @@ def launch(p: FaFwdParams, device: torch.device) -> None:
         raise FaFwdError(rc)
 
 
-def fa_forward_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, is_causal: bool = False,
-                     scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO,
-                     num_splits: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+def fa_forward_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, is_causal=False,
+                     scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
+                     bias: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """q [B, Hq, Sq, D], k/v [B, Hk, Sk, D] (any strides, contiguous last dim) -> out [B, Hq, Sq, D] (stored
-    [B, Sq, Hq, D] like the reference's dense wrapper, attention.cpp:146-148), lse [B, Hq, Sq] fp32."""
+    [B, Sq, Hq, D] like the reference's dense wrapper, attention.cpp:146-148), lse [B, Hq, Sq] fp32.
+    `bias`: anything that expands to [B, Hq, Sq, Sk]; `is_causal` may also be FA_MASK_CAUSAL_TOP_LEFT."""
     B, Hq, Sq, D = q.shape
+    if bias is not None:
+        bias = bias.expand(B, Hq, Sq, k.shape[2])
     out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
     p = make_params(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), out, lse, scale=scale,
-                    is_causal=is_causal, kernel=kernel, num_splits=num_splits)
+                    is_causal=is_causal, kernel=kernel, num_splits=num_splits, bias=bias)
     launch(p, q.device)
     return out.transpose(1, 2), lse
 

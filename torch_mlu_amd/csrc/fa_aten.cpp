@@ -395,6 +395,142 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> scaled_dot_product_flash_attentio
   return std::make_tuple(grad_q.transpose(1, 2), grad_k.transpose(1, 2), grad_v.transpose(1, 2));
 }
 
+namespace {
+// The mem-efficient entry points of this build have no backward: refuse loudly instead of letting autograd pair this
+// forward with another implementation's backward.
+void check_no_gradient_required(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                const std::optional<at::Tensor>& bias) {
+  TORCH_CHECK(!(at::GradMode::is_enabled() && (q.requires_grad() || k.requires_grad() || v.requires_grad() ||
+                                                (bias.has_value() && bias->defined() && bias->requires_grad()))),
+              "efficient attention forward: this build has no backward for the mem-efficient entry points; use the "
+              "flash or math backend for training");
+}
+}  // namespace
+
+// ---- _efficient_attention_forward -------------------------------------------------------------------------------
+// cnnl__efficient_attention_forward (attention.cpp:390-508) + mem_eff_fwd (FlashAttention_internal.cpp:485-690):
+// inputs [B, S, H, D], optional additive bias broadcastable to [B, H, Sq, Skv], custom_mask_type 0 (none),
+// 1 (causal from the top-left corner) or 2 (causal from the bottom-right corner).  No contiguous copies of q/k/v.
+// Returned as the installed PyTorch's schema asks: output [B, Sq, H, D] (the dense wrapper transposes it),
+// logsumexp [B, H, Sq] (or [B, H, 0] without compute_log_sumexp), philox slots, and the two maximum lengths.
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::SymInt> efficient_attention_forward(
+    const at::Tensor& query, const at::Tensor& key, const at::Tensor& value, const std::optional<at::Tensor>& bias,
+    const std::optional<at::Tensor>& cu_seqlens_q, const std::optional<at::Tensor>& cu_seqlens_k,
+    std::optional<c10::SymInt> max_seqlen_q, std::optional<c10::SymInt> max_seqlen_k, double dropout_p,
+    int64_t custom_mask_type, bool compute_log_sumexp, std::optional<double> scale,
+    const std::optional<at::Tensor>& seqlen_k, std::optional<int64_t> window_size) {
+  (void)max_seqlen_q;
+  (void)max_seqlen_k;
+  // the reference's checks, in its order (attention.cpp:405-423)
+  TORCH_CHECK(query.dim() == 4 && key.dim() == 4 && value.dim() == 4, "query, key and value must be 4-dimensional "
+              "(batch, seq_len, num_heads, head_dim)");
+  TORCH_CHECK(query.size(0) == key.size(0) && query.size(0) == value.size(0), "query, key and value must have the same batch size");
+  TORCH_CHECK(key.size(1) == value.size(1), "key and value must have the same sequence length");
+  TORCH_CHECK(key.size(2) == value.size(2) && key.size(2) > 0 && query.size(2) % key.size(2) == 0,
+              "Number of heads in key/value must divide number of heads in query");
+  TORCH_CHECK(query.size(3) == key.size(3), "query and key must have the same head dimension");
+  TORCH_CHECK(value.size(3) == query.size(3), "this build needs value.size(-1) == query.size(-1)");
+  TORCH_CHECK(!(cu_seqlens_q.has_value() && cu_seqlens_q->defined()) && !(cu_seqlens_k.has_value() && cu_seqlens_k->defined()),
+              "efficient attention forward: cu_seqlens are not supported by this build (use _flash_attention_forward)");
+  TORCH_CHECK(!(seqlen_k.has_value() && seqlen_k->defined()), "efficient attention forward: seqlen_k is not supported");
+  TORCH_CHECK(!window_size.has_value() || *window_size <= 0, "efficient attention forward: sliding window is not supported");
+  TORCH_CHECK(dropout_p == 0.0, "efficient attention forward: dropout_p > 0 is not supported by this build");
+  TORCH_CHECK(custom_mask_type >= 0 && custom_mask_type <= 2, "custom_mask_type must be 0, 1 or 2");
+  check_no_gradient_required(query, key, value, bias);
+  // mem_eff_fwd's checks (FlashAttention_internal.cpp:500-527)
+  const auto dt = query.scalar_type();
+  TORCH_CHECK(dt == at::kHalf || dt == at::kBFloat16, "FlashAttention only support fp16 and bf16 data type");
+  TORCH_CHECK(key.scalar_type() == dt, "query and key must have the same dtype");
+  TORCH_CHECK(value.scalar_type() == dt, "query and value must have the same dtype");
+  TORCH_CHECK(query.is_cuda() && key.is_cuda() && value.is_cuda(), "Input tensor must be on HIP device");
+  TORCH_CHECK(query.stride(-1) == 1 && key.stride(-1) == 1 && value.stride(-1) == 1,
+              "Input tensor must have contiguous last dimension");
+  const int64_t B = query.size(0), Sq = query.size(1), Hq = query.size(2), D = query.size(3);
+  const int64_t Sk = key.size(1), Hk = key.size(2);
+  TORCH_CHECK(B > 0, "batch size must be positive");
+  TORCH_CHECK(D <= 256, "FlashAttention forward only supports head dimension at most 256");
+  TORCH_CHECK(D % 8 == 0, "head dimension must be a multiple of 8");
+  TORCH_CHECK(Sq <= INT32_MAX && Sk <= INT32_MAX && B <= INT32_MAX, "sequence length too large");
+
+  const c10::OptionalDeviceGuard guard(query.device());
+  const float softmax_scale = resolve_scale(query, scale);
+  const at::Tensor q = aligned_or_copy(query), k = aligned_or_copy(key), v = aligned_or_copy(value);
+  at::Tensor output = at::empty({B, Sq, Hq, D}, q.options());
+  at::Tensor lse = at::empty({B, Hq, Sq}, q.options().dtype(at::kFloat));
+
+  at::Tensor bias_e;  // [B, H, Sq, Sk] view (stride 0 where broadcast), 4-element groups 8-byte aligned
+  if (bias.has_value() && bias->defined()) {
+    TORCH_CHECK(bias->scalar_type() == dt, "bias must have the same dtype as query");
+    TORCH_CHECK(bias->is_cuda(), "bias must be on HIP device");
+    TORCH_CHECK(bias->dim() <= 4, "bias must have at most 4 dimensions");
+    bias_e = bias->expand({B, Hq, Sq, Sk});
+    const bool ok = Sk == 0 || (bias_e.stride(3) == 1 && bias_e.stride(0) % 4 == 0 && bias_e.stride(1) % 4 == 0 &&
+                                bias_e.stride(2) % 4 == 0 && reinterpret_cast<uintptr_t>(bias_e.data_ptr()) % 8 == 0);
+    if (!ok) {  // one copy of the un-broadcast bias with rows padded to a multiple of 8 columns (the reference always copies)
+      const int64_t Skp = (Sk + 7) / 8 * 8;
+      at::Tensor b4 = *bias;
+      while (b4.dim() < 4) b4 = b4.unsqueeze(0);
+      at::Tensor padded = at::empty({b4.size(0), b4.size(1), b4.size(2), Skp}, b4.options());
+      padded.narrow(3, 0, Sk).copy_(b4.expand({b4.size(0), b4.size(1), b4.size(2), Sk}));
+      bias_e = padded.narrow(3, 0, Sk).expand({B, Hq, Sq, Sk});
+    }
+  }
+
+  fa_fwd_params p{};
+  p.q = q.data_ptr(); p.k = k.data_ptr(); p.v = v.data_ptr(); p.out = output.data_ptr();
+  p.lse = lse.data_ptr<float>();
+  fill_strides(q, false, p.q_stride_b, p.q_stride_s, p.q_stride_h);
+  fill_strides(k, false, p.k_stride_b, p.k_stride_s, p.k_stride_h);
+  fill_strides(v, false, p.v_stride_b, p.v_stride_s, p.v_stride_h);
+  fill_strides(output, false, p.o_stride_b, p.o_stride_s, p.o_stride_h);
+  p.lse_stride_b = lse.stride(0); p.lse_stride_h = lse.stride(1); p.lse_stride_s = lse.stride(2);
+  p.batch = static_cast<int32_t>(B);
+  p.heads_q = static_cast<int32_t>(Hq);
+  p.heads_k = static_cast<int32_t>(Hk);
+  p.seqlen_q = static_cast<int32_t>(Sq);
+  p.seqlen_k = static_cast<int32_t>(Sk);
+  p.head_dim = static_cast<int32_t>(D);
+  p.scale = softmax_scale;
+  p.dtype = dt == at::kBFloat16 ? FA_DTYPE_BF16 : FA_DTYPE_FP16;
+  p.is_causal = custom_mask_type == 1 ? FA_MASK_CAUSAL_TOP_LEFT
+                                      : (custom_mask_type == 2 ? FA_MASK_CAUSAL_BOTTOM_RIGHT : FA_MASK_NONE);
+  p.kernel = FA_KERNEL_AUTO;
+  if (bias_e.defined() && Sk > 0) {
+    p.bias = bias_e.data_ptr();
+    p.bias_stride_b = bias_e.stride(0); p.bias_stride_h = bias_e.stride(1); p.bias_stride_q = bias_e.stride(2);
+  }
+  if (B * Sq * Hq > 0) {
+    const size_t ws_bytes = fa_fwd_workspace_bytes(&p);
+    at::Tensor ws;
+    if (ws_bytes) ws = at::empty({static_cast<int64_t>(ws_bytes)}, q.options().dtype(at::kByte));
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
+    const int rc = fa_fwd_launch(&p, ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, stream);
+    TORCH_CHECK(rc == FA_OK, "fa_fwd_launch failed: ", fa_fwd_error_string(rc), " (rc=", rc, ")");
+    g_launches.fetch_add(1, std::memory_order_relaxed);
+  }
+  at::Tensor seed_t = at::empty({}, q.options().dtype(at::kLong));
+  at::Tensor offset_t = at::empty({}, q.options().dtype(at::kLong));
+  if (!compute_log_sumexp) lse = at::empty({B, Hq, 0}, q.options().dtype(at::kFloat));
+  return std::make_tuple(output, lse, seed_t, offset_t, c10::SymInt(Sq), c10::SymInt(Sk));
+}
+
+// ---- _scaled_dot_product_efficient_attention -------------------------------------------------------------------
+// cnnl__scaled_dot_product_efficient_attention, attention.cpp:350-388: [B, H, S, D] in, transposes, causal from the
+// top-left corner (:368-370), output returned as the [B, H, Sq, D] view of [B, Sq, H, D] storage.
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> scaled_dot_product_efficient_attention(
+    const at::Tensor& query, const at::Tensor& key, const at::Tensor& value, const std::optional<at::Tensor>& attn_bias,
+    bool compute_log_sumexp, double dropout_p, bool is_causal, std::optional<double> scale) {
+  TORCH_CHECK(query.dim() == 4 && key.dim() == 4 && value.dim() == 4,
+              "query, key and value must be 4-dimensional (batch, num_heads, seq_len, head_dim)");
+  check_no_gradient_required(query, key, value, attn_bias);  // the views made below do not carry requires_grad
+  auto [out, lse, seed, offset, mq, mk] = efficient_attention_forward(
+      query.transpose(1, 2), key.transpose(1, 2), value.transpose(1, 2), attn_bias, std::nullopt, std::nullopt,
+      std::nullopt, std::nullopt, dropout_p, is_causal ? 1 : 0, compute_log_sumexp, scale, std::nullopt, std::nullopt);
+  (void)mq;
+  (void)mk;
+  return std::make_tuple(out.transpose(1, 2), lse, seed, offset);
+}
+
 // ---- test hooks -----------------------------------------------------------------------------------------------
 int64_t launch_count() { return g_launches.load(std::memory_order_relaxed); }
 
@@ -418,6 +554,8 @@ TORCH_LIBRARY_IMPL(aten, CUDA, m) {
   m.impl("_scaled_dot_product_flash_attention_backward",
          TORCH_FN(torch_mlu_amd::scaled_dot_product_flash_attention_backward));
   m.impl("_flash_attention_backward", TORCH_FN(torch_mlu_amd::flash_attention_backward));
+  m.impl("_scaled_dot_product_efficient_attention", TORCH_FN(torch_mlu_amd::scaled_dot_product_efficient_attention));
+  m.impl("_efficient_attention_forward", TORCH_FN(torch_mlu_amd::efficient_attention_forward));
 }
 
 TORCH_LIBRARY(torch_mlu_amd, m) {

@@ -53,6 +53,9 @@ struct KArgs {
   int32_t is_causal;
   int32_t neg_scale;  // scale < 0: Q is negated on load and |scale| is used, so that max() tracks the true row max
   float scale_log2;   // |scale| * log2(e)
+  int32_t causal_tl;  // causal mask aligned to the top-left corner (col <= row) instead of the bottom-right one
+  const unsigned char* bias;  // optional additive bias, dense mode: [b][h][row][col] through byte strides
+  int64_t bias_sb, bias_sh, bias_sq;
   float* ws_o;        // split-KV partials: [batch*heads_q*n_splits][head_dim] fp32, unnormalised
   float* ws_ml;       // [batch*heads_q*n_splits][2]: m (log2 domain), l
 };
@@ -82,7 +85,9 @@ __device__ __forceinline__ int swzV(int row) {
 // depend on which maximum was in use.
 constexpr float kLazyLog2 = 8.0f;
 
-template <typename T, int DP, int MINB>
+// BIAS: an additive bias tile is read straight from global memory into the score layout (one lane = one query row,
+// groups of 4 consecutive keys = 8 bytes) and the softmax then runs on scores already in the log2 domain.
+template <typename T, int DP, int MINB, bool BIAS>
 __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   constexpr int CPR = DP / 8;          // 16-byte chunks per row
   constexpr int ROWB = DP * 2;         // bytes per LDS row
@@ -139,7 +144,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   const int blk_first = (a.cu_q ? a.n_mblk : nblk) - 1 - pslot;
   if (a.pair ? (2 * pslot >= nblk) : (blk_first < 0 || blk_first >= nblk)) return;
   const int n_own = (DP != 256 && a.pair && blk_first != pslot) ? 2 : 1;  // head_dim 256 never pairs (registers)
-  const int off = Lk - Lq;  // causal: col visible iff col <= row + off
+  const int off = a.causal_tl ? 0 : Lk - Lq;  // causal: col visible iff col <= row + off
 
   const unsigned char* qp = a.q + qb + (int64_t)q0 * a.q_ss + (int64_t)h * a.q_sh;
   const unsigned char* kp = a.k + kb + (int64_t)k0 * a.k_ss + (int64_t)hk * a.k_sh;
@@ -206,8 +211,10 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
     vaddr[mb] = v_row * ROWB + (L & 1) * 8 + (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzV<DP>(v_row)) * 16);
-  const float c = a.scale_log2;
-  const float lazy = kLazyLog2 / c;  // threshold in raw-score units
+  // without a bias the scores stay raw and scale * log2(e) is folded into the exponent's FMA; with one they are
+  // moved to the log2 domain when the bias is added, and the factor from there on is 1
+  const float c = BIAS ? 1.0f : a.scale_log2;
+  const float lazy = kLazyLog2 / c;  // threshold in score units
 
   for (int own = 0; own < n_own; ++own) {
   const int m0 = (own == 0 ? blk_first : pslot) * BM;
@@ -244,6 +251,9 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
 
   const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
   const int wave_row_lo = m0 + 32 * wave, wave_row_hi = wave_row_lo + 31;
+  const unsigned char* brow = nullptr;  // this lane's bias row, at its first key group (4 g)
+  if constexpr (BIAS)
+    brow = a.bias + (int64_t)b * a.bias_sb + (int64_t)h * a.bias_sh + (int64_t)min(row, Lq - 1) * a.bias_sq + 8 * g;
 
   auto tile = [&](int j, auto bufc) {
     constexpr int BUF = decltype(bufc)::value;
@@ -283,6 +293,35 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
         if (ks + 2 < KS) {
           ka[ks & 1][0] = *(const s16x8*)(kt + kaddr[ks + 2]);
           ka[ks & 1][1] = *(const s16x8*)(kt + kaddr[ks + 2] + 32 * ROWB);
+        }
+      }
+    }
+
+    // ---- bias: register v of block blk <-> key j BN + 32 blk + 8 (v >> 2) + 4 g + (v & 3) ----
+    if constexpr (BIAS) {
+      const float cs = a.scale_log2;
+      typedef T T4 __attribute__((ext_vector_type(4)));
+      const unsigned char* bt = brow + (int64_t)j * (BN * 2);
+      if (j * BN + BN <= Lk) {
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            const T4 bv = __builtin_bit_cast(T4, *(const u32x2*)(bt + (32 * blk + 8 * q4) * 2));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (blk) s1[4 * q4 + e] = s1[4 * q4 + e] * cs + (float)bv[e] * kLog2e;
+              else s0[4 * q4 + e] = s0[4 * q4 + e] * cs + (float)bv[e] * kLog2e;
+            }
+          }
+      } else {  // last, partial tile: element-wise, columns clamped to the last valid one (masked below anyway)
+        const T* be = (const T*)bt;
+        const int cmax = last_k - j * BN - 4 * g;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int e = 8 * (v >> 2) + (v & 3);
+          s0[v] = s0[v] * cs + (float)be[min(e, cmax)] * kLog2e;
+          s1[v] = s1[v] * cs + (float)be[min(32 + e, cmax)] * kLog2e;
         }
       }
     }
@@ -725,8 +764,16 @@ int validate(const fa_fwd_params* p) {
   if (p->lse_stride_h < 0 || p->lse_stride_s < 0) return FA_ERR_BAD_ARG;
   // the kernels form per-row byte offsets as 32-bit row x 32-bit stride
   if (p->k_stride_s * 2 > 0x7fffffffLL || p->v_stride_s * 2 > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
+  if (p->is_causal < FA_MASK_NONE || p->is_causal > FA_MASK_CAUSAL_TOP_LEFT) return FA_ERR_BAD_ARG;
+  if (p->bias) {
+    if (((uintptr_t)p->bias & 7) || p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_q < 0 ||
+        ((p->bias_stride_b | p->bias_stride_h | p->bias_stride_q) & 3))
+      return FA_ERR_BAD_ARG;
+    if (p->cu_seqlens_q || p->kernel == FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
+  }
   if (p->kernel == FA_KERNEL_SPLITKV) {
     if (p->seqlen_q != 1 || p->heads_q / p->heads_k > 16) return FA_ERR_UNSUPPORTED;
+    if (p->is_causal == FA_MASK_CAUSAL_TOP_LEFT) return FA_ERR_UNSUPPORTED;  // the single query row would see key 0 only
   }
   return FA_OK;
 }
@@ -734,7 +781,10 @@ int validate(const fa_fwd_params* p) {
 void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   int kern = p->kernel;
   const int group = p->heads_q / p->heads_k;
-  if (kern == FA_KERNEL_AUTO) kern = (p->seqlen_q == 1 && group <= 16 && p->seqlen_k >= 256) ? FA_KERNEL_SPLITKV : FA_KERNEL_TILE;
+  if (kern == FA_KERNEL_AUTO)
+    kern = (p->seqlen_q == 1 && group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT)
+               ? FA_KERNEL_SPLITKV
+               : FA_KERNEL_TILE;
   int ns = 1;
   if (kern == FA_KERNEL_SPLITKV) {
     ns = p->num_splits;
@@ -778,6 +828,9 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   a.pair = 0;
   a.n_splits = ns;
   a.is_causal = p->is_causal ? 1 : 0;
+  a.causal_tl = p->is_causal == FA_MASK_CAUSAL_TOP_LEFT ? 1 : 0;
+  a.bias = (const unsigned char*)p->bias;
+  a.bias_sb = p->bias_stride_b * 2; a.bias_sh = p->bias_stride_h * 2; a.bias_sq = p->bias_stride_q * 2;
   a.neg_scale = p->scale < 0.f ? 1 : 0;
   a.scale_log2 = (p->scale < 0.f ? -p->scale : p->scale) * kLog2e;
   // scale == 0: masked scores are -inf and -inf * 0 is NaN; a tiny positive factor keeps -inf masked and maps every
@@ -793,10 +846,10 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   return a;
 }
 
-template <typename T, int DP, int MINB>
+template <typename T, int DP, int MINB, bool BIAS>
 int launch_tile(KArgs a, hipStream_t st) {
   constexpr int lds = 4 * 64 * DP * 2;
-  auto kfn = fa_tile_kernel<T, DP, MINB>;
+  auto kfn = fa_tile_kernel<T, DP, MINB, BIAS>;
   if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
     (void)hipGetLastError();
     return FA_ERR_LAUNCH;
@@ -838,9 +891,14 @@ int dispatch(const KArgs& a, int kern, hipStream_t st) {
     if (dp == 128) return launch_splitkv<T, 128>(a, st);
     return launch_splitkv<T, 256>(a, st);
   }
-  if (dp == 64) return launch_tile<T, 64, 2>(a, st);
-  if (dp == 128) return launch_tile<T, 128, 2>(a, st);
-  return launch_tile<T, 256, 1>(a, st);
+  if (a.bias) {
+    if (dp == 64) return launch_tile<T, 64, 2, true>(a, st);
+    if (dp == 128) return launch_tile<T, 128, 2, true>(a, st);
+    return launch_tile<T, 256, 1, true>(a, st);
+  }
+  if (dp == 64) return launch_tile<T, 64, 2, false>(a, st);
+  if (dp == 128) return launch_tile<T, 128, 2, false>(a, st);
+  return launch_tile<T, 256, 1, false>(a, st);
 }
 
 }  // namespace

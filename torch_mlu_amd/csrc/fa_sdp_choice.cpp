@@ -5,7 +5,8 @@
 // sdp_utils.h:99-472 with their warning texts.  What is not mirrored are the MLU-specific heuristics
 // (sdp_utils.h:475-524: device series, "split condition", "valid data ratio") and the xformers-derived priority order
 // (sdp_utils.cpp:8-53): on MI355X the flash kernels of this build are preferred whenever they are eligible — they
-// take GQA, head dims up to 256, and single-query decode (split-KV) — and everything else is left to PyTorch's own
+// take GQA, head dims up to 256, and single-query decode (split-KV) —, then its mem-efficient entry points (additive
+// attn_mask, top-left causal on non-square problems; inference only), and everything else is left to PyTorch's own
 // choice among its remaining backends.
 #include <ATen/ATen.h>
 #include <ATen/Context.h>
@@ -174,29 +175,94 @@ bool use_flash_attention(const sdp_params& p, bool debug) {
   return true;
 }
 
+bool check_runtime_disabled_mem_efficient(const sdp_params&, bool debug) {
+  if (!at::globalContext().userEnabledMemEfficientSDP()) {
+    if (debug) TORCH_WARN("Memory Efficient attention has been runtime disabled.");
+    return false;
+  }
+  return true;
+}
+
+bool check_head_dim_size_mem_efficient(const sdp_params& p, bool debug) {
+  const int64_t dq = p.query.size(-1), dk = p.key.size(-1), dv = p.value.size(-1);
+  if (!(dq == dk && dq == dv && dq <= 256 && dq >= 8 && dq % 8 == 0)) {
+    if (debug)
+      TORCH_WARN("Mem efficient attention requires query.size(-1)==key.size(-1)==value.size(-1), at most 256.",
+                 " Mem efficient attention requires last dimension of Q/V to be divisible by 8.",
+                 " Got Query.size(-1): ", dq, ", Key.size(-1): ", dk, ", Value.size(-1): ", dv, " instead.");
+    return false;
+  }
+  return true;
+}
+
+// Not in the reference (its mem-efficient path has a backward and dropout): what this build's does not implement.
+bool check_this_build_mem_efficient(const sdp_params& p, bool debug) {
+  if (p.dropout > 0.0) {
+    if (debug) TORCH_WARN("The mem-efficient kernels of this build do not implement dropout (dropout_p must be 0).");
+    return false;
+  }
+  const bool mask_grad = p.attn_mask.has_value() && p.attn_mask->defined() && p.attn_mask->requires_grad();
+  if (input_requires_grad(p) || (at::GradMode::is_enabled() && mask_grad)) {
+    if (debug) TORCH_WARN("The mem-efficient entry points of this build have no backward; a gradient is required.");
+    return false;
+  }
+  if (p.attn_mask.has_value() && p.attn_mask->defined()) {
+    const auto mt = p.attn_mask->scalar_type();
+    if ((mt != at::kBool && mt != p.query.scalar_type()) || p.attn_mask->dim() > 4 || !p.attn_mask->is_cuda() ||
+        p.attn_mask->is_nested()) {
+      if (debug) TORCH_WARN("attn_mask must be a boolean mask or have the dtype of query, at most 4 dimensions, on the HIP device.");
+      return false;
+    }
+  }
+  if (!p.query.is_cuda() || !p.key.is_cuda() || !p.value.is_cuda()) {
+    if (debug) TORCH_WARN("The mem-efficient kernels of this build need all inputs on the HIP device.");
+    return false;
+  }
+  return true;
+}
+
+// use_mem_efficient_attention, sdp_utils.cpp:76-95
+bool use_mem_efficient_attention(const sdp_params& p, bool debug) {
+  constexpr std::array<bool (*)(const sdp_params&, bool), 9> constraints{
+      check_runtime_disabled_mem_efficient, check_not_nested, check_tensor_shapes, check_batch_size_and_num_heads,
+      check_head_dim_size_mem_efficient, check_nonzero_sequence_lengths, check_last_dim_stride_equals_1,
+      check_tensor_dtype, check_this_build_mem_efficient};
+  for (auto c : constraints)
+    if (!c(p, debug)) return false;
+  return true;
+}
+
 SDPBackend select_sdp_backend(const sdp_params& p, std::optional<double> scale) {
   auto& ctx = at::globalContext();
   if (!ctx.userEnabledMathSDP() && !ctx.userEnabledFlashSDP() && !ctx.userEnabledMemEfficientSDP() &&
       !ctx.userEnabledCuDNNSDP())
     return SDPBackend::error;
+  // flash first, then mem-efficient (attn_mask, top-left causal on non-square problems), as the reference's default
+  // order (sdp_utils.cpp:9-12)
   if (use_flash_attention(p, /*debug=*/false)) return SDPBackend::flash_attention;
-  // Not eligible here: PyTorch's own selector decides among what is left.  Its flash choice would land on this build's
-  // registered op again, so flash is masked out while it looks.
-  const bool flash_was = ctx.userEnabledFlashSDP();
-  const bool others = ctx.userEnabledMathSDP() || ctx.userEnabledMemEfficientSDP() || ctx.userEnabledCuDNNSDP();
-  if (others) {
+  if (use_mem_efficient_attention(p, /*debug=*/false)) return SDPBackend::efficient_attention;
+  // Not eligible here: PyTorch's own selector decides among what is left.  Its flash and mem-efficient choices would
+  // land on this build's registered ops again, so both are masked out while it looks.
+  if (ctx.userEnabledMathSDP() || ctx.userEnabledCuDNNSDP()) {
     struct Restore {
       at::Context& c;
-      bool v;
-      ~Restore() { c.setSDPUseFlash(v); }
-    } restore{ctx, flash_was};
+      bool flash, mem;
+      ~Restore() {
+        c.setSDPUseFlash(flash);
+        c.setSDPUseMemEfficient(mem);
+      }
+    } restore{ctx, ctx.userEnabledFlashSDP(), ctx.userEnabledMemEfficientSDP()};
     ctx.setSDPUseFlash(false);
+    ctx.setSDPUseMemEfficient(false);
     const at::AutoDispatchBelowAutograd below;  // skip this file's own registration of the op, reach PyTorch's
     const int64_t choice = at::_fused_sdp_choice(p.query, p.key, p.value, p.attn_mask, p.dropout, p.is_causal, scale,
                                                  p.enable_gqa);
     return static_cast<SDPBackend>(choice);
   }
-  // Only flash is enabled and it cannot take these inputs: say why, as the reference does (sdp_utils.cpp:135-146).
+  // Only fused kernels are enabled and they cannot take these inputs: say why, as the reference does
+  // (sdp_utils.cpp:135-146).
+  TORCH_WARN("Memory efficient kernel not used because:");
+  use_mem_efficient_attention(p, /*debug=*/true);
   TORCH_WARN("Flash attention kernel not used because:");
   use_flash_attention(p, /*debug=*/true);
   TORCH_CHECK(false, "No available kernel.  Aborting execution.");
@@ -214,6 +280,21 @@ int64_t fused_sdp_choice(const at::Tensor& query, const at::Tensor& key, const a
               "No viable backend for scaled_dot_product_attention was found. ",
               "This is likely due to turning off both the math kernel and the fused kernels.");
   return static_cast<int64_t>(backend);
+}
+
+std::string mem_efficient_refusal_reason(const at::Tensor& query, const at::Tensor& key, const at::Tensor& value,
+                                         const std::optional<at::Tensor>& attn_mask, double dropout_p, bool is_causal,
+                                         bool enable_gqa) {
+  const sdp::sdp_params p{query, key, value, attn_mask, dropout_p, is_causal, enable_gqa};
+  if (sdp::use_mem_efficient_attention(p, false)) return "";
+  c10::WarningUtils::WarnAlways always(true);
+  struct Collect : c10::WarningHandler {
+    std::string text;
+    void process(const c10::Warning& w) override { text += w.msg(); }
+  } collect;
+  c10::WarningUtils::WarningHandlerGuard guard(&collect);
+  sdp::use_mem_efficient_attention(p, true);
+  return collect.text.empty() ? "refused" : collect.text;
 }
 
 // Why the flash kernels would refuse these inputs ("" if they take them); used by the tests and for diagnostics.
@@ -254,4 +335,8 @@ TORCH_LIBRARY_FRAGMENT(torch_mlu_amd, m) {
       "_flash_refusal_reason(Tensor query, Tensor key, Tensor value, Tensor? attn_mask=None, float dropout_p=0.0, "
       "bool is_causal=False, bool enable_gqa=False) -> str",
       &torch_mlu_amd::flash_refusal_reason);
+  m.def(
+      "_mem_efficient_refusal_reason(Tensor query, Tensor key, Tensor value, Tensor? attn_mask=None, float dropout_p=0.0, "
+      "bool is_causal=False, bool enable_gqa=False) -> str",
+      &torch_mlu_amd::mem_efficient_refusal_reason);
 }
