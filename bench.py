@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the flash-attention forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask] [--no-extras] [--no-cpu-baseline]
 
 A "step" is one call of the registered op on one batch of seeded synthetic input that is already resident in HBM.
 The headline workload is BASELINE.json configs[1] (causal prefill, bf16 MHA, B=4 H=32 S=4096 D=128); the other
@@ -81,6 +81,23 @@ def make_workload(name, dev):
         return dict(call=call, check=check, flops=10 * B * H * S * S * D / 2, bytes_kv=2 * B * H * S * D * 2,
                     desc=f"backward of causal prefill bf16 B={B} H={H} S={S} D={D}", dtype="bf16", bound="mfma",
                     kernel="fa_bwd_dq_kernel + fa_bwd_dkv_kernel<dK> + fa_bwd_dkv_kernel<dV>")
+    if name == "cfg2_mask":
+        # the mem-efficient entry point on the headline shape: non-causal with an additive [B, 1, S, S] mask that is
+        # broadcast over heads (what F.scaled_dot_product_attention(attn_mask=...) hands to the fused path)
+        B, H, S, D = 4, 32, 4096, 128
+        q, k, v = (seeded((B, H, S, D), 1 + i, bf).to(dev) for i in range(3))
+        bias = seeded((B, 1, S, S), 9, bf, std=1.0).to(dev)
+
+        def call():
+            return aten._scaled_dot_product_efficient_attention(q, k, v, bias, True)
+
+        def check():
+            out, lse = call()[:2]
+            return _check_heads(q, k, v, out, lse, False, [(0, 0), (B - 1, H - 1)], bias=bias)
+
+        return dict(call=call, check=check, flops=4 * B * H * S * S * D, bytes_kv=2 * B * H * S * D * 2,
+                    desc=f"non-causal prefill with additive [B,1,S,S] mask bf16 B={B} H={H} S={S} D={D}", dtype="bf16",
+                    bound="mfma", kernel="fa_tile_kernel<bias>")
     if name == "cfg4":
         g = torch.Generator().manual_seed(3)
         lens = torch.randint(256, 2049, (16,), generator=g).tolist()
@@ -142,13 +159,15 @@ def make_workload(name, dev):
 
 
 @torch.no_grad()
-def _check_heads(q, k, v, out, lse, causal, heads):
+def _check_heads(q, k, v, out, lse, causal, heads, bias=None):
     """max-abs error of sampled (batch, head) pairs against fp32 math on the device."""
     g = q.shape[1] // k.shape[1]
     Sq, Sk, D = q.shape[2], k.shape[2], q.shape[3]
     eo = el = 0.0
     for b, h in heads:
         s = (q[b, h].float() @ k[b, h // g].float().T) / math.sqrt(D)
+        if bias is not None:
+            s = s + bias[b, 0].float()
         if causal:
             r = torch.arange(Sq, device=q.device)[:, None]
             c = torch.arange(Sk, device=q.device)[None, :]
@@ -236,7 +255,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "copy1g"])
+    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask", "copy1g"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -281,7 +300,7 @@ def main():
     main_r = run(args.config, args.steps, args.warmup)
     extras = []
     if not args.no_extras:
-        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd"):
+        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask"):
             if name != args.config:
                 extras.append(run(name, args.steps, args.warmup))
 
@@ -301,7 +320,8 @@ def main():
         "data": "synthetic (seeded N(0, 0.5^2), generated on the CPU in fp32 and cast)",
         "config": {"workload": main_r["workload"], "name": args.config,
                    "entry": {"cfg4": "aten::_flash_attention_forward",
-                             "cfg2_bwd": "aten::_scaled_dot_product_flash_attention_backward"}.get(
+                             "cfg2_bwd": "aten::_scaled_dot_product_flash_attention_backward",
+                             "cfg2_mask": "aten::_scaled_dot_product_efficient_attention"}.get(
                                  args.config, "aten::_scaled_dot_product_flash_attention")},
         "roofline": main_r["roofline"],
         "parity": dict({k: v for k, v in main_r.items() if k.startswith("max_abs_err")},

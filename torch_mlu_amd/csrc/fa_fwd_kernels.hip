@@ -53,6 +53,7 @@ struct KArgs {
   int32_t is_causal;
   int32_t neg_scale;  // scale < 0: Q is negated on load and |scale| is used, so that max() tracks the true row max
   float scale_log2;   // |scale| * log2(e)
+  float scale_abs;    // |scale| (bias path)
   int32_t causal_tl;  // causal mask aligned to the top-left corner (col <= row) instead of the bottom-right one
   const unsigned char* bias;  // optional additive bias, dense mode: [b][h][row][col] through byte strides
   int64_t bias_sb, bias_sh, bias_sq;
@@ -211,9 +212,9 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
     vaddr[mb] = v_row * ROWB + (L & 1) * 8 + (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzV<DP>(v_row)) * 16);
-  // without a bias the scores stay raw and scale * log2(e) is folded into the exponent's FMA; with one they are
-  // moved to the log2 domain when the bias is added, and the factor from there on is 1
-  const float c = BIAS ? 1.0f : a.scale_log2;
+  // without a bias the scores stay raw and scale * log2(e) is folded into the exponent's FMA; with one they become
+  // scale * s + bias when the bias is added, and the factor from there on is log2(e)
+  const float c = BIAS ? kLog2e : a.scale_log2;
   const float lazy = kLazyLog2 / c;  // threshold in score units
 
   for (int own = 0; own < n_own; ++own) {
@@ -270,6 +271,17 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     const unsigned char* kt = smem + BUF * TILE;
     const unsigned char* vt = smem + 2 * TILE + BUF * TILE;
 
+    // bias of a full tile: 8 loads of 4 keys each, issued now and consumed after the S MFMAs
+    const bool full_tile = j * BN + BN <= Lk;
+    u32x2 braw[BIAS ? 8 : 1];
+    if constexpr (BIAS) {
+      if (full_tile) {
+        const unsigned char* bt = brow + (int64_t)j * (BN * 2);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) braw[i] = *(const u32x2*)(bt + (32 * (i >> 2) + 8 * (i & 3)) * 2);
+      }
+    }
+
     // ---- S^T = K Q^T : two 32(kv) x 32(q) blocks; K fragments are fetched two k-steps ahead of their MFMAs ----
     f32x16 s0, s1;
 #pragma unroll
@@ -297,31 +309,31 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
       }
     }
 
-    // ---- bias: register v of block blk <-> key j BN + 32 blk + 8 (v >> 2) + 4 g + (v & 3) ----
+    // ---- bias: register v of block blk <-> key j BN + 32 blk + 8 (v >> 2) + 4 g + (v & 3); scores become
+    //      scale * s + bias (natural units) ----
     if constexpr (BIAS) {
-      const float cs = a.scale_log2;
+      const float cs = a.scale_abs;
       typedef T T4 __attribute__((ext_vector_type(4)));
-      const unsigned char* bt = brow + (int64_t)j * (BN * 2);
-      if (j * BN + BN <= Lk) {
+      if (full_tile) {
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
           for (int q4 = 0; q4 < 4; ++q4) {
-            const T4 bv = __builtin_bit_cast(T4, *(const u32x2*)(bt + (32 * blk + 8 * q4) * 2));
+            const T4 bv = __builtin_bit_cast(T4, braw[4 * blk + q4]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              if (blk) s1[4 * q4 + e] = s1[4 * q4 + e] * cs + (float)bv[e] * kLog2e;
-              else s0[4 * q4 + e] = s0[4 * q4 + e] * cs + (float)bv[e] * kLog2e;
+              if (blk) s1[4 * q4 + e] = s1[4 * q4 + e] * cs + (float)bv[e];
+              else s0[4 * q4 + e] = s0[4 * q4 + e] * cs + (float)bv[e];
             }
           }
       } else {  // last, partial tile: element-wise, columns clamped to the last valid one (masked below anyway)
-        const T* be = (const T*)bt;
+        const T* be = (const T*)(brow + (int64_t)j * (BN * 2));
         const int cmax = last_k - j * BN - 4 * g;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int e = 8 * (v >> 2) + (v & 3);
-          s0[v] = s0[v] * cs + (float)be[min(e, cmax)] * kLog2e;
-          s1[v] = s1[v] * cs + (float)be[min(32 + e, cmax)] * kLog2e;
+          s0[v] = s0[v] * cs + (float)be[min(e, cmax)];
+          s1[v] = s1[v] * cs + (float)be[min(32 + e, cmax)];
         }
       }
     }
@@ -836,6 +848,7 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   // scale == 0: masked scores are -inf and -inf * 0 is NaN; a tiny positive factor keeps -inf masked and maps every
   // finite score to (numerically) zero, which is the scale == 0 answer.
   if (!(a.scale_log2 > 0.f)) a.scale_log2 = 1e-30f;
+  a.scale_abs = a.scale_log2 * kLn2;
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
   if (ws && ns > 1) {
