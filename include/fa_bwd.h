@@ -13,6 +13,7 @@
  *     dV  = P^T dO
  *     dP  = dO V^T,   delta = rowsum(dO o O),   dS = P o (dP - delta)
  *     dQ  = scale * dS K,   dK = scale * dS^T Q
+ * (with dropout: dV = (P o M)^T dO / (1-p) and dP = M o (dO V^T) / (1-p), M regenerated from the forward's seed/offset)
  * with the forward's masking (bottom-right aligned causal) and head grouping (dK, dV of a kv head sum over the
  * query heads that read it).  Same rules as fa_fwd.h: plain C, device pointers, element strides, no allocation,
  * no synchronisation, work is only enqueued on the caller's stream.
@@ -70,6 +71,13 @@ typedef struct fa_bwd_params {
   int32_t dtype;     /* FA_DTYPE_* */
   int32_t is_causal;
   int32_t reserved;  /* must be 0 */
+
+  /* dropout: same p as the forward and the two numbers it stored (device pointers, read by the kernels, so that no
+     host synchronisation is needed); ignored when dropout_p == 0 */
+  float dropout_p;
+  int32_t reserved2; /* must be 0 */
+  const int64_t* philox_seed;
+  const int64_t* philox_offset;
 } fa_bwd_params;
 
 /* Host-only validation: FA_OK or a negative code (FA_ERR_UNSUPPORTED for head_dim > 128). */

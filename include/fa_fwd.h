@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FA_FWD_ABI_VERSION 2
+#define FA_FWD_ABI_VERSION 3
 
 /* element types accepted for q/k/v/out (FlashAttention_internal.cpp:73-80 allows exactly these two) */
 #define FA_DTYPE_FP16 0
@@ -52,7 +52,8 @@ extern "C" {
  *     S   = scale * Q[b,h] K[b,h/(heads_q/heads_k)]^T      (fp32 accumulate)
  *     S  += bias[b,h]                                      (optional additive bias, mem-efficient entry points)
  *     S   = -inf where is_causal and col > row + Lk_b - Lq_b (bottom-right aligned; FA_MASK_CAUSAL_TOP_LEFT: col > row)
- *     LSE = ln sum_j exp(S[:,j]),   out = softmax_row(S) V
+ *     LSE = ln sum_j exp(S[:,j]),   out = softmax_row(S) V      (dropout_p > 0: out = (softmax_row(S) o M) V / (1 - p)
+ *                                                          with a keep-mask M; LSE is that of the undropped S)
  * which is what cnnlFlashAttentionForward_v2 is asked to compute (FlashAttention_internal.cpp:147-161,231-258; with
  * the bias descriptor of the mem-efficient launcher, :585-590,659-686).
  *
@@ -103,6 +104,18 @@ typedef struct fa_fwd_params {
 
   const void* bias;  /* device or NULL */
   int64_t bias_stride_b, bias_stride_h, bias_stride_q;
+
+  /* dropout on the softmax probabilities (tile kernel only; 0 = off).  The mask is a pure function of
+     (philox_seed, philox_offset, sequence, query head, row, col), so the backward regenerates it from the two numbers. */
+  float dropout_p;         /* 0 <= p < 1 */
+  int32_t reserved2;       /* must be 0 */
+  uint64_t philox_seed;
+  uint64_t philox_offset;
+  int64_t* rng_seed_out;   /* device int64 or NULL: the launch stores philox_seed there (the op's philox_seed slot) */
+  int64_t* rng_offset_out; /* device int64 or NULL */
+  void* dropout_mask;      /* device or NULL: debug output, dense [batch][heads_q][seqlen_q][seqlen_k] elements of
+                              `dtype`, +1 kept / -1 dropped, positions outside a sequence or masked left untouched
+                              (dense mode only) */
 } fa_fwd_params;
 
 #define FA_MAX_SPLITS 64

@@ -9,6 +9,7 @@ from .attention_oracle import (  # noqa: F401
     cpu_sdpa_flash,
     default_atol,
     default_rtol,
+    dropout_keep_mask,
     get_tolerances,
     sdpa_backward_oracle,
     sdpa_oracle,

@@ -56,11 +56,15 @@ def construct_local_mask(seqlen_q: int, seqlen_k: int, window_size=(-1, -1)) -> 
 
 
 def attention_ref(q, k, v, scale: Optional[float] = None, causal: bool = False, dtype=np.float64,
-                  attn_bias=None, causal_top_left: bool = False) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
+                  attn_bias=None, causal_top_left: bool = False, dropout_p: float = 0.0, dropout_mask=None
+                  ) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
     """q [B, Sq, Hq, D], k/v [B, Sk, Hk, D]  (the reference oracle's layout, :94-97).
 
     Returns (output [B, Hq, Sq, D], attention [B, Hq, Sq, Sk], lse [B, Hq, Sq]) — the first two are what the
     reference's `attention_ref` returns (:103-105, :161); lse is added.
+
+    `dropout_mask` (True = kept, [B, Hq, Sq, Sk]) and `dropout_p` as in the reference (:85-86, :152-157): the
+    returned attention is the undropped softmax, the output uses attention o mask with v scaled by 1 / (1 - p).
 
     Two additions for the mem-efficient entry points, which the reference's `attention_ref` does not cover (its tests
     compare those against the math backend): `attn_bias`, added to the scaled scores (broadcastable to
@@ -102,12 +106,14 @@ def attention_ref(q, k, v, scale: Optional[float] = None, causal: bool = False, 
     if masked_rows is not None and masked_rows.any():
         attention[:, :, masked_rows, :] = 0.0
         lse[:, :, masked_rows] = np.inf
-    output = np.matmul(attention, vh)                    # einsum("bhts,bshd->bthd") then transpose(1,2)
+    attention_drop = attention if dropout_mask is None else np.where(np.asarray(dropout_mask, dtype=bool), attention, 0.0)
+    output = np.matmul(attention_drop, vh * (1.0 / (1.0 - dropout_p)))  # einsum("bhts,bshd->bthd"), :152-158
     return output, attention, lse
 
 
 def sdpa_oracle(q, k, v, is_causal: bool = False, scale: Optional[float] = None, dtype=np.float64, attn_bias=None,
-                causal_top_left: bool = False) -> Tuple[np.ndarray, np.ndarray]:
+                causal_top_left: bool = False, dropout_p: float = 0.0, dropout_mask=None
+                ) -> Tuple[np.ndarray, np.ndarray]:
     """Dense op layout: q [B, Hq, Sq, D], k/v [B, Hk, Sk, D] -> (out [B, Hq, Sq, D], lse [B, Hq, Sq]).
 
     The [B,H,S,D] -> [B,S,H,D] transposes are the ones the reference's dense wrapper makes
@@ -116,7 +122,7 @@ def sdpa_oracle(q, k, v, is_causal: bool = False, scale: Optional[float] = None,
     q, k, v = _np(q, dtype), _np(k, dtype), _np(v, dtype)
     out, _, lse = attention_ref(q.transpose(0, 2, 1, 3), k.transpose(0, 2, 1, 3), v.transpose(0, 2, 1, 3),
                                 scale=scale, causal=is_causal, dtype=dtype, attn_bias=attn_bias,
-                                causal_top_left=causal_top_left)
+                                causal_top_left=causal_top_left, dropout_p=dropout_p, dropout_mask=dropout_mask)
     return out, lse
 
 
@@ -145,8 +151,8 @@ def varlen_oracle(q, k, v, cu_seqlens_q, cu_seqlens_k, is_causal: bool = False, 
     return out, lse
 
 
-def sdpa_backward_oracle(q, k, v, dout, is_causal: bool = False, scale: Optional[float] = None, dtype=np.float64
-                         ) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
+def sdpa_backward_oracle(q, k, v, dout, is_causal: bool = False, scale: Optional[float] = None, dtype=np.float64,
+                         dropout_p: float = 0.0, dropout_mask=None) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
     """Gradients of the dense op.  q, dout [B, Hq, Sq, D], k/v [B, Hk, Sk, D] -> (dq, dk, dv) with the inputs' shapes.
 
     The reference has no backward oracle of its own — its tests differentiate `attention_ref` with autograd
@@ -154,18 +160,23 @@ def sdpa_backward_oracle(q, k, v, dout, is_causal: bool = False, scale: Optional
         P = softmax(scale Q K^T + mask),  dV = P^T dO,  dP = dO V^T,  dS = P o (dP - rowsum(dO o O)),
         dQ = scale dS K,  dK = scale dS^T Q,
     with dK, dV of a kv head summed over the query heads that read it (the "(h g)" repeat at :119-120 differentiated).
-    Pinned in tests/test_oracle.py against torch.autograd on PyTorch's float64 math SDPA."""
+    With a dropout mask M (True = kept) and r = 1 / (1 - p): dV = (P o M)^T dO r, dP = M o (dO V^T) r, and delta is
+    still rowsum(dO o O) with the dropped-out O.
+    Pinned in tests/test_oracle_backward.py against torch.autograd on PyTorch's float64 math attention."""
     q, k, v, dout = _np(q, dtype), _np(k, dtype), _np(v, dtype), _np(dout, dtype)
     B, Hq, Sq, D = q.shape
     Hk, Sk = k.shape[1], k.shape[2]
     g = Hq // Hk
     sc = (1.0 / math.sqrt(D)) if scale is None else float(scale)
     out, p, _ = attention_ref(q.transpose(0, 2, 1, 3), k.transpose(0, 2, 1, 3), v.transpose(0, 2, 1, 3), scale=scale,
-                              causal=is_causal, dtype=dtype)      # out [B,Hq,Sq,D], p [B,Hq,Sq,Sk]
+                              causal=is_causal, dtype=dtype, dropout_p=dropout_p,
+                              dropout_mask=dropout_mask)           # out [B,Hq,Sq,D], p [B,Hq,Sq,Sk] (undropped)
     kr = np.repeat(k, g, axis=1)
     vr = np.repeat(v, g, axis=1)
-    dv_r = np.matmul(p.transpose(0, 1, 3, 2), dout)                 # [B,Hq,Sk,D]
-    dp = np.matmul(dout, vr.transpose(0, 1, 3, 2))                  # [B,Hq,Sq,Sk]
+    m = np.ones_like(p) if dropout_mask is None else np.asarray(dropout_mask, dtype=dtype)
+    r = 1.0 / (1.0 - dropout_p)
+    dv_r = np.matmul((p * m * r).transpose(0, 1, 3, 2), dout)       # [B,Hq,Sk,D]
+    dp = np.matmul(dout, vr.transpose(0, 1, 3, 2)) * m * r          # [B,Hq,Sq,Sk]
     delta = (dout * out).sum(axis=-1, keepdims=True)
     ds = p * (dp - delta)
     dq = sc * np.matmul(ds, kr)
@@ -193,6 +204,48 @@ def varlen_backward_oracle(q, k, v, dout, cu_seqlens_q, cu_seqlens_k, is_causal:
         dk[k0:k1] = bb[0].transpose(1, 0, 2)
         dv[k0:k1] = cc[0].transpose(1, 0, 2)
     return dq, dk, dv
+
+
+# ---- this build's dropout mask, restated ---------------------------------------------------------------------------
+_M32 = np.uint64(0xFFFFFFFF)
+
+
+def _mix32(h):
+    """murmur3's 32-bit finaliser on uint64 arrays holding 32-bit values."""
+    h = h & _M32
+    h ^= h >> np.uint64(16)
+    h = (h * np.uint64(0x85EBCA6B)) & _M32
+    h ^= h >> np.uint64(13)
+    h = (h * np.uint64(0xC2B2AE35)) & _M32
+    h ^= h >> np.uint64(16)
+    return h
+
+
+def dropout_keep_mask(seed: int, offset: int, bh: int, seqlen_q: int, seqlen_k: int, dropout_p: float) -> np.ndarray:
+    """The keep-mask [seqlen_q, seqlen_k] (True = kept) the HIP kernels use for sequence-and-head index
+    bh = b * heads_q + h of a call with (philox_seed, philox_offset) = (seed, offset).
+
+    The reference's mask comes out of the closed vendor kernel and cannot be reproduced (its tests only ever feed the
+    returned mask back into `attention_ref`, test_scaled_dot_product_attention.py:1049-1070); this restates THIS
+    build's definition so that the tests can check that forward, debug mask and backward all use one and the same
+    mask: one 32-bit word per 2 x 2 patch, word = mix(key ^ row_term(row >> 1) ^ col_term(col >> 1)), element kept
+    iff byte 2 (row & 1) + (col & 1) of the word <= floor((1 - p) * 255)."""
+    u = np.uint64
+    seed, offset = int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1)
+    k = (_mix32(u((seed & 0xFFFFFFFF) ^ 0x2545F491)) + u(seed >> 32)) & _M32
+    k = _mix32(k) ^ u(offset & 0xFFFFFFFF)
+    k = (_mix32(k) + u(offset >> 32)) & _M32
+    key = _mix32(k ^ u((bh * 0x9E3779B1 + 0x7F4A7C15) & 0xFFFFFFFF))
+    rp = (np.arange(seqlen_q, dtype=np.uint64) >> u(1))[:, None]
+    cp = (np.arange(seqlen_k, dtype=np.uint64) >> u(1))[None, :]
+    row_term = ((rp << u(16)) & _M32) ^ (((rp >> u(16)) * u(0x9E3779B1)) & _M32)
+    col_term = (cp & u(0xFFFF)) ^ (((cp >> u(16)) * u(0x7F4A7C15)) & _M32)
+    word = _mix32(key ^ row_term ^ col_term)
+    sel = (u(2) * (np.arange(seqlen_q, dtype=np.uint64) & u(1)))[:, None] + (np.arange(seqlen_k, dtype=np.uint64) & u(1))[None, :]
+    byte = (word >> (u(8) * sel)) & u(0xFF)
+    # the threshold is formed in float32, as the launcher does from its float dropout_p
+    thr = int(np.floor((np.float32(1.0) - np.float32(dropout_p)) * np.float32(255.0)))
+    return byte <= u(thr)
 
 
 def get_tolerances(true_value, computed_value, dtype_name: str, fudge_factor: Optional[float] = 2.0

@@ -93,8 +93,8 @@ def test_device_check_comes_after_dtype_checks_as_in_the_reference():
 def test_unsupported_features_are_refused_loudly():
     q, k, v = _qkv()
     f = torch.ops.torch_mlu_amd._flash_attention_forward
-    with pytest.raises(RuntimeError, match="dropout_p > 0 is not supported"):
-        f(q, k, v, None, None, 8, 8, 0.1, False, False)
+    with pytest.raises(RuntimeError, match=r"dropout_p must be in \[0, 1\)"):
+        f(q, k, v, None, None, 8, 8, 1.0, False, False)
     with pytest.raises(RuntimeError, match="sliding window is not supported"):
         f(q, k, v, None, None, 8, 8, 0.0, False, False, window_size_left=4)
     with pytest.raises(RuntimeError, match="alibi_slopes is not supported"):

@@ -228,9 +228,12 @@ def test_backward_errors():
     q, k, v, do = (t[..., :64].contiguous() for t in (q, k, v, do))
     out, lse, cq, ck, mq, mk, seed, offset, _ = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, 0.0, False,
                                                                                                   False)
-    with pytest.raises(RuntimeError, match="dropout"):
-        torch.ops.aten._scaled_dot_product_flash_attention_backward(do, q, k, v, out, lse, cq, ck, mq, mk, 0.1, False,
+    with pytest.raises(RuntimeError, match="dropout_p must be in"):
+        torch.ops.aten._scaled_dot_product_flash_attention_backward(do, q, k, v, out, lse, cq, ck, mq, mk, 1.5, False,
                                                                     seed, offset)
+    with pytest.raises(RuntimeError, match="int64 device scalars"):
+        torch.ops.aten._scaled_dot_product_flash_attention_backward(do, q, k, v, out, lse, cq, ck, mq, mk, 0.1, False,
+                                                                    seed.cpu(), offset.cpu())
     with pytest.raises(RuntimeError, match="same dtype"):
         torch.ops.aten._scaled_dot_product_flash_attention_backward(do.half(), q, k, v, out, lse, cq, ck, mq, mk, 0.0,
                                                                     False, seed, offset)

@@ -1,0 +1,145 @@
+"""Dropout on the GPU.  The mask of the reference comes out of its closed vendor kernel, so — exactly as the reference's
+own tests do (test/torch_ops/test_scaled_dot_product_attention.py:1049-1110) — parity means: with the mask the op
+returns, out and the gradients equal the oracle's.  On top of that the returned mask must be the documented function of
+(philox_seed, philox_offset, sequence, head, row, col), which is what lets the backward regenerate it."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+import torch_mlu_amd
+from tests._util import lse_close, out_close, seeded
+from torch_mlu_amd import capi
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF, HF = torch.bfloat16, torch.float16
+EPS = {BF: 2.0 ** -8, HF: 2.0 ** -11}
+aten = torch.ops.aten
+
+
+def _inputs(B, Hq, Hk, Sq, Sk, D, dtype, seed):
+    return (seeded((B, Hq, Sq, D), seed, dtype), seeded((B, Hk, Sk, D), seed + 1, dtype),
+            seeded((B, Hk, Sk, D), seed + 2, dtype), seeded((B, Hq, Sq, D), seed + 3, dtype))
+
+
+def _visible(Sq, Sk, causal):
+    i, j = np.arange(Sq)[:, None], np.arange(Sk)[None, :]
+    return (j <= i + Sk - Sq) if causal else np.ones((Sq, Sk), dtype=bool)
+
+
+def _expected_mask(seed, offset, B, Hq, Sq, Sk, p):
+    return np.stack([np.stack([oracle.dropout_keep_mask(seed, offset, b * Hq + h, Sq, Sk, p) for h in range(Hq)])
+                     for b in range(B)])
+
+
+def _grad_check(got, want, dtype):
+    for name, g, w in zip(("dq", "dk", "dv"), got, want):
+        g = g.float().cpu().double().numpy()
+        assert np.isfinite(g).all(), name
+        err = float(np.abs(g - w).max())
+        assert err <= 2.0 * EPS[dtype] * max(float(np.abs(w).max()), 0.25), (name, err)
+
+
+@pytest.mark.parametrize("dtype,D", [(BF, 128), (HF, 64), (HF, 256), (BF, 96)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_forward_and_backward_through_c_abi(dtype, D, causal):
+    for i, (B, Hq, Hk, Sq, Sk, p) in enumerate([(2, 4, 2, 130, 130, 0.1), (1, 2, 2, 257, 65, 0.5), (1, 4, 1, 70, 333, 0.25),
+                                                 (2, 2, 2, 1, 300, 0.3), (1, 2, 2, 64, 64, 0.9)]):
+        q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, dtype, 20 * i)
+        qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
+        seed, offset = 0x1234_5678_9ABC_DEF0 + i, 4 * (i + 1) + (i << 40)
+        rng = torch.zeros(2, dtype=torch.int64, device=DEV)
+        dmask = torch.zeros(B, Hq, Sq, Sk, dtype=dtype, device=DEV)
+        out, lse = capi.fa_forward_dense(qd, kd, vd, is_causal=causal, dropout_p=p, philox_seed=seed,
+                                         philox_offset=offset, rng_out=rng, dropout_mask=dmask)
+        assert rng.tolist() == [seed, offset]
+        keep = _expected_mask(seed, offset, B, Hq, Sq, Sk, p)
+        vis = np.broadcast_to(_visible(Sq, Sk, causal), keep.shape)
+        dm = dmask.float().cpu().numpy()
+        assert ((dm > 0) == (keep & vis)).all() and ((dm < 0) == (~keep & vis)).all()
+        ro, rl = oracle.sdpa_oracle(q, k, v, is_causal=causal, dropout_p=p, dropout_mask=keep)
+        out_close(out.float().cpu().numpy(), ro, dtype, tol=2 * EPS[dtype] * max(1.0, float(np.abs(ro).max())))
+        lse_close(lse.cpu().numpy(), rl, tol=2e-3 if dtype == BF else 1e-3)
+        if D <= 128:
+            got = capi.fa_backward_dense(dod, qd, kd, vd, out, lse, is_causal=causal, dropout_p=p, rng=rng)
+            want = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=causal, dropout_p=p, dropout_mask=keep)
+            _grad_check(got, want, dtype)
+
+
+def test_dense_op_returns_mask_and_state_and_trains():
+    """aten::_scaled_dot_product_flash_attention with dropout: int64 device scalars for seed / offset, a debug mask
+    that is > 0 where kept, reproducible under torch.manual_seed, a fresh mask on the next call; autograd through it
+    regenerates the same mask in the backward."""
+    B, H, S, D, p = 2, 4, 200, 64, 0.2
+    q, k, v, do = _inputs(B, H, H, S, S, D, HF, 5)
+    qd, kd, vd = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    torch.manual_seed(123)
+    n0 = torch_mlu_amd.launch_count()
+    out, lse, cq, ck, mq, mk, seed, offset, dbg = aten._scaled_dot_product_flash_attention(qd, kd, vd, p, True, True)
+    assert seed.is_cuda and seed.dtype == torch.int64 and seed.dim() == 0 and offset.is_cuda and offset.dim() == 0
+    assert dbg.shape == (B, H, S, S) and dbg.dtype == HF
+    assert seed.item() == 123
+    keep = dbg.float().cpu().numpy() > 0
+    vis = np.broadcast_to(_visible(S, S, True), keep.shape)
+    assert (keep == (_expected_mask(seed.item(), offset.item(), B, H, S, S, p) & vis)).all()
+    frac = keep[vis].mean()
+    assert abs(frac - (np.floor(np.float32(0.8) * 255) + 1) / 256) < 5e-3
+    ro, rl = oracle.sdpa_oracle(q, k, v, is_causal=True, dropout_p=p, dropout_mask=keep)
+    out_close(out.detach().float().cpu().numpy(), ro, HF)
+    lse_close(lse.detach().cpu().numpy(), rl)
+    out.backward(do.to(DEV))
+    assert torch_mlu_amd.launch_count() == n0 + 2
+    want = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True, dropout_p=p, dropout_mask=keep)
+    _grad_check((qd.grad, kd.grad, vd.grad), want, HF)
+    # same generator state -> same mask; next call -> another one
+    torch.manual_seed(123)
+    dbg2 = aten._scaled_dot_product_flash_attention(qd.detach(), kd.detach(), vd.detach(), p, True, True)[8]
+    dbg3 = aten._scaled_dot_product_flash_attention(qd.detach(), kd.detach(), vd.detach(), p, True, True)[8]
+    assert torch.equal(dbg2, dbg) and not torch.equal(dbg3, dbg)
+    agree = ((dbg3 > 0) == (dbg > 0))[torch.from_numpy(vis.copy()).to(DEV)].float().mean().item()
+    assert abs(agree - (0.8 ** 2 + 0.2 ** 2)) < 0.01
+
+
+def test_plain_sdpa_with_dropout_trains_on_this_build():
+    q, k, v, _ = _inputs(2, 4, 4, 128, 128, 64, BF, 9)
+    qd, kd, vd = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    n0 = torch_mlu_amd.launch_count()
+    out = F.scaled_dot_product_attention(qd, kd, vd, dropout_p=0.1, is_causal=True)
+    out.float().sum().backward()
+    assert torch_mlu_amd.launch_count() == n0 + 2
+    assert all(torch.isfinite(t.grad).all().item() for t in (qd, kd, vd))
+    # E[out] over masks = the undropped output: the mean over many draws comes close
+    with torch.no_grad():
+        acc = torch.zeros_like(out, dtype=torch.float32)
+        for _ in range(64):
+            acc += F.scaled_dot_product_attention(qd, kd, vd, dropout_p=0.1, is_causal=True).float()
+        ref = F.scaled_dot_product_attention(qd, kd, vd, is_causal=True).float()
+    assert (acc / 64 - ref).abs().mean().item() < 0.02
+
+
+def test_packed_forward_and_backward_with_dropout():
+    lens = [130, 1, 64, 257]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    Hq, Hk, D, p = 4, 2, 128, 0.15
+    T = int(cu[-1])
+    q, k, v, do = (seeded((T, Hq, D), 30, BF), seeded((T, Hk, D), 31, BF), seeded((T, Hk, D), 32, BF),
+                   seeded((T, Hq, D), 33, BF))
+    qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
+    c = torch.from_numpy(cu).to(DEV)
+    torch.manual_seed(7)
+    out, lse, seed, offset, dbg = aten._flash_attention_forward(qd, kd, vd, c, c, max(lens), max(lens), p, True, True)
+    assert dbg.numel() == 0                                  # no debug mask in packed mode
+    dq, dk, dv = aten._flash_attention_backward(dod, qd, kd, vd, out, lse, c, c, max(lens), max(lens), p, True, seed,
+                                                offset)
+    sd, of = seed.item(), offset.item()
+    for b, L in enumerate(lens):
+        s = slice(int(cu[b]), int(cu[b + 1]))
+        keep = np.stack([oracle.dropout_keep_mask(sd, of, b * Hq + h, L, L, p) for h in range(Hq)])[None]
+        args = [t[s].transpose(0, 1)[None] for t in (q, k, v)]
+        ro, _ = oracle.sdpa_oracle(*args, is_causal=True, dropout_p=p, dropout_mask=keep)
+        out_close(out[s].transpose(0, 1)[None].float().cpu().numpy(), ro, BF, tol=3e-2)
+        want = oracle.sdpa_backward_oracle(*args, do[s].transpose(0, 1)[None], is_causal=True, dropout_p=p,
+                                           dropout_mask=keep)
+        _grad_check([t[s].transpose(0, 1)[None] for t in (dq, dk, dv)], want, BF)

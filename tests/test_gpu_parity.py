@@ -386,8 +386,8 @@ def test_errors_on_device_tensors():
         f(q, k[:, :3], v[:, :3])
     with pytest.raises(RuntimeError, match="Key and Value must have the same sequence length"):
         f(q, k, v[:, :, :8])
-    with pytest.raises(RuntimeError, match="dropout_p > 0 is not supported"):
-        f(q, k, v, 0.1)
+    with pytest.raises(RuntimeError, match="dropout_p must be in"):
+        f(q, k, v, 1.0)
     with pytest.raises(RuntimeError, match="contiguous last dimension"):
         f(q.transpose(-1, -2).contiguous().transpose(-1, -2), k, v)
     big = torch.zeros(1, 1, 4, 264, dtype=HF, device=DEV)

@@ -151,3 +151,48 @@ def test_packed_backward_equals_per_sequence_dense():
                           True, None)
         for g, r in zip((dq[qs], dk[ks], dv[ks]), w):
             assert np.abs(g - r[0].transpose(1, 0, 2)).max() < 1e-12
+
+
+# ---- dropout ------------------------------------------------------------------------------------------------------------
+def test_dropout_forward_and_backward_oracle_vs_autograd_float64():
+    """out = ((softmax o M) / (1 - p)) v and its derivative, against autograd on the same expression."""
+    B, Hq, Hk, Sq, Sk, D, p = 2, 4, 2, 13, 21, 8, 0.3
+    q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, seed=90)
+    keep = torch.rand(B, Hq, Sq, Sk, generator=torch.Generator().manual_seed(7)) > p
+    qq, kk, vv = (t.double().clone().requires_grad_() for t in (q, k, v))
+    kr, vr = kk.repeat_interleave(2, 1), vv.repeat_interleave(2, 1)
+    s = torch.matmul(qq, kr.transpose(-1, -2)) / math.sqrt(D)
+    i, j = torch.arange(Sq)[:, None], torch.arange(Sk)[None, :]
+    s = s.masked_fill(j > i + (Sk - Sq), float("-inf"))
+    out = torch.matmul(torch.softmax(s, -1) * keep / (1 - p), vr)
+    out.backward(do.double())
+    o, lse = oracle.sdpa_oracle(q, k, v, is_causal=True, dropout_p=p, dropout_mask=keep.numpy())
+    assert np.abs(o - out.detach().numpy()).max() < 1e-13
+    assert np.abs(lse - torch.logsumexp(s, -1).detach().numpy()).max() < 1e-13      # LSE ignores dropout
+    got = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True, dropout_p=p, dropout_mask=keep.numpy())
+    for g, w in zip(got, (qq.grad, kk.grad, vv.grad)):
+        assert np.abs(g - w.numpy()).max() < 1e-12
+
+
+def test_dropout_mask_restatement_properties():
+    """The mask function: deterministic, the documented keep probability (floor((1-p) 255) + 1) / 256, independent
+    across heads / offsets / seeds, a 2 x 2 patch structure that is invisible in the statistics, and the same value for
+    an element whatever the matrix size."""
+    p = 0.25
+    m = oracle.dropout_keep_mask(42, 4, 0, 512, 768, p)
+    assert (m == oracle.dropout_keep_mask(42, 4, 0, 512, 768, p)).all()
+    assert abs(m.mean() - 192 / 256) < 4e-3
+    small = oracle.dropout_keep_mask(42, 4, 0, 100, 130, p)
+    assert (small == m[:100, :130]).all()
+    for other in (oracle.dropout_keep_mask(42, 4, 1, 512, 768, p), oracle.dropout_keep_mask(42, 8, 0, 512, 768, p),
+                  oracle.dropout_keep_mask(43, 4, 0, 512, 768, p), oracle.dropout_keep_mask(42 + 2 ** 32, 4, 0, 512, 768, p),
+                  oracle.dropout_keep_mask(42, 4 + 2 ** 32, 0, 512, 768, p)):
+        agree = (m == other).mean()
+        assert abs(agree - (0.75 ** 2 + 0.25 ** 2)) < 6e-3
+    # neighbours inside a patch and across patches are uncorrelated
+    for a, b in ((m[:, :-1], m[:, 1:]), (m[:-1], m[1:]), (m[::2, ::2], m[1::2, 1::2]), (m[:-2], m[2:])):
+        assert abs((a & b).mean() - 0.75 ** 2) < 6e-3
+    assert abs(m.mean(axis=0) - 0.75).max() < 0.09 and abs(m.mean(axis=1) - 0.75).max() < 0.08
+    # p = 0 keeps everything; thresholds follow float32 arithmetic
+    assert oracle.dropout_keep_mask(1, 0, 0, 64, 64, 0.0).all()
+    assert abs(oracle.dropout_keep_mask(1, 0, 0, 512, 512, 0.6).mean() - 102 / 256) < 5e-3

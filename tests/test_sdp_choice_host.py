@@ -47,7 +47,8 @@ def test_last_dim_stride():
 def test_attn_mask_dropout_and_non_square_causal():
     q, k, v = _qkv((2, 2, 3, 16))
     assert "Flash Attention does not support non-null attn_mask." in reason(q, k, v, torch.ones(2, 2, 3, 3, dtype=HF))
-    assert "dropout" in reason(q, k, v, None, 0.1)
+    assert "HIP device" in reason(q, k, v, None, 0.1)           # dropout is taken by the flash kernels
+    assert "0 <= dropout_p < 1" in reason(q, k, v, None, 1.0)
     q2, k2, v2 = _qkv((2, 2, 3, 16), size_k=(2, 2, 7, 16))
     assert "top-left" in reason(q2, k2, v2, None, 0.0, True)
     assert "HIP device" in reason(q2, k2, v2, None, 0.0, False)

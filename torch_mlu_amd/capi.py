@@ -77,6 +77,13 @@ class FaFwdParams(ctypes.Structure):
         ("reserved", ctypes.c_int32),
         ("bias", ctypes.c_void_p),
         ("bias_stride_b", ctypes.c_int64), ("bias_stride_h", ctypes.c_int64), ("bias_stride_q", ctypes.c_int64),
+        ("dropout_p", ctypes.c_float),
+        ("reserved2", ctypes.c_int32),
+        ("philox_seed", ctypes.c_uint64),
+        ("philox_offset", ctypes.c_uint64),
+        ("rng_seed_out", ctypes.c_void_p),
+        ("rng_offset_out", ctypes.c_void_p),
+        ("dropout_mask", ctypes.c_void_p),
     ]
 
 
@@ -91,6 +98,8 @@ class FaBwdParams(ctypes.Structure):
         + [(n, ctypes.c_int32) for n in ("batch", "heads_q", "heads_k", "seqlen_q", "seqlen_k", "head_dim")]
         + [("total_q", ctypes.c_int64), ("scale", ctypes.c_float)]
         + [(n, ctypes.c_int32) for n in ("dtype", "is_causal", "reserved")]
+        + [("dropout_p", ctypes.c_float), ("reserved2", ctypes.c_int32), ("philox_seed", ctypes.c_void_p),
+           ("philox_offset", ctypes.c_void_p)]
     )
 
 
@@ -151,7 +160,9 @@ def make_params(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Te
                 cu_seqlens_q: Optional[torch.Tensor] = None, cu_seqlens_k: Optional[torch.Tensor] = None,
                 max_seqlen_q: int = 0, max_seqlen_k: int = 0, scale: Optional[float] = None,
                 is_causal=False, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
-                bias: Optional[torch.Tensor] = None) -> FaFwdParams:
+                bias: Optional[torch.Tensor] = None, dropout_p: float = 0.0, philox_seed: int = 0,
+                philox_offset: int = 0, rng_out: Optional[torch.Tensor] = None,
+                dropout_mask: Optional[torch.Tensor] = None) -> FaFwdParams:
     """Fill a params struct.  `is_causal`: False / True (bottom-right aligned) or one of the FA_MASK_* codes; `bias`:
     a [B, Hq, Sq, Sk] view (dense mode; stride 0 where broadcast) of the inputs' dtype.
 
@@ -197,6 +208,11 @@ def make_params(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Te
         p.bias_stride_b, p.bias_stride_h, p.bias_stride_q = bias.stride(0), bias.stride(1), bias.stride(2)
     else:
         p.bias = None
+    p.dropout_p, p.reserved2 = float(dropout_p), 0
+    p.philox_seed, p.philox_offset = philox_seed, philox_offset
+    p.rng_seed_out = rng_out[0:].data_ptr() if rng_out is not None else None
+    p.rng_offset_out = rng_out[1:].data_ptr() if rng_out is not None else None
+    p.dropout_mask = dropout_mask.data_ptr() if dropout_mask is not None else None
     return p
 
 
@@ -213,32 +229,39 @@ def launch(p: FaFwdParams, device: torch.device) -> None:
 
 def fa_forward_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, is_causal=False,
                      scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
-                     bias: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                     bias: Optional[torch.Tensor] = None, dropout_p: float = 0.0, philox_seed: int = 0,
+                     philox_offset: int = 0, rng_out: Optional[torch.Tensor] = None,
+                     dropout_mask: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """q [B, Hq, Sq, D], k/v [B, Hk, Sk, D] (any strides, contiguous last dim) -> out [B, Hq, Sq, D] (stored
     [B, Sq, Hq, D] like the reference's dense wrapper, attention.cpp:146-148), lse [B, Hq, Sq] fp32.
-    `bias`: anything that expands to [B, Hq, Sq, Sk]; `is_causal` may also be FA_MASK_CAUSAL_TOP_LEFT."""
+    `bias`: anything that expands to [B, Hq, Sq, Sk]; `is_causal` may also be FA_MASK_CAUSAL_TOP_LEFT.
+    Dropout: `dropout_p`, the two numbers that define the mask, `rng_out` (int64[2] on the device, receives them) and
+    `dropout_mask` (zero-initialised [B, Hq, Sq, Sk] of q's dtype, receives +1 kept / -1 dropped)."""
     B, Hq, Sq, D = q.shape
     if bias is not None:
         bias = bias.expand(B, Hq, Sq, k.shape[2])
     out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
     p = make_params(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), out, lse, scale=scale,
-                    is_causal=is_causal, kernel=kernel, num_splits=num_splits, bias=bias)
+                    is_causal=is_causal, kernel=kernel, num_splits=num_splits, bias=bias, dropout_p=dropout_p,
+                    philox_seed=philox_seed, philox_offset=philox_offset, rng_out=rng_out, dropout_mask=dropout_mask)
     launch(p, q.device)
     return out.transpose(1, 2), lse
 
 
 def fa_forward_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor,
                       cu_seqlens_k: torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, *, is_causal: bool = False,
-                      scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO,
-                      num_splits: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+                      scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
+                      dropout_p: float = 0.0, philox_seed: int = 0, philox_offset: int = 0,
+                      rng_out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """q [Tq, Hq, D], k/v [Tk, Hk, D], cu_seqlens int32 [B+1] on the device -> out [Tq, Hq, D], lse [Hq, Tq]."""
     Tq, Hq, D = q.shape
     out = torch.empty((Tq, Hq, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((Hq, Tq), dtype=torch.float32, device=q.device)
     p = make_params(q, k, v, out, lse, cu_seqlens_q=cu_seqlens_q, cu_seqlens_k=cu_seqlens_k,
                     max_seqlen_q=max_seqlen_q, max_seqlen_k=max_seqlen_k, scale=scale, is_causal=is_causal,
-                    kernel=kernel, num_splits=num_splits)
+                    kernel=kernel, num_splits=num_splits, dropout_p=dropout_p, philox_seed=philox_seed,
+                    philox_offset=philox_offset, rng_out=rng_out)
     launch(p, q.device)
     return out, lse
 
@@ -255,7 +278,8 @@ def _set_strides(p, name, t, packed):
 
 
 def fa_backward_dense(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
-                      lse: torch.Tensor, *, is_causal: bool = False, scale: Optional[float] = None
+                      lse: torch.Tensor, *, is_causal: bool = False, scale: Optional[float] = None,
+                      dropout_p: float = 0.0, rng: Optional[torch.Tensor] = None
                       ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """All of dout, q, out [B, Hq, Sq, D] and k, v [B, Hk, Sk, D] (any strides, contiguous last dim), lse [B, Hq, Sq]
     -> (dq, dk, dv) stored [B, S, H, D] and returned as [B, H, S, D] views, like the reference's dense wrapper
@@ -279,12 +303,14 @@ def fa_backward_dense(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: t
     p.total_q = 0
     p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
     p.dtype, p.is_causal, p.reserved = _dtype_code(q.dtype), 1 if is_causal else 0, 0
+    _set_dropout(p, dropout_p, rng)
     _launch_bwd(p, q.device)
     return dq.transpose(1, 2), dk.transpose(1, 2), dv.transpose(1, 2)
 
 
 def fa_backward_packed(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, max_seqlen_k: int, *,
-                       is_causal: bool = False, scale: Optional[float] = None):
+                       is_causal: bool = False, scale: Optional[float] = None, dropout_p: float = 0.0,
+                       rng: Optional[torch.Tensor] = None):
     """Packed: dout, q, out [Tq, Hq, D], k, v [Tk, Hk, D], lse [Hq, Tq] -> (dq, dk, dv) with the inputs' shapes."""
     Tq, Hq, D = q.shape
     dq, dk, dv = torch.empty_like(q, memory_format=torch.contiguous_format), torch.empty_like(
@@ -301,8 +327,16 @@ def fa_backward_packed(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_
     p.seqlen_q, p.seqlen_k, p.head_dim, p.total_q = max_seqlen_q, max_seqlen_k, D, Tq
     p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
     p.dtype, p.is_causal, p.reserved = _dtype_code(q.dtype), 1 if is_causal else 0, 0
+    _set_dropout(p, dropout_p, rng)
     _launch_bwd(p, q.device)
     return dq, dk, dv
+
+
+def _set_dropout(p: FaBwdParams, dropout_p: float, rng: Optional[torch.Tensor]) -> None:
+    """`rng`: the int64[2] device tensor (seed, offset) the forward filled."""
+    p.dropout_p, p.reserved2 = float(dropout_p), 0
+    p.philox_seed = rng[0:].data_ptr() if rng is not None else None
+    p.philox_offset = rng[1:].data_ptr() if rng is not None else None
 
 
 def _launch_bwd(p: FaBwdParams, device: torch.device) -> None:

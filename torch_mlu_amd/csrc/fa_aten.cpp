@@ -19,6 +19,7 @@
 //     FlashAttention_internal.cpp:261-265, which is what the installed PyTorch's shape contract says.
 #include <ATen/ATen.h>
 #include <ATen/hip/HIPContext.h>
+#include <ATen/hip/HIPGeneratorImpl.h>
 #include <c10/hip/HIPGraphsC10Utils.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/core/DeviceGuard.h>
@@ -138,7 +139,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> flash_att
   const bool packed = cum_seq_q.has_value() && cum_seq_q->defined();
   TORCH_CHECK(packed == (cum_seq_k.has_value() && cum_seq_k->defined()),
               "cum_seq_q and cum_seq_k must be given together");
-  TORCH_CHECK(dropout_p == 0.0, "flash attention forward: dropout_p > 0 is not supported by this build");
+  TORCH_CHECK(dropout_p >= 0.0 && dropout_p < 1.0, "flash attention forward: dropout_p must be in [0, 1), got ", dropout_p);
   TORCH_CHECK(!window_size_left.has_value() || *window_size_left < 0, "flash attention forward: sliding window is not supported");
   TORCH_CHECK(!window_size_right.has_value() || *window_size_right < 0 || (is_causal && *window_size_right == 0),
               "flash attention forward: sliding window is not supported");
@@ -191,6 +192,35 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> flash_att
   p.kernel = FA_KERNEL_AUTO;
   p.num_splits = 0;
 
+  // p == 0: the reference returns two uninitialised 0-d int64 tensors (FlashAttention_internal.cpp:211-213); p > 0:
+  // the generator's Philox state, advanced under its mutex (:198-210) — here the kernel stores the two numbers into
+  // the slots, which live on the device as the installed PyTorch's backward expects.
+  at::Tensor seed_t = at::empty({}, q.options().dtype(at::kLong));
+  at::Tensor offset_t = at::empty({}, q.options().dtype(at::kLong));
+  at::Tensor debug_attn_mask = at::empty({0}, q.options());
+  if (dropout_p > 0.0) {
+    TORCH_CHECK(c10::hip::currentStreamCaptureStatusMayInitCtx() == c10::hip::CaptureStatus::None,
+                "flash attention forward: dropout under graph capture is not supported by this build");
+    auto* gen = at::get_generator_or_default<at::CUDAGeneratorImpl>(std::nullopt, at::cuda::detail::getDefaultCUDAGenerator());
+    {
+      std::lock_guard<std::mutex> lock(gen->mutex_);
+      // one call consumes one (seed, offset) pair; the increment only has to keep later consumers off this offset
+      const uint64_t increment = 4 * static_cast<uint64_t>((seqlen_q * seqlen_k + 1023) / 1024 + 1);
+      const at::PhiloxCudaState st = gen->philox_cuda_state(increment);
+      p.philox_seed = st.seed_.val;
+      p.philox_offset = st.offset_.val;
+    }
+    p.dropout_p = static_cast<float>(dropout_p);
+    p.rng_seed_out = seed_t.data_ptr<int64_t>();
+    p.rng_offset_out = offset_t.data_ptr<int64_t>();
+    if (return_debug_mask && !packed) {
+      // [B, H, max_q, max_k], > 0 where kept (the reference: zeros filled by the kernel, :141-146; its tests use
+      // `mask > 0`, test_scaled_dot_product_attention.py:1049-1050)
+      debug_attn_mask = at::zeros({batch, heads, seqlen_q, seqlen_k}, q.options());
+      p.dropout_mask = debug_attn_mask.data_ptr();
+    }
+  }
+
   if (total_q > 0) {
     // workspace: stream-ordered caching allocator, as the reference does (FlashAttention_internal.cpp:215-230)
     const size_t ws_bytes = fa_fwd_workspace_bytes(&p);
@@ -202,12 +232,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> flash_att
     g_launches.fetch_add(1, std::memory_order_relaxed);
   }
 
-  // p == 0: the reference returns two uninitialised 0-d int64 tensors (FlashAttention_internal.cpp:211-213)
-  at::Tensor seed_t = at::empty({}, q.options().dtype(at::kLong));
-  at::Tensor offset_t = at::empty({}, q.options().dtype(at::kLong));
   // return_debug_mask only has an effect with dropout (attention.cpp:178-199)
-  (void)return_debug_mask;
-  at::Tensor debug_attn_mask = at::empty({0}, q.options());
   return std::make_tuple(output, lse, seed_t, offset_t, debug_attn_mask);
 }
 
@@ -289,9 +314,13 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> flash_attention_backward(
     int64_t max_q, int64_t max_k, double dropout_p, bool is_causal, const at::Tensor& philox_seed,
     const at::Tensor& philox_offset, std::optional<double> scale, std::optional<int64_t> window_size_left,
     std::optional<int64_t> window_size_right) {
-  (void)philox_seed;
-  (void)philox_offset;
-  TORCH_CHECK(dropout_p == 0.0, "flash attention backward: dropout_p > 0 is not supported by this build");
+  TORCH_CHECK(dropout_p >= 0.0 && dropout_p < 1.0, "flash attention backward: dropout_p must be in [0, 1), got ", dropout_p);
+  if (dropout_p > 0.0)
+    TORCH_CHECK(philox_seed.defined() && philox_offset.defined() && philox_seed.is_cuda() && philox_offset.is_cuda() &&
+                    philox_seed.scalar_type() == at::kLong && philox_offset.scalar_type() == at::kLong &&
+                    philox_seed.numel() == 1 && philox_offset.numel() == 1,
+                "flash attention backward: philox_seed and philox_offset must be the int64 device scalars the forward "
+                "returned");
   TORCH_CHECK(!window_size_left.has_value() || *window_size_left < 0, "flash attention backward: sliding window is not supported");
   TORCH_CHECK(!window_size_right.has_value() || *window_size_right < 0 || (is_causal && *window_size_right == 0),
               "flash attention backward: sliding window is not supported");
@@ -357,6 +386,11 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> flash_attention_backward(
   p.scale = softmax_scale;
   p.dtype = q.scalar_type() == at::kBFloat16 ? FA_DTYPE_BF16 : FA_DTYPE_FP16;
   p.is_causal = is_causal ? 1 : 0;
+  if (dropout_p > 0.0) {
+    p.dropout_p = static_cast<float>(dropout_p);
+    p.philox_seed = philox_seed.data_ptr<int64_t>();
+    p.philox_offset = philox_offset.data_ptr<int64_t>();
+  }
 
   if (total_q == 0 || k.numel() == 0) {
     dq.zero_(); dk.zero_(); dv.zero_();

@@ -17,6 +17,7 @@
 // S and dP are recomputed in each kernel (7 matrix products per tile pair instead of 5) in exchange for not needing
 // fp32 atomics on dQ.
 #include <hip/hip_runtime.h>
+#include <math.h>
 #include <stdint.h>
 
 #include "fa_bwd.h"
@@ -55,6 +56,10 @@ struct BArgs {
   int32_t is_causal;
   float scale;       // signed softmax scale
   float scale_log2;  // scale * log2(e), signed
+  uint32_t drop_thr;  // dropout: an element was kept iff its byte <= drop_thr
+  float drop_rp;      // 1 / (1 - p)
+  const int64_t* seed_ptr;    // the forward's philox_seed / philox_offset slots (device)
+  const int64_t* offset_ptr;
 };
 
 // One swizzle for tiles that are read both by rows (16 lanes = 16 consecutive rows, same logical chunk) and
@@ -79,7 +84,7 @@ struct TileIO {
 // ---------------------------------------------------------------------------------------------------------
 // dQ kernel
 // ---------------------------------------------------------------------------------------------------------
-template <typename T, int DP>
+template <typename T, int DP, bool DROP>
 __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
   using IO = TileIO<T, DP>;
   constexpr int CPR = IO::CPR, ROWB = IO::ROWB, TILE = IO::TILE, NI = IO::NI, RPI = IO::RPI, KS = IO::KS, MB = IO::MB;
@@ -209,6 +214,11 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
   const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
+  // dropout: the forward's mask, regenerated (same patch words, same lane layout as the forward's scores)
+  uint32_t drop_row = 0;
+  if constexpr (DROP)
+    drop_row = drop_head_key((uint64_t)*a.seed_ptr, (uint64_t)*a.offset_ptr, (uint32_t)bh) ^ drop_row_term((uint32_t)row >> 1);
+  const int drop_sh = 16 * (row & 1);
 
   for (int j = 0; j < ntiles; ++j) {
     const int buf = j & 1;
@@ -236,6 +246,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
     // P^T = exp2(S^T c - LSE), dS^T = P^T (dP^T - delta); masked positions contribute nothing
     const bool need_mask = (j * BN + BN > Lk) || (a.is_causal && j * BN + BN - 1 > wave_row_lo + off);
     const int lim = need_mask ? min(last_k, causal_row_lim) - j * BN - 4 * g : 0x7fffffff;
+    const uint32_t drop_tile = DROP ? (drop_row ^ drop_col_term((uint32_t)(j * (BN / 2) + 2 * g))) : 0u;
     s16x8 dsb[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -243,12 +254,19 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
 #pragma unroll
       for (int e2 = 0; e2 < 4; ++e2) {
         float ds[2];
+        uint32_t word = 0;
+        if constexpr (DROP) {
+          const int v0 = 8 * (t & 1) + 2 * e2;
+          word = drop_mix(drop_tile ^ (uint32_t)(16 * (t >> 1) + 4 * (v0 >> 2) + ((v0 & 3) >> 1))) >> drop_sh;
+        }
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
           const int v = 8 * (t & 1) + 2 * e2 + u;
           const int e = 32 * (t >> 1) + 8 * (v >> 2) + (v & 3);
-          const float sv = (t < 2) ? s0[v] : s1[v], dpv = (t < 2) ? p0[v] : p1[v];
+          const float sv = (t < 2) ? s0[v] : s1[v];
+          float dpv = (t < 2) ? p0[v] : p1[v];
           const float p = (e <= lim) ? fast_exp2(sv * c - lse2) : 0.f;
+          if constexpr (DROP) dpv = (((word >> (8 * u)) & 0xffu) <= a.drop_thr) ? dpv * a.drop_rp : 0.f;
           ds[u] = p * (dpv - delta);
         }
         w[e2] = Mma<T>::pack2(ds[0], ds[1]);
@@ -293,7 +311,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
 // more); with head_dim <= 64 one launch produces both.
 constexpr int kDK = 1, kDV = 2;
 
-template <typename T, int DP, int WHAT>
+template <typename T, int DP, int WHAT, bool DROP>
 __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
   constexpr bool DO_K = (WHAT & kDK) != 0, DO_V = (WHAT & kDV) != 0;
   using IO = TileIO<T, DP>;
@@ -362,6 +380,14 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
 
   const int n0 = pslot * BKV;
   const int kvrow = n0 + 32 * wave + c32;  // this lane's key row
+  // dropout: column term of this lane's key, and which byte pair of a patch word belongs to it
+  const uint32_t drop_col = DROP ? drop_col_term((uint32_t)kvrow >> 1) : 0u;
+  const int drop_sh = 8 * (kvrow & 1);
+  uint64_t drop_seed = 0, drop_offset = 0;
+  if constexpr (DROP) {
+    drop_seed = (uint64_t)*a.seed_ptr;
+    drop_offset = (uint64_t)*a.offset_ptr;
+  }
   const int wave_kv_lo = n0 + 32 * wave;
   // query tiles that can see this key block: rows q with q + off >= n0
   int jq_begin = 0;
@@ -429,6 +455,12 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     const int qlo = jq * BQ;
     // every (q, kv) of this tile masked for this wavefront: q + off < kv for all pairs
     if (a.is_causal && qlo + BQ - 1 + off < wave_kv_lo) continue;
+    // dropout: key of this iteration's query head ^ column term ^ row term of the tile's first row pair (+ 2 g);
+    // the row pair of registers (v, v + 1) adds a compile-time constant with disjoint bits
+    uint32_t drop_tile = 0;
+    if constexpr (DROP)
+      drop_tile = drop_head_key(drop_seed, drop_offset, (uint32_t)(b * a.heads_q + hk * a.group + it / nq)) ^ drop_col ^
+                  drop_row_term((uint32_t)(qlo / 2 + 2 * g));
 
     const unsigned char* qt = smem + buf * TILE;
     const unsigned char* dt = smem + 2 * TILE + buf * TILE;
@@ -470,8 +502,19 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
             p0 = ok0 ? p0 : 0.f;
             p1 = ok1 ? p1 : 0.f;
           }
-          if constexpr (DO_V) wp[e2] = Mma<T>::pack2(p0, p1);
-          if constexpr (DO_K) wd[e2] = Mma<T>::pack2(p0 * (dp[v] - d0), p1 * (dp[v + 1] - d1));
+          float dp0 = DO_K ? dp[v] : 0.f, dp1 = DO_K ? dp[v + 1] : 0.f;
+          float pv0 = p0, pv1 = p1;  // what multiplies dO in dV: P o M / (1 - p)
+          if constexpr (DROP) {
+            const uint32_t rp_const = 16 * qbk + 4 * (v >> 2) + ((v & 3) >> 1);
+            const uint32_t word = drop_mix(drop_tile ^ (rp_const << 16)) >> drop_sh;
+            const bool k0 = (word & 0xffu) <= a.drop_thr, k1 = ((word >> 16) & 0xffu) <= a.drop_thr;
+            pv0 = k0 ? p0 * a.drop_rp : 0.f;
+            pv1 = k1 ? p1 * a.drop_rp : 0.f;
+            dp0 = k0 ? dp0 * a.drop_rp : 0.f;
+            dp1 = k1 ? dp1 * a.drop_rp : 0.f;
+          }
+          if constexpr (DO_V) wp[e2] = Mma<T>::pack2(pv0, pv1);
+          if constexpr (DO_K) wd[e2] = Mma<T>::pack2(p0 * (dp0 - d0), p1 * (dp1 - d1));
         }
         pb[t] = __builtin_bit_cast(s16x8, wp);
         dsb[t] = __builtin_bit_cast(s16x8, wd);
@@ -533,7 +576,11 @@ int bwd_validate(const fa_bwd_params* p) {
   if ((p->cu_seqlens_q == nullptr) != (p->cu_seqlens_k == nullptr)) return FA_ERR_BAD_ARG;
   if (p->batch <= 0 || p->heads_q <= 0 || p->heads_k <= 0) return FA_ERR_BAD_ARG;
   if (p->seqlen_q < 0 || p->seqlen_k < 0 || p->head_dim <= 0) return FA_ERR_BAD_ARG;
-  if (p->reserved != 0) return FA_ERR_BAD_ARG;
+  if (p->reserved != 0 || p->reserved2 != 0) return FA_ERR_BAD_ARG;
+  if (!(p->dropout_p >= 0.f && p->dropout_p < 1.f)) return FA_ERR_BAD_ARG;
+  if (p->dropout_p > 0.f && (!p->philox_seed || !p->philox_offset ||
+                             (((uintptr_t)p->philox_seed | (uintptr_t)p->philox_offset) & 7)))
+    return FA_ERR_BAD_ARG;
   if (p->cu_seqlens_q && p->total_q < 0) return FA_ERR_BAD_ARG;
   if (p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_UNSUPPORTED;
   if (p->head_dim > 128 || (p->head_dim & 7)) return FA_ERR_UNSUPPORTED;
@@ -565,14 +612,14 @@ size_t bwd_ws_bytes(const fa_bwd_params* p) {
   return (rows * p->heads_q * 4 + 15) & ~(size_t)15;
 }
 
-template <typename T, int DP>
+template <typename T, int DP, bool DROP>
 int bwd_launch(const BArgs& a, hipStream_t st) {
   constexpr int lds_dq = 4 * 64 * DP * 2;
   constexpr int lds_dkv = 4 * 64 * DP * 2 + 4 * 256;
   constexpr bool split = DP > 64;  // head_dim 128: dK and dV as two launches
-  auto kq = fa_bwd_dq_kernel<T, DP>;
-  auto kkv = fa_bwd_dkv_kernel<T, DP, split ? kDK : (kDK | kDV)>;
-  auto kv2 = fa_bwd_dkv_kernel<T, DP, kDV>;
+  auto kq = fa_bwd_dq_kernel<T, DP, DROP>;
+  auto kkv = fa_bwd_dkv_kernel<T, DP, split ? kDK : (kDK | kDV), DROP>;
+  auto kv2 = fa_bwd_dkv_kernel<T, DP, kDV, DROP>;
   if (hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dq) != hipSuccess ||
       hipFuncSetAttribute((const void*)kkv, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv) != hipSuccess ||
       (split && hipFuncSetAttribute((const void*)kv2, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv) != hipSuccess)) {
@@ -640,10 +687,21 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   a.n_kslot = (p->seqlen_k + 127) / 128;
   a.scale = p->scale;
   a.scale_log2 = p->scale * kLog2e;
+  const float p_keep = 1.f - p->dropout_p;
+  a.drop_thr = (uint32_t)floorf(p_keep * 255.f);
+  a.drop_rp = 1.f / p_keep;
+  a.seed_ptr = p->philox_seed;
+  a.offset_ptr = p->philox_offset;
   hipStream_t st = (hipStream_t)stream;
   const int dp = p->head_dim <= 64 ? 64 : 128;
-  if (p->dtype == FA_DTYPE_BF16) return dp == 64 ? bwd_launch<__bf16, 64>(a, st) : bwd_launch<__bf16, 128>(a, st);
-  return dp == 64 ? bwd_launch<_Float16, 64>(a, st) : bwd_launch<_Float16, 128>(a, st);
+  if (p->dropout_p > 0.f) {
+    if (p->dtype == FA_DTYPE_BF16)
+      return dp == 64 ? bwd_launch<__bf16, 64, true>(a, st) : bwd_launch<__bf16, 128, true>(a, st);
+    return dp == 64 ? bwd_launch<_Float16, 64, true>(a, st) : bwd_launch<_Float16, 128, true>(a, st);
+  }
+  if (p->dtype == FA_DTYPE_BF16)
+    return dp == 64 ? bwd_launch<__bf16, 64, false>(a, st) : bwd_launch<__bf16, 128, false>(a, st);
+  return dp == 64 ? bwd_launch<_Float16, 64, false>(a, st) : bwd_launch<_Float16, 128, false>(a, st);
 }
 
 }  // extern "C"

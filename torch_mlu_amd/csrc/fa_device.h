@@ -106,6 +106,31 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return r;
 }
 
+// ---- dropout ---------------------------------------------------------------------------------------------
+// One 32-bit word per 2 x 2 patch of the attention matrix of one (sequence, query head); element (row, col) keeps its
+// probability iff byte 2 (row & 1) + (col & 1) of the patch's word is <= the threshold.  The word is a murmur3
+// finaliser over a counter that is unique per patch while both pair indices are below 65536 (beyond that the high
+// parts are folded in), so forward and backward — whose lanes own different elements — regenerate the same mask from
+// (seed, offset, sequence, head, row, col) alone.
+__device__ __forceinline__ uint32_t drop_mix(uint32_t h) {
+  h ^= h >> 16;
+  h *= 0x85ebca6bu;
+  h ^= h >> 13;
+  h *= 0xc2b2ae35u;
+  h ^= h >> 16;
+  return h;
+}
+// key of one (sequence b, query head h) of one call: bh = b * heads_q + h
+__device__ __forceinline__ uint32_t drop_head_key(uint64_t seed, uint64_t offset, uint32_t bh) {
+  uint32_t k = drop_mix((uint32_t)seed ^ 0x2545f491u) + (uint32_t)(seed >> 32);
+  k = drop_mix(k) ^ (uint32_t)offset;
+  k = drop_mix(k) + (uint32_t)(offset >> 32);
+  return drop_mix(k ^ (bh * 0x9e3779b1u + 0x7f4a7c15u));
+}
+// the part of a patch's counter that depends on its row pair / on its column pair; the counter is their XOR with the key
+__device__ __forceinline__ uint32_t drop_row_term(uint32_t rowpair) { return (rowpair << 16) ^ ((rowpair >> 16) * 0x9e3779b1u); }
+__device__ __forceinline__ uint32_t drop_col_term(uint32_t colpair) { return (colpair & 0xffffu) ^ ((colpair >> 16) * 0x7f4a7c15u); }
+
 }  // namespace fa
 
 #endif  // FA_DEVICE_H_

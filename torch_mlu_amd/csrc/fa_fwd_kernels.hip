@@ -57,6 +57,12 @@ struct KArgs {
   int32_t causal_tl;  // causal mask aligned to the top-left corner (col <= row) instead of the bottom-right one
   const unsigned char* bias;  // optional additive bias, dense mode: [b][h][row][col] through byte strides
   int64_t bias_sb, bias_sh, bias_sq;
+  uint32_t drop_thr;  // dropout: an element is kept iff its byte <= drop_thr
+  float drop_rp;      // 1 / (1 - p)
+  uint64_t seed, offset;
+  int64_t* rng_seed_out;
+  int64_t* rng_offset_out;
+  unsigned char* dmask;  // debug mask [batch][heads_q][seqlen_q][seqlen_k] elements, or null
   float* ws_o;        // split-KV partials: [batch*heads_q*n_splits][head_dim] fp32, unnormalised
   float* ws_ml;       // [batch*heads_q*n_splits][2]: m (log2 domain), l
 };
@@ -88,7 +94,9 @@ constexpr float kLazyLog2 = 8.0f;
 
 // BIAS: an additive bias tile is read straight from global memory into the score layout (one lane = one query row,
 // groups of 4 consecutive keys = 8 bytes) and the softmax then runs on scores already in the log2 domain.
-template <typename T, int DP, int MINB, bool BIAS>
+// DROP: dropout on the probabilities.  The row sums (and LSE) are those of the undropped probabilities; dropped
+// entries are zeroed in the P operand of the PV product and 1 / (1 - p) is folded into the final normalisation.
+template <typename T, int DP, int MINB, bool BIAS, bool DROP = false>
 __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   constexpr int CPR = DP / 8;          // 16-byte chunks per row
   constexpr int ROWB = DP * 2;         // bytes per LDS row
@@ -126,6 +134,14 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   }
   const int h = bh % a.heads_q, b = bh / a.heads_q;
   const int hk = h / a.group;
+  uint32_t drop_key = 0;
+  if constexpr (DROP) {
+    drop_key = drop_head_key(a.seed, a.offset, (uint32_t)bh);
+    if (blockIdx.x == 0 && tid == 0) {
+      if (a.rng_seed_out) *a.rng_seed_out = (int64_t)a.seed;
+      if (a.rng_offset_out) *a.rng_offset_out = (int64_t)a.offset;
+    }
+  }
 
   int q0 = 0, k0 = 0, Lq = a.seqlen_q, Lk = a.seqlen_k;
   int64_t qb = (int64_t)b * a.q_sb, kb = (int64_t)b * a.k_sb, vb = (int64_t)b * a.v_sb, ob = (int64_t)b * a.o_sb;
@@ -252,7 +268,13 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
 
   const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
   const int wave_row_lo = m0 + 32 * wave, wave_row_hi = wave_row_lo + 31;
+  // dropout: key ^ row term of this lane's row pair, and which half of a patch word belongs to this row
+  const uint32_t drop_row = DROP ? (drop_key ^ drop_row_term((uint32_t)row >> 1)) : 0u;
+  const int drop_sh = 16 * (row & 1);
   const unsigned char* brow = nullptr;  // this lane's bias row, at its first key group (4 g)
+  unsigned char* drow = nullptr;  // this lane's row of the debug mask
+  if constexpr (DROP)
+    if (a.dmask) drow = a.dmask + (((int64_t)b * a.heads_q + h) * a.seqlen_q + min(row, Lq - 1)) * (int64_t)a.seqlen_k * 2;
   if constexpr (BIAS)
     brow = a.bias + (int64_t)b * a.bias_sb + (int64_t)h * a.bias_sh + (int64_t)min(row, Lq - 1) * a.bias_sq + 8 * g;
 
@@ -371,6 +393,9 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
         for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
     }
     const float mc = (m_run == -INFINITY) ? 0.f : m_run * c;
+    // dropout: counter of a patch = key ^ row term ^ column term; the column pair of this lane's groups is
+    // 32 j + 2 g + a compile-time constant with disjoint bits
+    const uint32_t drop_tile = DROP ? (drop_row ^ drop_col_term((uint32_t)(j * (BN / 2) + 2 * g))) : 0u;
 
     // ---- per 16-key chunk t: P = exp2(S c - m c), row sums, P^T as B operand, O^T += V^T P^T.  The V^T fragments
     //      of chunk t + 1 are fetched while chunk t's MFMAs run. ----
@@ -394,8 +419,24 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
       for (int e2 = 0; e2 < 4; ++e2) {
         const int v = 8 * (t & 1) + 2 * e2;
         const float x0 = (t < 2) ? s0[v] : s1[v], x1 = (t < 2) ? s0[v + 1] : s1[v + 1];
-        const float p0 = fast_exp2(x0 * c - mc), p1 = fast_exp2(x1 * c - mc);
+        float p0 = fast_exp2(x0 * c - mc), p1 = fast_exp2(x1 * c - mc);
         rs += p0 + p1;
+        if constexpr (DROP) {
+          // keys j BN + 32 (t >> 1) + 8 (v >> 2) + 4 g + (v & 3), + 1: one column pair, one patch word
+          const uint32_t cp_const = 16 * (t >> 1) + 4 * (v >> 2) + ((v & 3) >> 1);
+          const uint32_t word = drop_mix(drop_tile ^ cp_const) >> drop_sh;
+          const bool k0 = (word & 0xffu) <= a.drop_thr, k1 = ((word >> 8) & 0xffu) <= a.drop_thr;
+          if (a.dmask) {
+            const int col = j * BN + 32 * (t >> 1) + 8 * (v >> 2) + 4 * g + (v & 3);
+            if (row < Lq && col + 1 <= min(last_k, causal_row_lim)) {
+              *(unsigned*)(drow + (int64_t)col * 2) = Mma<T>::pack2(k0 ? 1.f : -1.f, k1 ? 1.f : -1.f);
+            } else if (row < Lq && col <= min(last_k, causal_row_lim)) {
+              *(T*)(drow + (int64_t)col * 2) = (T)(k0 ? 1.f : -1.f);
+            }
+          }
+          p0 = k0 ? p0 : 0.f;
+          p1 = k1 ? p1 : 0.f;
+        }
         w[e2] = Mma<T>::pack2(p0, p1);
       }
       const s16x8 pb = __builtin_bit_cast(s16x8, w);
@@ -416,7 +457,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
 
   // ---- epilogue ----
   l_run = pair_sum32(l_run);
-  const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
+  const float inv = (l_run > 0.f) ? (DROP ? a.drop_rp : 1.f) / l_run : 0.f;
   if (row < Lq) {
     unsigned char* orow = a.out + ob + (int64_t)(q0 + row) * a.o_ss + (int64_t)h * a.o_sh;
 #pragma unroll
@@ -777,6 +818,12 @@ int validate(const fa_fwd_params* p) {
   // the kernels form per-row byte offsets as 32-bit row x 32-bit stride
   if (p->k_stride_s * 2 > 0x7fffffffLL || p->v_stride_s * 2 > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
   if (p->is_causal < FA_MASK_NONE || p->is_causal > FA_MASK_CAUSAL_TOP_LEFT) return FA_ERR_BAD_ARG;
+  if (p->reserved2 != 0 || !(p->dropout_p >= 0.f && p->dropout_p < 1.f)) return FA_ERR_BAD_ARG;
+  if (p->dropout_p > 0.f) {
+    if (p->bias || p->kernel == FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
+    if (p->dropout_mask && (p->cu_seqlens_q || ((uintptr_t)p->dropout_mask & 3))) return FA_ERR_UNSUPPORTED;
+    if (((uintptr_t)p->rng_seed_out | (uintptr_t)p->rng_offset_out) & 7) return FA_ERR_BAD_ARG;
+  }
   if (p->bias) {
     if (((uintptr_t)p->bias & 7) || p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_q < 0 ||
         ((p->bias_stride_b | p->bias_stride_h | p->bias_stride_q) & 3))
@@ -794,7 +841,8 @@ void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   int kern = p->kernel;
   const int group = p->heads_q / p->heads_k;
   if (kern == FA_KERNEL_AUTO)
-    kern = (p->seqlen_q == 1 && group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT)
+    kern = (p->seqlen_q == 1 && group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT &&
+            !(p->dropout_p > 0.f))
                ? FA_KERNEL_SPLITKV
                : FA_KERNEL_TILE;
   int ns = 1;
@@ -849,6 +897,12 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   // finite score to (numerically) zero, which is the scale == 0 answer.
   if (!(a.scale_log2 > 0.f)) a.scale_log2 = 1e-30f;
   a.scale_abs = a.scale_log2 * kLn2;
+  const float p_keep = 1.f - p->dropout_p;
+  a.drop_thr = (uint32_t)floorf(p_keep * 255.f);
+  a.drop_rp = 1.f / p_keep;
+  a.seed = p->philox_seed; a.offset = p->philox_offset;
+  a.rng_seed_out = p->rng_seed_out; a.rng_offset_out = p->rng_offset_out;
+  a.dmask = (unsigned char*)p->dropout_mask;
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
   if (ws && ns > 1) {
@@ -859,10 +913,10 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   return a;
 }
 
-template <typename T, int DP, int MINB, bool BIAS>
+template <typename T, int DP, int MINB, bool BIAS, bool DROP = false>
 int launch_tile(KArgs a, hipStream_t st) {
   constexpr int lds = 4 * 64 * DP * 2;
-  auto kfn = fa_tile_kernel<T, DP, MINB, BIAS>;
+  auto kfn = fa_tile_kernel<T, DP, MINB, BIAS, DROP>;
   if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
     (void)hipGetLastError();
     return FA_ERR_LAUNCH;
@@ -903,6 +957,11 @@ int dispatch(const KArgs& a, int kern, hipStream_t st) {
     if (dp == 64) return launch_splitkv<T, 64>(a, st);
     if (dp == 128) return launch_splitkv<T, 128>(a, st);
     return launch_splitkv<T, 256>(a, st);
+  }
+  if (a.drop_thr < 255u) {  // dropout_p > 0
+    if (dp == 64) return launch_tile<T, 64, 2, false, true>(a, st);
+    if (dp == 128) return launch_tile<T, 128, 2, false, true>(a, st);
+    return launch_tile<T, 256, 1, false, true>(a, st);
   }
   if (a.bias) {
     if (dp == 64) return launch_tile<T, 64, 2, true>(a, st);

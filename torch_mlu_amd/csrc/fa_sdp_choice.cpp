@@ -145,8 +145,8 @@ bool check_tensor_dtype(const sdp_params& p, bool debug) {
 // Not in the reference: what this build's flash kernels do not implement, and the one place where the flash
 // convention differs from F.scaled_dot_product_attention's definition.
 bool check_this_build(const sdp_params& p, bool debug) {
-  if (p.dropout > 0.0) {
-    if (debug) TORCH_WARN("The flash kernels of this build do not implement dropout (dropout_p must be 0).");
+  if (!(p.dropout >= 0.0 && p.dropout < 1.0)) {
+    if (debug) TORCH_WARN("The flash kernels of this build need 0 <= dropout_p < 1.");
     return false;
   }
   if (p.is_causal && p.query.size(-2) != p.key.size(-2)) {
