@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the flash-attention forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop] [--no-extras] [--no-cpu-baseline]
 
 A "step" is one call of the registered op on one batch of seeded synthetic input that is already resident in HBM.
 The headline workload is BASELINE.json configs[1] (causal prefill, bf16 MHA, B=4 H=32 S=4096 D=128); the other
@@ -30,9 +30,11 @@ PEAK_HBM_GBS = 8000.0
 # their commands are recorded under profiles/.  Counters cannot be read from inside a timed run, so these are the
 # recorded values (None: not profiled).
 TRAFFIC_BYTES = {
-    "cfg2": int((522.1 + 130.0) * 2 ** 20),
+    "cfg2": int((521.9 + 130.0) * 2 ** 20),
     "cfg5": int(2.0021 * 2 ** 30 + 4.25 * 2 ** 20),
-    "cfg2_bwd": int((1701.8 + 386.1) * 2 ** 20),  # the three launches of one backward together
+    "cfg2_bwd": int((1702.7 + 386.1) * 2 ** 20),  # the three launches of one backward together
+    "cfg2_mask": int(2.96 * 2 ** 30 + 228.8 * 2 ** 20),
+    "cfg2_drop": int((641.4 + 195.7) * 2 ** 20),
 }
 
 
@@ -81,6 +83,21 @@ def make_workload(name, dev):
         return dict(call=call, check=check, flops=10 * B * H * S * S * D / 2, bytes_kv=2 * B * H * S * D * 2,
                     desc=f"backward of causal prefill bf16 B={B} H={H} S={S} D={D}", dtype="bf16", bound="mfma",
                     kernel="fa_bwd_dq_kernel + fa_bwd_dkv_kernel<dK> + fa_bwd_dkv_kernel<dV>")
+    if name == "cfg2_drop":
+        # the headline workload with dropout_p = 0.1 (training-time forward)
+        B, H, S, D, pd = 4, 32, 4096, 128, 0.1
+        q, k, v = (seeded((B, H, S, D), 1 + i, bf).to(dev) for i in range(3))
+
+        def call():
+            return aten._scaled_dot_product_flash_attention(q, k, v, pd, True, False)
+
+        def check():
+            r = aten._scaled_dot_product_flash_attention(q, k, v, pd, True, True)
+            return _check_heads(q, k, v, r[0], r[1], True, [(0, 0), (B - 1, H - 1)], keep=r[8] > 0, dropout_p=pd)
+
+        return dict(call=call, check=check, flops=4 * B * H * S * S * D / 2, bytes_kv=2 * B * H * S * D * 2,
+                    desc=f"causal prefill with dropout 0.1 bf16 B={B} H={H} S={S} D={D}", dtype="bf16", bound="mfma",
+                    kernel="fa_tile_kernel<dropout>")
     if name == "cfg2_mask":
         # the mem-efficient entry point on the headline shape: non-causal with an additive [B, 1, S, S] mask that is
         # broadcast over heads (what F.scaled_dot_product_attention(attn_mask=...) hands to the fused path)
@@ -159,7 +176,7 @@ def make_workload(name, dev):
 
 
 @torch.no_grad()
-def _check_heads(q, k, v, out, lse, causal, heads, bias=None):
+def _check_heads(q, k, v, out, lse, causal, heads, bias=None, keep=None, dropout_p=0.0):
     """max-abs error of sampled (batch, head) pairs against fp32 math on the device."""
     g = q.shape[1] // k.shape[1]
     Sq, Sk, D = q.shape[2], k.shape[2], q.shape[3]
@@ -173,7 +190,10 @@ def _check_heads(q, k, v, out, lse, causal, heads, bias=None):
             c = torch.arange(Sk, device=q.device)[None, :]
             s.masked_fill_(c > r + Sk - Sq, float("-inf"))
         l = torch.logsumexp(s, -1)
-        o = torch.exp(s - l[:, None]) @ v[b, h // g].float()
+        pm = torch.exp(s - l[:, None])
+        if keep is not None:
+            pm = pm * keep[b, h] / (1.0 - dropout_p)
+        o = pm @ v[b, h // g].float()
         eo = max(eo, (out[b, h].float() - o).abs().max().item())
         el = max(el, (lse[b, h] - l).abs().max().item())
     return eo, el
@@ -255,7 +275,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask", "copy1g"])
+    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "copy1g"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -300,7 +320,7 @@ def main():
     main_r = run(args.config, args.steps, args.warmup)
     extras = []
     if not args.no_extras:
-        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask"):
+        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask", "cfg2_drop"):
             if name != args.config:
                 extras.append(run(name, args.steps, args.warmup))
 
