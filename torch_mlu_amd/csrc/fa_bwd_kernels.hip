@@ -54,6 +54,9 @@ struct BArgs {
   int32_t seqlen_q, seqlen_k, head_dim;
   int32_t n_qslot, n_kslot;  // workgroups per (sequence, head) of the dQ kernel / per (sequence, kv head) of the dK/dV kernel
   int32_t is_causal;
+  // causal problems with few workgroups per CU: heads of an XCD's range interleaved, heaviest block index first
+  // (better balance); otherwise head after head (better L2 reuse)
+  int32_t blockmajor_q, blockmajor_k;
   float scale;       // signed softmax scale
   float scale_log2;  // scale * log2(e), signed
   uint32_t drop_thr;  // dropout: an element was kept iff its byte <= drop_thr
@@ -107,9 +110,17 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
     bh = lid % nbh;
   } else {
     const int per = gridDim.x >> 3;
-    if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
-    pslot = lid % a.n_qslot;
-    bh = lid / a.n_qslot;
+    const int nh = per / a.n_qslot;  // whole heads per XCD range
+    if (a.blockmajor_q && lid < (per << 3) && nh * a.n_qslot == per) {
+      // within an XCD's range run the heaviest block index of all its heads first (longest first)
+      const int idx = lid >> 3;
+      pslot = idx / nh;
+      bh = (lid & 7) * nh + idx % nh;
+    } else {
+      if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
+      pslot = lid % a.n_qslot;
+      bh = lid / a.n_qslot;
+    }
   }
   const int h = bh % a.heads_q, b = bh / a.heads_q;
   const int hk = h / a.group;
@@ -335,9 +346,16 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     bhk = lid % nbh;
   } else {
     const int per = gridDim.x >> 3;
-    if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
-    pslot = lid % a.n_kslot;
-    bhk = lid / a.n_kslot;
+    const int nh = per / a.n_kslot;
+    if (a.blockmajor_k && lid < (per << 3) && nh * a.n_kslot == per) {
+      const int idx = lid >> 3;
+      pslot = idx / nh;
+      bhk = (lid & 7) * nh + idx % nh;
+    } else {
+      if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
+      pslot = lid % a.n_kslot;
+      bhk = lid / a.n_kslot;
+    }
   }
   const int hk = bhk % a.heads_k, b = bhk / a.heads_k;
 
@@ -685,6 +703,8 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   a.is_causal = p->is_causal ? 1 : 0;
   a.n_qslot = (p->seqlen_q + 127) / 128;
   a.n_kslot = (p->seqlen_k + 127) / 128;
+  a.blockmajor_q = a.is_causal && (int64_t)p->batch * p->heads_q * a.n_qslot < 8 * 256;
+  a.blockmajor_k = a.is_causal && (int64_t)p->batch * p->heads_k * a.n_kslot < 8 * 256;
   a.scale = p->scale;
   a.scale_log2 = p->scale * kLog2e;
   const float p_keep = 1.f - p->dropout_p;
