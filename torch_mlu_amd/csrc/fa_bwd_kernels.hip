@@ -635,15 +635,11 @@ int bwd_launch(const BArgs& a, hipStream_t st) {
   constexpr int lds_dq = 4 * 64 * DP * 2;
   constexpr int lds_dkv = 4 * 64 * DP * 2 + 4 * 256;
   constexpr bool split = DP > 64;  // head_dim 128: dK and dV as two launches
-  auto kq = fa_bwd_dq_kernel<T, DP, DROP>;
-  auto kkv = fa_bwd_dkv_kernel<T, DP, split ? kDK : (kDK | kDV), DROP>;
-  auto kv2 = fa_bwd_dkv_kernel<T, DP, kDV, DROP>;
-  if (hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dq) != hipSuccess ||
-      hipFuncSetAttribute((const void*)kkv, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv) != hipSuccess ||
-      (split && hipFuncSetAttribute((const void*)kv2, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv) != hipSuccess)) {
-    (void)hipGetLastError();
+  constexpr auto kq = fa_bwd_dq_kernel<T, DP, DROP>;
+  constexpr auto kkv = fa_bwd_dkv_kernel<T, DP, split ? kDK : (kDK | kDV), DROP>;
+  constexpr auto kv2 = fa_bwd_dkv_kernel<T, DP, kDV, DROP>;
+  if (!ensure_dynamic_lds<kq>(lds_dq) || !ensure_dynamic_lds<kkv>(lds_dkv) || (split && !ensure_dynamic_lds<kv2>(lds_dkv)))
     return FA_ERR_LAUNCH;
-  }
   const int64_t gq = (int64_t)a.batch * a.heads_q * a.n_qslot;
   const int64_t gk = (int64_t)a.batch * a.heads_k * a.n_kslot;
   if (gq > 0x7fffffffLL || gk > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;

@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace fa {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -130,6 +132,22 @@ __device__ __forceinline__ uint32_t drop_head_key(uint64_t seed, uint64_t offset
 // the part of a patch's counter that depends on its row pair / on its column pair; the counter is their XOR with the key
 __device__ __forceinline__ uint32_t drop_row_term(uint32_t rowpair) { return (rowpair << 16) ^ ((rowpair >> 16) * 0x9e3779b1u); }
 __device__ __forceinline__ uint32_t drop_col_term(uint32_t colpair) { return (colpair & 0xffffu) ^ ((colpair >> 16) * 0x7f4a7c15u); }
+
+// ---- host: opt a kernel into more than 64 KiB of dynamic LDS, once per kernel and device ---------------------
+template <auto KFN>
+inline bool ensure_dynamic_lds(int bytes) {
+  static std::atomic<uint64_t> done{0};  // bit d: set for device d
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const uint64_t bit = dev < 64 ? (uint64_t)1 << dev : 0;
+  if (bit && (done.load(std::memory_order_acquire) & bit)) return true;
+  if (hipFuncSetAttribute((const void*)KFN, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  done.fetch_or(bit, std::memory_order_release);
+  return true;
+}
 
 }  // namespace fa
 

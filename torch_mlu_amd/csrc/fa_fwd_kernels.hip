@@ -916,11 +916,8 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
 template <typename T, int DP, int MINB, bool BIAS, bool DROP = false>
 int launch_tile(KArgs a, hipStream_t st) {
   constexpr int lds = 4 * 64 * DP * 2;
-  auto kfn = fa_tile_kernel<T, DP, MINB, BIAS, DROP>;
-  if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
-    (void)hipGetLastError();
-    return FA_ERR_LAUNCH;
-  }
+  constexpr auto kfn = fa_tile_kernel<T, DP, MINB, BIAS, DROP>;
+  if (!ensure_dynamic_lds<kfn>(lds)) return FA_ERR_LAUNCH;
   const int nblk = (a.seqlen_q + 127) / 128;
   a.pair = (DP != 256 && !a.cu_q && a.is_causal && nblk >= 2 && (int64_t)a.batch * a.heads_q * ((nblk + 1) / 2) >= 1024) ? 1 : 0;
   a.n_mblk = a.pair ? (nblk + 1) / 2 : nblk;
@@ -934,11 +931,8 @@ int launch_tile(KArgs a, hipStream_t st) {
 template <typename T, int DP>
 int launch_splitkv(const KArgs& a, hipStream_t st) {
   constexpr int lds = SplitCfg<DP>::LDS;
-  auto kfn = fa_splitkv_kernel<T, DP>;
-  if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
-    (void)hipGetLastError();
-    return FA_ERR_LAUNCH;
-  }
+  constexpr auto kfn = fa_splitkv_kernel<T, DP>;
+  if (!ensure_dynamic_lds<kfn>(lds)) return FA_ERR_LAUNCH;
   const int64_t grid = (int64_t)a.batch * a.heads_k * a.n_splits;
   if (grid > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(SplitCfg<DP>::NW * 64), lds, st, a);
