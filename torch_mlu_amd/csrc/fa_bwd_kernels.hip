@@ -484,11 +484,24 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     const unsigned char* dt = smem + 2 * TILE + buf * TILE;
     const float* lse_t = (const float*)(smem + VEC + (0 * 2 + buf) * 256);
     const float* del_t = (const float*)(smem + VEC + (1 * 2 + buf) * 256);
+    // Which query rows of this tile may this lane's key see?  Rows ql (relative to the tile) with lo <= ql < hi:
+    // hi cuts the rows beyond the sequence, lo is the causal bound kv - off (or "none" for a key beyond the sequence).
     const bool need_mask =
         (qlo + BQ > Lq) || (a.is_causal && qlo + off < wave_kv_lo + 31) || (wave_kv_lo + 32 > Lk);
+    const int m_lo = (kvrow < Lk) ? (a.is_causal ? kvrow - off - qlo : -0x40000000) : 0x40000000;
+    const unsigned m_span = (unsigned)max(Lq - qlo - m_lo, 0);  // visible iff (unsigned)(ql - m_lo) < m_span
+    const int m_base = m_lo - 4 * g;
 
 #pragma unroll
     for (int qbk = 0; qbk < 2; ++qbk) {  // two blocks of 32 query rows
+      // LSE and delta of this lane's 16 rows (register v <-> row 32 qbk + 8 (v >> 2) + 4 g + (v & 3)), fetched ahead
+      // of the MFMAs that hide their latency
+      f32x4 lv[4], dl[4];
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        lv[q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
+        if constexpr (DO_K) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
+      }
       f32x16 s, dp;
 #pragma unroll
       for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; }
@@ -501,7 +514,6 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
           dp = Mma<T>::m32(da, vf[ks], dp);
         }
       }
-      // register v of this lane <-> query row qlo + 32 qbk + 8 (v >> 2) + 4 g + (v & 3), key row kvrow
       s16x8 pb[2], dsb[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
@@ -509,16 +521,13 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
 #pragma unroll
         for (int e2 = 0; e2 < 4; ++e2) {
           const int v = 8 * t + 2 * e2;  // v, v + 1: consecutive query rows
-          const int ql = 32 * qbk + 8 * (v >> 2) + 4 * g + (v & 3);
-          const float l0 = lse_t[ql] * kLog2e, l1 = lse_t[ql + 1] * kLog2e;
-          const float d0 = DO_K ? del_t[ql] : 0.f, d1 = DO_K ? del_t[ql + 1] : 0.f;
+          const float l0 = lv[v >> 2][v & 3] * kLog2e, l1 = lv[v >> 2][(v & 3) + 1] * kLog2e;
+          const float d0 = DO_K ? dl[v >> 2][v & 3] : 0.f, d1 = DO_K ? dl[v >> 2][(v & 3) + 1] : 0.f;
           float p0 = fast_exp2(s[v] * c - l0), p1 = fast_exp2(s[v + 1] * c - l1);
           if (need_mask) {
-            const int qa0 = qlo + ql;
-            const bool ok0 = (qa0 < Lq) && (kvrow < Lk) && (!a.is_causal || kvrow <= qa0 + off);
-            const bool ok1 = (qa0 + 1 < Lq) && (kvrow < Lk) && (!a.is_causal || kvrow <= qa0 + 1 + off);
-            p0 = ok0 ? p0 : 0.f;
-            p1 = ok1 ? p1 : 0.f;
+            const int qc = 32 * qbk + 8 * (v >> 2) + (v & 3);  // ql - 4 g
+            p0 = ((unsigned)(qc - m_base) < m_span) ? p0 : 0.f;
+            p1 = ((unsigned)(qc + 1 - m_base) < m_span) ? p1 : 0.f;
           }
           float dp0 = DO_K ? dp[v] : 0.f, dp1 = DO_K ? dp[v + 1] : 0.f;
           float pv0 = p0, pv1 = p1;  // what multiplies dO in dV: P o M / (1 - p)
