@@ -243,16 +243,28 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
     f32x16 s0, s1, p0, p1;
 #pragma unroll
     for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; p0[v] = 0.f; p1[v] = 0.f; }
+    {
+      // K and V fragments are fetched one k-step ahead of the MFMAs that consume them
+      s16x8 fr[2][4];
+      fr[0][0] = *(const s16x8*)(kt + kaddr[0]);
+      fr[0][1] = *(const s16x8*)(kt + kaddr[0] + 32 * ROWB);
+      fr[0][2] = *(const s16x8*)(vt + kaddr[0]);
+      fr[0][3] = *(const s16x8*)(vt + kaddr[0] + 32 * ROWB);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const s16x8 k0f = *(const s16x8*)(kt + kaddr[ks]);
-      const s16x8 k1f = *(const s16x8*)(kt + kaddr[ks] + 32 * ROWB);
-      const s16x8 v0f = *(const s16x8*)(vt + kaddr[ks]);
-      const s16x8 v1f = *(const s16x8*)(vt + kaddr[ks] + 32 * ROWB);
-      s0 = Mma<T>::m32(k0f, qf[ks], s0);
-      s1 = Mma<T>::m32(k1f, qf[ks], s1);
-      p0 = Mma<T>::m32(v0f, dof[ks], p0);
-      p1 = Mma<T>::m32(v1f, dof[ks], p1);
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + 1 < KS) {
+          fr[(ks + 1) & 1][0] = *(const s16x8*)(kt + kaddr[ks + 1]);
+          fr[(ks + 1) & 1][1] = *(const s16x8*)(kt + kaddr[ks + 1] + 32 * ROWB);
+          fr[(ks + 1) & 1][2] = *(const s16x8*)(vt + kaddr[ks + 1]);
+          fr[(ks + 1) & 1][3] = *(const s16x8*)(vt + kaddr[ks + 1] + 32 * ROWB);
+        }
+        s0 = Mma<T>::m32(fr[ks & 1][0], qf[ks], s0);
+        s1 = Mma<T>::m32(fr[ks & 1][1], qf[ks], s1);
+        p0 = Mma<T>::m32(fr[ks & 1][2], dof[ks], p0);
+        p1 = Mma<T>::m32(fr[ks & 1][3], dof[ks], p1);
+        __builtin_amdgcn_sched_barrier(0);  // keep the loads of step ks + 1 ahead of these MFMAs
+      }
     }
     // P^T = exp2(S^T c - LSE), dS^T = P^T (dP^T - delta); masked positions contribute nothing
     const bool need_mask = (j * BN + BN > Lk) || (a.is_causal && j * BN + BN - 1 > wave_row_lo + off);
@@ -284,16 +296,28 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
       }
       dsb[t] = __builtin_bit_cast(s16x8, w);
     }
-    // dQ^T += K^T dS^T
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
+    // dQ^T += K^T dS^T; the transposed K fragments of chunk t + 1 are fetched while chunk t's MFMAs run
+    {
+      auto kfrag = [&](int mb, int t) {
         const s16x4 lo = lds_read_tr(kt + taddr[0][mb] + (16 * t) * ROWB);
         const s16x4 hi = lds_read_tr(kt + taddr[1][mb] + (16 * t) * ROWB);
-        const s16x8 av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        acc[mb] = Mma<T>::m32(av, dsb[t], acc[mb]);
+        return s16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      };
+      s16x8 ka[2][MB];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) ka[0][mb] = kfrag(mb, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        if (t + 1 < 4) {
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) ka[(t + 1) & 1][mb] = kfrag(mb, t + 1);
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[mb] = Mma<T>::m32(ka[t & 1][mb], dsb[t], acc[mb]);
+        __builtin_amdgcn_sched_barrier(0);
       }
+    }
   }
 
   if (row < Lq) {
@@ -505,13 +529,24 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
       f32x16 s, dp;
 #pragma unroll
       for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; }
+      {
+        // Q (and dO) row fragments are fetched two k-steps ahead of the MFMAs that consume them
+        s16x8 qa[2], da[2];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const s16x8 qa = *(const s16x8*)(qt + kaddr[ks] + qbk * 32 * ROWB);
-        s = Mma<T>::m32(qa, kf[ks], s);
-        if constexpr (DO_K) {
-          const s16x8 da = *(const s16x8*)(dt + kaddr[ks] + qbk * 32 * ROWB);
-          dp = Mma<T>::m32(da, vf[ks], dp);
+        for (int ks = 0; ks < 2; ++ks) {
+          qa[ks] = *(const s16x8*)(qt + kaddr[ks] + qbk * 32 * ROWB);
+          if constexpr (DO_K) da[ks] = *(const s16x8*)(dt + kaddr[ks] + qbk * 32 * ROWB);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          s = Mma<T>::m32(qa[ks & 1], kf[ks], s);
+          if constexpr (DO_K) dp = Mma<T>::m32(da[ks & 1], vf[ks], dp);
+          if (ks + 2 < KS) {
+            qa[ks & 1] = *(const s16x8*)(qt + kaddr[ks + 2] + qbk * 32 * ROWB);
+            if constexpr (DO_K) da[ks & 1] = *(const s16x8*)(dt + kaddr[ks + 2] + qbk * 32 * ROWB);
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
       s16x8 pb[2], dsb[2];
@@ -547,24 +582,29 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
         dsb[t] = __builtin_bit_cast(s16x8, wd);
       }
       // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 32 query rows of this block)
+      {
+        // transposed dO / Q fragments of step i + 1 are fetched while step i's MFMAs run (step = (t, mb))
+        auto tfrag = [&](const unsigned char* tile, int i) {
+          const int ro = (32 * qbk + 16 * (i / MB)) * ROWB;
+          const s16x4 lo = lds_read_tr(tile + taddr[0][i % MB] + ro);
+          const s16x4 hi = lds_read_tr(tile + taddr[1][i % MB] + ro);
+          return s16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        };
+        s16x8 dav[2], qav[2];
+        if constexpr (DO_V) dav[0] = tfrag(dt, 0);
+        if constexpr (DO_K) qav[0] = tfrag(qt, 0);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-          const int ro = (32 * qbk + 16 * t) * ROWB;
-          if constexpr (DO_V) {
-            const s16x4 dlo = lds_read_tr(dt + taddr[0][mb] + ro);
-            const s16x4 dhi = lds_read_tr(dt + taddr[1][mb] + ro);
-            const s16x8 dav = {dlo[0], dlo[1], dlo[2], dlo[3], dhi[0], dhi[1], dhi[2], dhi[3]};
-            dv[mb] = Mma<T>::m32(dav, pb[t], dv[mb]);
+        for (int i = 0; i < 2 * MB; ++i) {
+          if (i + 1 < 2 * MB) {
+            if constexpr (DO_V) dav[(i + 1) & 1] = tfrag(dt, i + 1);
+            if constexpr (DO_K) qav[(i + 1) & 1] = tfrag(qt, i + 1);
           }
-          if constexpr (DO_K) {
-            const s16x4 qlo4 = lds_read_tr(qt + taddr[0][mb] + ro);
-            const s16x4 qhi4 = lds_read_tr(qt + taddr[1][mb] + ro);
-            const s16x8 qav = {qlo4[0], qlo4[1], qlo4[2], qlo4[3], qhi4[0], qhi4[1], qhi4[2], qhi4[3]};
-            dk[mb] = Mma<T>::m32(qav, dsb[t], dk[mb]);
-          }
+          if constexpr (DO_V) dv[i % MB] = Mma<T>::m32(dav[i & 1], pb[i / MB], dv[i % MB]);
+          if constexpr (DO_K) dk[i % MB] = Mma<T>::m32(qav[i & 1], dsb[i / MB], dk[i % MB]);
+          __builtin_amdgcn_sched_barrier(0);
         }
+      }
     }
   }
 
