@@ -14,9 +14,15 @@
  *     dP  = dO V^T,   delta = rowsum(dO o O),   dS = P o (dP - delta)
  *     dQ  = scale * dS K,   dK = scale * dS^T Q
  * (with dropout: dV = (P o M)^T dO / (1-p) and dP = M o (dO V^T) / (1-p), M regenerated from the forward's seed/offset)
- * with the forward's masking (bottom-right aligned causal) and head grouping (dK, dV of a kv head sum over the
+ * with the forward's masking (the FA_MASK_* modes of fa_fwd.h) and head grouping (dK, dV of a kv head sum over the
  * query heads that read it).  Same rules as fa_fwd.h: plain C, device pointers, element strides, no allocation,
  * no synchronisation, work is only enqueued on the caller's stream.
+ *
+ * The same launcher serves the mem-efficient backward `mem_eff_bwd` (FlashAttention_internal.cpp:692-906, vendor call
+ * cnnlFlashAttentionBackward_v2 at :861-903): an additive bias enters the recomputed scores (scale * Q K^T + bias),
+ * the causal mask may be aligned to the top-left corner (custom_mask_type 1, :776-779,803-807), and the gradient of
+ * the bias, dBias = dS, can be written out.  (The reference allocates that gradient but never hands it to the vendor
+ * call, :836,861-903 — it comes back uninitialised there; here it is computed.)
  */
 #ifndef FA_BWD_H_
 #define FA_BWD_H_
@@ -69,7 +75,7 @@ typedef struct fa_bwd_params {
 
   float scale;
   int32_t dtype;     /* FA_DTYPE_* */
-  int32_t is_causal;
+  int32_t is_causal; /* FA_MASK_NONE / FA_MASK_CAUSAL_BOTTOM_RIGHT (= 1) / FA_MASK_CAUSAL_TOP_LEFT, as the forward */
   int32_t reserved;  /* must be 0 */
 
   /* dropout: same p as the forward and the two numbers it stored (device pointers, read by the kernels, so that no
@@ -78,6 +84,16 @@ typedef struct fa_bwd_params {
   int32_t reserved2; /* must be 0 */
   const int64_t* philox_seed;
   const int64_t* philox_offset;
+
+  /* optional additive bias of the forward (same dtype as q; NULL = none), dense mode only, not with dropout:
+     element (b, h, row, col) at bias + b*bias_stride_b + h*bias_stride_h + row*bias_stride_q + col, h a query head.
+     Strides may be 0 (broadcast) and must be multiples of 4; the pointer must be 8-byte aligned (as in the forward). */
+  const void* bias;
+  int64_t bias_stride_b, bias_stride_h, bias_stride_q;
+  /* optional output (needs bias): the gradient of the bias, [batch, heads_q, seqlen_q, seqlen_k] in q's dtype,
+     addressed like bias but never broadcast (every element of it is written, masked positions with 0) */
+  void* dbias;
+  int64_t dbias_stride_b, dbias_stride_h, dbias_stride_q;
 } fa_bwd_params;
 
 /* Host-only validation: FA_OK or a negative code (FA_ERR_UNSUPPORTED for head_dim > 128). */

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FA_FWD_ABI_VERSION 3
+#define FA_FWD_ABI_VERSION 4
 
 /* element types accepted for q/k/v/out (FlashAttention_internal.cpp:73-80 allows exactly these two) */
 #define FA_DTYPE_FP16 0

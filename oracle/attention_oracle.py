@@ -152,16 +152,21 @@ def varlen_oracle(q, k, v, cu_seqlens_q, cu_seqlens_k, is_causal: bool = False, 
 
 
 def sdpa_backward_oracle(q, k, v, dout, is_causal: bool = False, scale: Optional[float] = None, dtype=np.float64,
-                         dropout_p: float = 0.0, dropout_mask=None) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
-    """Gradients of the dense op.  q, dout [B, Hq, Sq, D], k/v [B, Hk, Sk, D] -> (dq, dk, dv) with the inputs' shapes.
+                         dropout_p: float = 0.0, dropout_mask=None, attn_bias=None, causal_top_left: bool = False,
+                         return_dbias: bool = False):
+    """Gradients of the dense op.  q, dout [B, Hq, Sq, D], k/v [B, Hk, Sk, D] -> (dq, dk, dv) with the inputs' shapes
+    (and, with return_dbias, the gradient of the bias as a fourth array [B, Hq, Sq, Sk]).
 
     The reference has no backward oracle of its own — its tests differentiate `attention_ref` with autograd
     (test/torch_ops/test_scaled_dot_product_attention.py:1049-1113) — so this is the closed form of that derivative:
-        P = softmax(scale Q K^T + mask),  dV = P^T dO,  dP = dO V^T,  dS = P o (dP - rowsum(dO o O)),
-        dQ = scale dS K,  dK = scale dS^T Q,
+        P = softmax(scale Q K^T + bias + mask),  dV = P^T dO,  dP = dO V^T,  dS = P o (dP - rowsum(dO o O)),
+        dQ = scale dS K,  dK = scale dS^T Q,  dBias = dS,
     with dK, dV of a kv head summed over the query heads that read it (the "(h g)" repeat at :119-120 differentiated).
     With a dropout mask M (True = kept) and r = 1 / (1 - p): dV = (P o M)^T dO r, dP = M o (dO V^T) r, and delta is
     still rowsum(dO o O) with the dropped-out O.
+    `attn_bias` and `causal_top_left` are the mem-efficient backward's additions (mem_eff_bwd,
+    FlashAttention_internal.cpp:692-906); dBias is over the full [B, Hq, Sq, Sk] — a broadcast bias's gradient is its
+    sum over the broadcast axes, which is autograd's business.
     Pinned in tests/test_oracle_backward.py against torch.autograd on PyTorch's float64 math attention."""
     q, k, v, dout = _np(q, dtype), _np(k, dtype), _np(v, dtype), _np(dout, dtype)
     B, Hq, Sq, D = q.shape
@@ -169,8 +174,9 @@ def sdpa_backward_oracle(q, k, v, dout, is_causal: bool = False, scale: Optional
     g = Hq // Hk
     sc = (1.0 / math.sqrt(D)) if scale is None else float(scale)
     out, p, _ = attention_ref(q.transpose(0, 2, 1, 3), k.transpose(0, 2, 1, 3), v.transpose(0, 2, 1, 3), scale=scale,
-                              causal=is_causal, dtype=dtype, dropout_p=dropout_p,
-                              dropout_mask=dropout_mask)           # out [B,Hq,Sq,D], p [B,Hq,Sq,Sk] (undropped)
+                              causal=is_causal, dtype=dtype, dropout_p=dropout_p, dropout_mask=dropout_mask,
+                              attn_bias=attn_bias,
+                              causal_top_left=causal_top_left)   # out [B,Hq,Sq,D], p [B,Hq,Sq,Sk] (undropped)
     kr = np.repeat(k, g, axis=1)
     vr = np.repeat(v, g, axis=1)
     m = np.ones_like(p) if dropout_mask is None else np.asarray(dropout_mask, dtype=dtype)
@@ -183,6 +189,8 @@ def sdpa_backward_oracle(q, k, v, dout, is_causal: bool = False, scale: Optional
     dk_r = sc * np.matmul(ds.transpose(0, 1, 3, 2), q)
     dk = dk_r.reshape(B, Hk, g, Sk, D).sum(axis=2)
     dv = dv_r.reshape(B, Hk, g, Sk, D).sum(axis=2)
+    if return_dbias:
+        return dq, dk, dv, ds
     return dq, dk, dv
 
 

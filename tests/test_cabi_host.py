@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_version_and_error_strings():
     L = capi.lib()
-    assert L.fa_fwd_version() == 3
+    assert L.fa_fwd_version() == 4
     assert capi.error_string(0) == "ok"
     for rc in (-1, -2, -3, -99):
         assert capi.error_string(rc)
@@ -157,6 +157,11 @@ def test_bwd_validate_accepts_good_params_and_sizes_delta_scratch():
     packed = _good_bwd(cu_seqlens_q=0xa000, cu_seqlens_k=0xb000, total_q=200)
     assert L.fa_bwd_validate(ctypes.byref(packed)) == capi.FA_OK
     assert L.fa_bwd_workspace_bytes(ctypes.byref(packed)) == 200 * 8 * 4
+    # the mem-efficient backward's additions: mask aligned top-left, a (broadcast) bias, its gradient
+    full = _good_bwd(is_causal=capi.FA_MASK_CAUSAL_TOP_LEFT, bias=0xc000, bias_stride_b=0, bias_stride_h=0,
+                     bias_stride_q=256, dbias=0xd000, dbias_stride_b=8 * 128 * 256, dbias_stride_h=128 * 256,
+                     dbias_stride_q=256)
+    assert L.fa_bwd_validate(ctypes.byref(full)) == capi.FA_OK
 
 
 @pytest.mark.parametrize("over,rc", [
@@ -172,6 +177,15 @@ def test_bwd_validate_accepts_good_params_and_sizes_delta_scratch():
     (dict(head_dim=100), capi.FA_ERR_UNSUPPORTED),
     (dict(dtype=3), capi.FA_ERR_UNSUPPORTED),
     (dict(heads_k=3), capi.FA_ERR_UNSUPPORTED),
+    (dict(is_causal=3), capi.FA_ERR_BAD_ARG),                               # not a FA_MASK_* code
+    (dict(bias=0xc004, bias_stride_q=256), capi.FA_ERR_BAD_ARG),            # 4-key groups must be 8-byte aligned
+    (dict(bias=0xc000, bias_stride_q=258), capi.FA_ERR_BAD_ARG),
+    (dict(dbias=0xd000, dbias_stride_q=256), capi.FA_ERR_BAD_ARG),          # a bias gradient without a bias
+    (dict(bias=0xc000, bias_stride_q=256, dbias=0xd000, dbias_stride_q=0), capi.FA_ERR_BAD_ARG),   # broadcast output
+    (dict(bias=0xc000, bias_stride_q=256, dbias=0xd000, dbias_stride_q=256, dbias_stride_h=0), capi.FA_ERR_BAD_ARG),
+    (dict(bias=0xc000, bias_stride_q=256, dropout_p=0.1, philox_seed=0xe000, philox_offset=0xe008),
+     capi.FA_ERR_UNSUPPORTED),
+    (dict(bias=0xc000, bias_stride_q=256, cu_seqlens_q=0xa000, cu_seqlens_k=0xb000, total_q=200), capi.FA_ERR_UNSUPPORTED),
 ])
 def test_bwd_validate_rejects(over, rc):
     L = capi.lib()

@@ -115,8 +115,6 @@ def test_errors():
         aten._scaled_dot_product_efficient_attention(q, k, v, None, False, 0.1)
     with pytest.raises(RuntimeError, match="same dtype as query"):
         aten._scaled_dot_product_efficient_attention(q, k, v, torch.zeros(16, 16, device=DEV), False)
-    with pytest.raises(RuntimeError, match="no backward"):
-        aten._scaled_dot_product_efficient_attention(q.clone().requires_grad_(), k, v, None, True)
     with pytest.raises(RuntimeError, match="only support fp16 and bf16"):
         aten._scaled_dot_product_efficient_attention(q.float(), k.float(), v.float(), None, False)
     # C ABI: misaligned bias strides are refused before anything is enqueued

@@ -1,0 +1,332 @@
+"""GPU parity tests of the mem-efficient backward — additive bias, causal mask aligned to the top-left corner, gradient
+of the bias — through the C ABI, through the registered ATen backward ops and through autograd of
+F.scaled_dot_product_attention with an attn_mask, against the float64 CPU oracle on the same seeded inputs.
+
+Bar per gradient: max-abs error <= 2 ulp of the dtype at the gradient's largest magnitude (bf16 2^-8, fp16 2^-11); the
+reference's own tests compare these entry points with the math backend under the rule
+"no worse than fudge x the low-precision math error" (test/torch_ops/test_scaled_dot_product_attention.py:1072-1110),
+checked here as well for the dense wrapper.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+import torch_mlu_amd
+from tests._util import seeded
+from torch_mlu_amd import capi
+from torch_mlu_amd.backends import SDPBackend
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF, HF = torch.bfloat16, torch.float16
+EPS = {BF: 2.0 ** -8, HF: 2.0 ** -11}
+NAME = {BF: "bfloat16", HF: "float16"}
+MASKS = {"none": capi.FA_MASK_NONE, "tl": capi.FA_MASK_CAUSAL_TOP_LEFT, "br": capi.FA_MASK_CAUSAL_BOTTOM_RIGHT}
+
+
+def _inputs(B, Hq, Hk, Sq, Sk, D, dtype, seed):
+    return (seeded((B, Hq, Sq, D), seed, dtype), seeded((B, Hk, Sk, D), seed + 1, dtype),
+            seeded((B, Hk, Sk, D), seed + 2, dtype), seeded((B, Hq, Sq, D), seed + 3, dtype))
+
+
+def _bias(shape, dtype, seed, holes=0.0):
+    """A bias whose rows are padded to a multiple of 8 columns in memory (the alignment rule of the C ABI), with a
+    fraction of -inf entries (what a boolean attn_mask becomes); column 0 stays finite so that no row is empty."""
+    Sk = shape[-1]
+    full = seeded(shape[:-1] + ((Sk + 7) // 8 * 8,), seed, dtype, std=1.5)
+    if holes:
+        m = torch.rand(full.shape, generator=torch.Generator().manual_seed(seed + 1)) < holes
+        m[..., 0] = False
+        full = full.masked_fill(m, float("-inf"))
+    return full
+
+
+def _close(name, g, w, dtype):
+    g = g.float().cpu().double().numpy()
+    assert g.shape == w.shape, (name, g.shape, w.shape)
+    assert np.isfinite(g).all(), f"{name}: non-finite gradient"
+    err = float(np.abs(g - w).max()) if g.size else 0.0
+    bar = 2.0 * EPS[dtype] * max(float(np.abs(w).max()) if w.size else 0.0, 0.25)
+    assert err <= bar, f"{name}: max-abs error {err:.3e} > {bar:.3e}"
+    return err
+
+
+def _run_capi(q, k, v, do, mask, scale, full_bias, want_dbias=True):
+    """Forward and backward through the C ABI; `full_bias` is the padded CPU bias (or None)."""
+    Sk = k.shape[2]
+    qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
+    bd = full_bias.to(DEV)[..., :Sk] if full_bias is not None else None
+    out, lse = capi.fa_forward_dense(qd, kd, vd, is_causal=MASKS[mask], scale=scale, bias=bd)
+    got = capi.fa_backward_dense(dod, qd, kd, vd, out, lse, is_causal=MASKS[mask], scale=scale, bias=bd,
+                                 want_dbias=want_dbias and bd is not None)
+    okw = dict(is_causal=mask != "none", causal_top_left=mask == "tl", scale=scale)
+    if full_bias is not None:
+        okw["attn_bias"] = full_bias[..., :Sk].double().numpy()
+    want = oracle.sdpa_backward_oracle(q, k, v, do, return_dbias=True, **okw)
+    return got, want
+
+
+@pytest.mark.parametrize("dtype", [BF, HF])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("mask", ["none", "tl"])
+def test_full_bias_small_shapes(dtype, D, mask):
+    for i, (Sq, Sk) in enumerate([(1, 1), (7, 5), (33, 64), (64, 33), (65, 129), (128, 128), (129, 257), (200, 77)]):
+        print(f"case Sq={Sq} Sk={Sk} D={D} {dtype} mask={mask}", flush=True)
+        B, Hq, Hk = 2, 4, 2
+        q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, dtype, 400 + 10 * i)
+        fb = _bias((B, Hq, Sq, Sk), dtype, 500 + i, holes=0.2 if i % 2 else 0.0)
+        got, want = _run_capi(q, k, v, do, mask, None, fb)
+        for name, g, w in zip(("dq", "dk", "dv", "dbias"), got, want):
+            _close(name, g, w, dtype)
+
+
+@pytest.mark.parametrize("bshape", ["b1qk", "bh1k", "11qk", "1h1k", "b11k"])
+@pytest.mark.parametrize("mask", ["none", "tl", "br"])
+def test_broadcast_bias_shapes(bshape, mask):
+    """Strides of 0 along batch, head or query row; dBias is still written for the full [B, H, Sq, Sk]."""
+    B, Hq, Hk, Sq, Sk, D = 3, 6, 2, 150, 210, 64
+    q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, BF, 600)
+    shp = {"b1qk": (B, 1, Sq, Sk), "bh1k": (B, Hq, 1, Sk), "11qk": (1, 1, Sq, Sk), "1h1k": (1, Hq, 1, Sk),
+           "b11k": (B, 1, 1, Sk)}[bshape]
+    fb = _bias(shp, BF, 610, holes=0.1)
+    got, want = _run_capi(q, k, v, do, mask, 0.2, fb)
+    for name, g, w in zip(("dq", "dk", "dv", "dbias"), got, want):
+        _close(name, g, w, BF)
+
+
+@pytest.mark.parametrize("dtype", [BF, HF])
+@pytest.mark.parametrize("shape", [(1, 2, 2, 300, 100, 128), (2, 4, 1, 100, 300, 128), (1, 3, 3, 257, 257, 96),
+                                   (2, 2, 2, 64, 512, 40), (1, 8, 2, 1, 333, 64)])
+def test_top_left_mask_without_bias(dtype, shape):
+    """custom_mask_type 1 (FlashAttention_internal.cpp:776-779): col <= row whatever the two lengths are."""
+    q, k, v, do = _inputs(*shape, dtype, 700)
+    got, want = _run_capi(q, k, v, do, "tl", None, None)
+    for name, g, w in zip(("dq", "dk", "dv"), got, want):
+        _close(name, g, w, dtype)
+    Sq, Sk = shape[3], shape[4]
+    if Sk > Sq:   # keys beyond the last query row are never seen: exact zeros
+        assert float(got[1][:, :, Sq:].abs().max()) == 0.0 and float(got[2][:, :, Sq:].abs().max()) == 0.0
+
+
+def test_negative_scale_and_large_bias():
+    B, Hq, Hk, Sq, Sk, D = 1, 4, 4, 190, 170, 128
+    q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, BF, 800)
+    fb = _bias((B, Hq, Sq, Sk), BF, 801) * 8.0
+    got, want = _run_capi(q, k, v, do, "none", -0.15, fb)
+    for name, g, w in zip(("dq", "dk", "dv", "dbias"), got, want):
+        _close(name, g, w, BF)
+
+
+def test_row_with_only_minus_inf_bias_has_zero_gradient():
+    """A query row whose bias is -inf throughout: forward output 0, LSE +inf; backward contributes nothing and its
+    dBias row is 0 (no NaN from inf - inf)."""
+    B, Hq, Hk, Sq, Sk, D = 1, 2, 2, 70, 90, 64
+    q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, HF, 810)
+    fb = _bias((B, Hq, Sq, Sk), HF, 811, holes=0.1)
+    fb[:, :, 5, :] = float("-inf")
+    fb[:, 1, 64:, :] = float("-inf")
+    got, want = _run_capi(q, k, v, do, "none", None, fb)
+    for name, g, w in zip(("dq", "dk", "dv", "dbias"), got, want):
+        _close(name, g, w, HF)
+    assert float(got[0][:, :, 5].abs().max()) == 0.0 and float(got[3][:, :, 5].abs().max()) == 0.0
+
+
+def test_dbias_is_optional_and_does_not_change_the_other_gradients():
+    B, Hq, Hk, Sq, Sk, D = 2, 2, 1, 130, 200, 128
+    q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, BF, 820)
+    fb = _bias((B, 1, Sq, Sk), BF, 821)
+    with_db, _ = _run_capi(q, k, v, do, "tl", None, fb, want_dbias=True)
+    without, _ = _run_capi(q, k, v, do, "tl", None, fb, want_dbias=False)
+    assert len(without) == 3
+    for a, b in zip(with_db, without):
+        assert torch.equal(a, b)
+
+
+def test_dbias_padding_columns_are_not_written():
+    """Only [.., :Sk] of each dBias row belongs to the gradient; the bytes between rows are left alone."""
+    B, Hq, Hk, Sq, Sk, D = 1, 2, 2, 40, 67, 64
+    q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, BF, 830)
+    qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
+    bd = _bias((B, Hq, Sq, Sk), BF, 831).to(DEV)[..., :Sk]
+    out, lse = capi.fa_forward_dense(qd, kd, vd, is_causal=capi.FA_MASK_CAUSAL_TOP_LEFT, bias=bd)
+    p = capi.FaBwdParams()
+    dq, dk, dv = (torch.empty((B, s, h, D), dtype=BF, device=DEV) for s, h in ((Sq, Hq), (Sk, Hk), (Sk, Hk)))
+    store = torch.full((B, Hq, Sq, 72), 7.0, dtype=BF, device=DEV)
+    views = {"q": qd.transpose(1, 2), "k": kd.transpose(1, 2), "v": vd.transpose(1, 2), "o": out.transpose(1, 2),
+             "do": dod.transpose(1, 2), "dq": dq, "dk": dk, "dv": dv}
+    p.q, p.k, p.v, p.out, p.dout = (views[n].data_ptr() for n in ("q", "k", "v", "o", "do"))
+    p.lse, p.dq, p.dk, p.dv = lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    for n, t in views.items():
+        capi._set_strides(p, n, t, False)
+    p.lse_stride_b, p.lse_stride_h, p.lse_stride_s = lse.stride(0), lse.stride(1), lse.stride(2)
+    p.batch, p.heads_q, p.heads_k, p.seqlen_q, p.seqlen_k, p.head_dim = B, Hq, Hk, Sq, Sk, D
+    p.scale, p.dtype, p.is_causal = 1.0 / math.sqrt(D), capi.FA_DTYPE_BF16, capi.FA_MASK_CAUSAL_TOP_LEFT
+    p.bias, p.bias_stride_b, p.bias_stride_h, p.bias_stride_q = bd.data_ptr(), bd.stride(0), bd.stride(1), bd.stride(2)
+    p.dbias, p.dbias_stride_b, p.dbias_stride_h, p.dbias_stride_q = store.data_ptr(), store.stride(0), store.stride(1), 72
+    capi._launch_bwd(p, qd.device)
+    torch.cuda.synchronize()
+    assert bool((store[..., Sk:] == 7.0).all())
+    want = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True, causal_top_left=True,
+                                       attn_bias=bd.cpu().double().numpy(), return_dbias=True)[3]
+    _close("dbias", store[..., :Sk], want, BF)
+    # the causal part is exact zeros, also in key tiles the kernel never computes
+    upper = torch.triu(torch.ones(Sq, Sk, dtype=torch.bool, device=DEV), diagonal=1)
+    assert float(store[..., :Sk][..., upper].abs().max()) == 0.0
+
+
+def test_bias_backward_at_a_prefill_shape():
+    """One larger problem (several key tiles per workgroup, many workgroups), checked on a subset of heads."""
+    B, H, S, D = 1, 4, 1024, 128
+    q, k, v, do = _inputs(B, H, H, S, S, D, BF, 840)
+    fb = _bias((B, H, S, S), BF, 841, holes=0.05)
+    got, want = _run_capi(q, k, v, do, "tl", None, fb)
+    for name, g, w in zip(("dq", "dk", "dv", "dbias"), got, want):
+        _close(name, g, w, BF)
+
+
+# ---- through the registered ATen ops and autograd -------------------------------------------------------------------
+aten = torch.ops.aten
+
+
+def _lowp_math_grads(q, k, v, do, bias, top_left, scale):
+    """The same math done naively in the inputs' dtype on the CPU with autograd (the reference tests' `*_lp_ref`)."""
+    q, k, v = (t.clone().requires_grad_() for t in (q, k, v))
+    b = bias.clone().requires_grad_() if bias is not None else None
+    Hq, Hk, Sq, Sk, D = q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3]
+    kr, vr = k.repeat_interleave(Hq // Hk, dim=1), v.repeat_interleave(Hq // Hk, dim=1)
+    s = torch.matmul(q, kr.transpose(-1, -2)) * (1.0 / math.sqrt(D) if scale is None else scale)
+    if b is not None:
+        s = s + b
+    if top_left:
+        s = s.masked_fill(torch.arange(Sk)[None, :] > torch.arange(Sq)[:, None], float("-inf"))
+    torch.matmul(torch.softmax(s, dim=-1), vr).backward(do)
+    return tuple(t.grad.double().numpy() for t in ((q, k, v) if b is None else (q, k, v, b)))
+
+
+@pytest.mark.parametrize("dtype", [BF, HF])
+@pytest.mark.parametrize("causal", [False, True])
+def test_dense_wrapper_forward_and_backward_ops(dtype, causal):
+    """_scaled_dot_product_efficient_attention + ..._backward called as autograd calls them; the reference rule of
+    test_scaled_dot_product_attention.py:1072-1110 on top of the fixed bar."""
+    B, H, Sq, Sk, D = 2, 4, 100, 140, 64
+    q, k, v, do = _inputs(B, H, H, Sq, Sk, D, dtype, 900)
+    bias = _bias((B, H, Sq, Sk), dtype, 901)[..., :Sk].contiguous()
+    qd, kd, vd, dod, bd = (t.to(DEV) for t in (q, k, v, do, bias))
+    n0 = torch_mlu_amd.launch_count()
+    out, lse, seed, offset = aten._scaled_dot_product_efficient_attention(qd, kd, vd, bd, True, 0.0, causal)
+    gq, gk, gv, gb = aten._scaled_dot_product_efficient_attention_backward(
+        dod, qd, kd, vd, bd, out, lse, seed, offset, 0.0, [True, True, True, True], causal)
+    assert torch_mlu_amd.launch_count() == n0 + 2
+    assert gq.shape == q.shape and gk.shape == k.shape and gv.shape == v.shape and gb.shape == bias.shape
+    assert gq.transpose(1, 2).is_contiguous()                         # [B, S, H, D] storage, like the forward's output
+    want = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=causal, causal_top_left=causal,
+                                       attn_bias=bias.double().numpy(), return_dbias=True)
+    lowp = _lowp_math_grads(q, k, v, do, bias, causal, None)
+    for name, g, w, lp, fudge in zip(("dq", "dk", "dv", "dbias"), (gq, gk, gv, gb), want, lowp, (4.0, 2.0, 2.0, 4.0)):
+        _close(name, g, w, dtype)
+        atol, rtol = oracle.get_tolerances(w, lp, NAME[dtype], fudge)
+        assert np.allclose(g.float().cpu().double().numpy(), w, atol=atol, rtol=rtol), name
+    # without a bias gradient the fourth result is undefined and nothing else changes
+    g3 = aten._scaled_dot_product_efficient_attention_backward(
+        dod, qd, kd, vd, bd, out, lse, seed, offset, 0.0, [True, True, True, False], causal)
+    assert g3[3] is None and all(torch.equal(a, b) for a, b in zip(g3[:3], (gq, gk, gv)))
+
+
+def test_efficient_attention_backward_op_layouts_and_mask_types():
+    """_efficient_attention_backward on [B, S, H, D] inputs: the three custom_mask_types, GQA, a bias that is broadcast
+    in its own shape (its gradient comes back summed to that shape), shared dq/dk/dv storage."""
+    B, Hq, Hk, S, D = 2, 4, 2, 96, 128
+    q, k, v, do = _inputs(B, Hq, Hk, S, S + 40, D, BF, 910)
+    bias = _bias((1, Hq, 1, S + 40), BF, 911)[..., :S + 40].contiguous()
+    qs, ks, vs, dos = (t.to(DEV).transpose(1, 2) for t in (q, k, v, do))
+    bd = bias.to(DEV)
+    for cmt, okw in ((0, {}), (1, dict(is_causal=True, causal_top_left=True)), (2, dict(is_causal=True))):
+        out, lse, seed, offset, mq, mk = aten._efficient_attention_forward(qs, ks, vs, bd, None, None, None, None, 0.0,
+                                                                           cmt, True)
+        gq, gk, gv, gb = aten._efficient_attention_backward(dos, qs, ks, vs, bd, out, None, None, mq, mk, lse, 0.0,
+                                                            seed, offset, cmt, True)
+        assert gq.shape == qs.shape and gk.shape == ks.shape and gb.shape == bias.shape
+        want = oracle.sdpa_backward_oracle(q, k, v, do, attn_bias=bias.double().numpy(), return_dbias=True, **okw)
+        for name, g, w in zip(("dq", "dk", "dv"), (gq, gk, gv), want):
+            _close(name, g.transpose(1, 2), w, BF)
+        wb = want[3].sum(axis=(0, 2), keepdims=True)
+        errb = np.abs(gb.float().cpu().double().numpy() - wb).max()
+        assert errb <= 2.0 * EPS[BF] * max(np.abs(wb).max(), 0.25) + B * S * 2.0 ** -9 * np.abs(want[3]).max()
+    q2, k2, v2, do2 = _inputs(B, Hq, Hq, S, S, D, BF, 920)
+    qs, ks, vs, dos = (t.to(DEV).transpose(1, 2) for t in (q2, k2, v2, do2))
+    out, lse, seed, offset, mq, mk = aten._efficient_attention_forward(qs, ks, vs, None, None, None, None, None, 0.0, 1, True)
+    gq, gk, gv, gb = aten._efficient_attention_backward(dos, qs, ks, vs, None, out, None, None, mq, mk, lse, 0.0, seed,
+                                                        offset, 1, False, shared_storage_dqdkdv=True)
+    assert gb is None
+    assert gk.data_ptr() == gq.data_ptr() + Hq * D * 2 and gv.data_ptr() == gq.data_ptr() + 2 * Hq * D * 2
+    want = oracle.sdpa_backward_oracle(q2, k2, v2, do2, is_causal=True)
+    for name, g, w in zip(("dq", "dk", "dv"), (gq, gk, gv), want):
+        _close(name, g.transpose(1, 2), w, BF)
+
+
+def test_backward_op_errors():
+    q, k, v, do = (t.to(DEV).transpose(1, 2) for t in _inputs(1, 2, 2, 16, 16, 64, HF, 930))
+    out, lse, seed, offset, mq, mk = aten._efficient_attention_forward(q, k, v, None, None, None, None, None, 0.0, 0, True)
+    args = lambda **o: aten._efficient_attention_backward(
+        o.get("do", do), q, k, v, o.get("bias"), out, o.get("cu"), o.get("cu"), mq, mk, o.get("lse", lse),
+        o.get("p", 0.0), seed, offset, o.get("cmt", 0), False)
+    with pytest.raises(RuntimeError, match="dropout"):
+        args(p=0.2)
+    with pytest.raises(RuntimeError, match="cu_seqlens are not supported"):
+        args(cu=torch.zeros(2, dtype=torch.int32, device=DEV))
+    with pytest.raises(RuntimeError, match="custom_mask_type"):
+        args(cmt=3)
+    with pytest.raises(RuntimeError, match="compute_log_sumexp"):
+        args(lse=torch.empty(1, 2, 0, device=DEV))
+    with pytest.raises(RuntimeError, match="same dtype"):
+        args(do=do.to(BF))
+    with pytest.raises(RuntimeError, match="same dtype as query"):
+        args(bias=torch.zeros(16, 16, device=DEV))
+    q256 = torch.zeros(1, 16, 2, 256, dtype=HF, device=DEV)
+    with pytest.raises(RuntimeError, match="at most 128"):
+        aten._efficient_attention_backward(q256, q256, q256, q256, None, q256, None, None, 16, 16,
+                                           torch.zeros(1, 2, 16, device=DEV), 0.0, seed, offset, 0, False)
+
+
+@pytest.mark.parametrize("mshape", ["full", "qk", "key_padding"])
+def test_training_with_attn_mask_through_plain_sdpa(mshape):
+    """F.scaled_dot_product_attention with an attn_mask that requires a gradient: the selector picks this build's
+    mem-efficient entry point, autograd pairs it with this build's backward (one launch each), and the gradients —
+    the mask's included, summed over what it was broadcast along — are the oracle's."""
+    B, Hq, Hk, Sq, Sk, D = 2, 4, 2, 72, 104, 64
+    q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, BF, 940)
+    shp = {"full": (B, Hq, Sq, Sk), "qk": (Sq, Sk), "key_padding": (B, 1, 1, Sk)}[mshape]
+    mask = seeded(shp, 941, BF, std=1.0)
+    qd, kd, vd = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    md = mask.to(DEV).requires_grad_()
+    assert torch._fused_sdp_choice(qd, kd, vd, md, 0.0, False, enable_gqa=True) == SDPBackend.EFFICIENT_ATTENTION
+    n0 = torch_mlu_amd.launch_count()
+    out = F.scaled_dot_product_attention(qd, kd, vd, attn_mask=md, enable_gqa=True)
+    out.backward(do.to(DEV))
+    assert torch_mlu_amd.launch_count() == n0 + 2
+    want = oracle.sdpa_backward_oracle(q, k, v, do, attn_bias=mask.double().numpy(), return_dbias=True)
+    for name, t, w in zip(("dq", "dk", "dv"), (qd, kd, vd), want):
+        _close(name, t.grad, w, BF)
+    full = np.broadcast_to(np.zeros(shp), (B, Hq, Sq, Sk)).shape
+    lead = len(full) - len(shp)
+    axes = tuple(range(lead)) + tuple(lead + i for i, n in enumerate(shp) if n == 1 and full[lead + i] != 1)
+    wb = want[3].sum(axis=axes, keepdims=True).reshape(shp)
+    nsum = want[3].size // wb.size                        # bf16 terms summed per element of the mask's gradient
+    errb = np.abs(md.grad.float().cpu().double().numpy() - wb).max()
+    assert errb <= 2.0 * EPS[BF] * max(np.abs(wb).max(), 0.25) + nsum * 2.0 ** -9 * np.abs(want[3]).max()
+
+
+def test_training_non_square_causal_through_plain_sdpa():
+    """is_causal with Sq != Sk is F.sdpa's top-left mask: mem-efficient forward and backward of this build."""
+    q, k, v, do = _inputs(1, 2, 2, 90, 150, 128, HF, 950)
+    qd, kd, vd = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    n0 = torch_mlu_amd.launch_count()
+    F.scaled_dot_product_attention(qd, kd, vd, is_causal=True).backward(do.to(DEV))
+    assert torch_mlu_amd.launch_count() == n0 + 2
+    want = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True, causal_top_left=True)
+    for name, t, w in zip(("dq", "dk", "dv"), (qd, kd, vd), want):
+        _close(name, t.grad, w, HF)

@@ -196,3 +196,69 @@ def test_dropout_mask_restatement_properties():
     # p = 0 keeps everything; thresholds follow float32 arithmetic
     assert oracle.dropout_keep_mask(1, 0, 0, 64, 64, 0.0).all()
     assert abs(oracle.dropout_keep_mask(1, 0, 0, 512, 512, 0.6).mean() - 102 / 256) < 5e-3
+
+
+# ---- additive bias, top-left causal mask, gradient of the bias (the mem-efficient backward's additions) -------------
+@pytest.mark.parametrize("causal_tl", [False, True])
+@pytest.mark.parametrize("bshape", ["full", "row", "head"])
+@pytest.mark.parametrize("scale", [None, -0.4])
+def test_bias_backward_oracle_vs_autograd_float64(causal_tl, bshape, scale):
+    """softmax(scale q k^T + bias [+ top-left causal mask]) v differentiated by autograd, including d/d bias (through
+    the broadcast, which sums) and -inf entries in the bias."""
+    B, Hq, Hk, Sq, Sk, D = 2, 4, 2, 19, 27, 16
+    q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, seed=300)
+    shp = {"full": (B, Hq, Sq, Sk), "row": (B, 1, 1, Sk), "head": (1, Hq, Sq, Sk)}[bshape]
+    bias = seeded(shp, 305, torch.float32, std=1.5).double()
+    hole = torch.rand(shp, generator=torch.Generator().manual_seed(9)) < 0.15
+    hole[..., 0] = False                                     # every row keeps a visible key
+    qq, kk, vv = (t.double().clone().requires_grad_() for t in (q, k, v))
+    bb = bias.clone().requires_grad_()
+    kr, vr = kk.repeat_interleave(Hq // Hk, 1), vv.repeat_interleave(Hq // Hk, 1)
+    s = torch.matmul(qq, kr.transpose(-1, -2)) * (1.0 / math.sqrt(D) if scale is None else scale)
+    s = s + bb.masked_fill(hole, float("-inf"))
+    if causal_tl:
+        s = s.masked_fill(torch.arange(Sk)[None, :] > torch.arange(Sq)[:, None], float("-inf"))
+    torch.matmul(torch.softmax(s, -1), vr).backward(do.double())
+    nb = bias.masked_fill(hole, float("-inf")).numpy()
+    dq, dk, dv, db = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=causal_tl, causal_top_left=causal_tl,
+                                                 scale=scale, attn_bias=nb, return_dbias=True)
+    for g, w in zip((dq, dk, dv), (qq.grad, kk.grad, vv.grad)):
+        assert np.abs(g - w.numpy()).max() < 1e-12
+    assert db.shape == (B, Hq, Sq, Sk)
+    red = [ax for ax in range(4) if shp[ax] == 1 and db.shape[ax] != 1]
+    db_r = db.sum(axis=tuple(red), keepdims=True) if red else db
+    assert np.abs(db_r - bb.grad.numpy()).max() < 1e-12
+    assert (db[np.broadcast_to(hole.numpy(), db.shape)] == 0).all()   # no gradient through a -inf entry
+
+
+def test_bias_gradient_vs_finite_differences():
+    """d<out, dout>/d bias by central differences of the forward oracle: no shared derivative code."""
+    B, Hq, Hk, Sq, Sk, D = 1, 2, 1, 3, 4, 4
+    q, k, v, do = (t.double().numpy() for t in _inputs(B, Hq, Hk, Sq, Sk, D, seed=310))
+    bias = seeded((B, Hq, Sq, Sk), 311, torch.float32).double().numpy()
+    db = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True, causal_top_left=True, scale=0.6, attn_bias=bias,
+                                     return_dbias=True)[3]
+    h, num = 1e-6, np.zeros_like(bias)
+    for idx in np.ndindex(*bias.shape):
+        bp, bm = bias.copy(), bias.copy()
+        bp[idx] += h
+        bm[idx] -= h
+        fp = (oracle.sdpa_oracle(q, k, v, is_causal=True, causal_top_left=True, scale=0.6, attn_bias=bp)[0] * do).sum()
+        fm = (oracle.sdpa_oracle(q, k, v, is_causal=True, causal_top_left=True, scale=0.6, attn_bias=bm)[0] * do).sum()
+        num[idx] = (fp - fm) / (2 * h)
+    assert np.abs(num - db).max() < 1e-8
+    # rows of dS sum to zero (softmax Jacobian), masked entries carry none
+    assert np.abs(db.sum(-1)).max() < 1e-12
+    assert (db[..., 0, 1:] == 0).all()
+
+
+def test_top_left_and_bottom_right_masks_differ_only_when_lengths_differ():
+    q, k, v, do = _inputs(1, 2, 2, 9, 14, 8, seed=320)
+    tl = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True, causal_top_left=True)
+    br = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True)
+    assert np.abs(tl[0] - br[0]).max() > 1e-3
+    assert np.abs(tl[1][:, :, 9:]).max() == 0 and np.abs(tl[2][:, :, 9:]).max() == 0   # keys beyond the last row: unseen
+    q2, k2, v2, do2 = _inputs(1, 2, 2, 11, 11, 8, seed=321)
+    for a_, b_ in zip(oracle.sdpa_backward_oracle(q2, k2, v2, do2, is_causal=True, causal_top_left=True),
+                      oracle.sdpa_backward_oracle(q2, k2, v2, do2, is_causal=True)):
+        assert np.array_equal(a_, b_)

@@ -91,7 +91,11 @@ def test_mem_efficient_constraints():
     assert "dropout" in mem_reason(q, k, v, None, 0.1)
     assert "Mem efficient attention requires query.size(-1)==key.size(-1)==value.size(-1)" in mem_reason(*_qkv((2, 2, 3, 12)))
     assert "4 dimensional" in mem_reason(*_qkv((2, 3, 8)))
-    assert "no backward" in mem_reason(q.clone().requires_grad_(), k, v)
-    assert "no backward" in mem_reason(q, k, v, mask.clone().requires_grad_())
+    assert "HIP device" in mem_reason(q.clone().requires_grad_(), k, v)   # a gradient is fine up to head_dim 128 ...
+    assert "HIP device" in mem_reason(q, k, v, mask.clone().requires_grad_())
+    q3, k3, v3 = _qkv((1, 2, 16, 256))
+    assert "HIP device" in mem_reason(q3, k3, v3)
+    assert "stops at head dimension 128" in mem_reason(q3.clone().requires_grad_(), k3, v3)     # ... and not beyond
+    assert "stops at head dimension 128" in mem_reason(q3, k3, v3, mask.clone().requires_grad_())
     with torch_mlu_amd.backends.sdp_kernel(enable_flash=True, enable_math=True, enable_mem_efficient=False):
         assert "Memory Efficient attention has been runtime disabled." in mem_reason(q, k, v)

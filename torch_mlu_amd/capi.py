@@ -100,6 +100,8 @@ class FaBwdParams(ctypes.Structure):
         + [(n, ctypes.c_int32) for n in ("dtype", "is_causal", "reserved")]
         + [("dropout_p", ctypes.c_float), ("reserved2", ctypes.c_int32), ("philox_seed", ctypes.c_void_p),
            ("philox_offset", ctypes.c_void_p)]
+        + [("bias", ctypes.c_void_p)] + [(f"bias_stride_{d}", ctypes.c_int64) for d in "bhq"]
+        + [("dbias", ctypes.c_void_p)] + [(f"dbias_stride_{d}", ctypes.c_int64) for d in "bhq"]
     )
 
 
@@ -278,12 +280,14 @@ def _set_strides(p, name, t, packed):
 
 
 def fa_backward_dense(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
-                      lse: torch.Tensor, *, is_causal: bool = False, scale: Optional[float] = None,
-                      dropout_p: float = 0.0, rng: Optional[torch.Tensor] = None
-                      ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                      lse: torch.Tensor, *, is_causal=False, scale: Optional[float] = None,
+                      dropout_p: float = 0.0, rng: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+                      want_dbias: bool = False):
     """All of dout, q, out [B, Hq, Sq, D] and k, v [B, Hk, Sk, D] (any strides, contiguous last dim), lse [B, Hq, Sq]
     -> (dq, dk, dv) stored [B, S, H, D] and returned as [B, H, S, D] views, like the reference's dense wrapper
-    (torch_mlu/csrc/aten/operators/cnnl/transformers/attention.cpp:297-302)."""
+    (torch_mlu/csrc/aten/operators/cnnl/transformers/attention.cpp:297-302).  `is_causal`: False / True (bottom-right
+    aligned) or a FA_MASK_* code; `bias`: anything that expands to [B, Hq, Sq, Sk]; with `want_dbias` a fourth result,
+    the gradient of the (expanded) bias [B, Hq, Sq, Sk], rows padded to a multiple of 8 columns in memory."""
     B, Hq, Sq, D = q.shape
     Hk, Sk = k.shape[1], k.shape[2]
     dq = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
@@ -302,9 +306,20 @@ def fa_backward_dense(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: t
     p.batch, p.heads_q, p.heads_k, p.seqlen_q, p.seqlen_k, p.head_dim = B, Hq, Hk, Sq, Sk, D
     p.total_q = 0
     p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
-    p.dtype, p.is_causal, p.reserved = _dtype_code(q.dtype), 1 if is_causal else 0, 0
+    p.dtype, p.is_causal, p.reserved = _dtype_code(q.dtype), int(is_causal), 0
     _set_dropout(p, dropout_p, rng)
+    dbias = None
+    if bias is not None:
+        bias = bias.expand(B, Hq, Sq, Sk)
+        p.bias = bias.data_ptr()
+        p.bias_stride_b, p.bias_stride_h, p.bias_stride_q = bias.stride(0), bias.stride(1), bias.stride(2)
+        if want_dbias:
+            dbias = torch.empty((B, Hq, Sq, (Sk + 7) // 8 * 8), dtype=q.dtype, device=q.device)[..., :Sk]
+            p.dbias = dbias.data_ptr()
+            p.dbias_stride_b, p.dbias_stride_h, p.dbias_stride_q = dbias.stride(0), dbias.stride(1), dbias.stride(2)
     _launch_bwd(p, q.device)
+    if want_dbias:
+        return dq.transpose(1, 2), dk.transpose(1, 2), dv.transpose(1, 2), dbias
     return dq.transpose(1, 2), dk.transpose(1, 2), dv.transpose(1, 2)
 
 

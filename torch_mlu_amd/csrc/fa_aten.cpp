@@ -430,14 +430,25 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> scaled_dot_product_flash_attentio
 }
 
 namespace {
-// The mem-efficient entry points of this build have no backward: refuse loudly instead of letting autograd pair this
-// forward with another implementation's backward.
-void check_no_gradient_required(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
-                                const std::optional<at::Tensor>& bias) {
-  TORCH_CHECK(!(at::GradMode::is_enabled() && (q.requires_grad() || k.requires_grad() || v.requires_grad() ||
-                                                (bias.has_value() && bias->defined() && bias->requires_grad()))),
-              "efficient attention forward: this build has no backward for the mem-efficient entry points; use the "
-              "flash or math backend for training");
+// The bias as a [B, H, Sq, Sk] view (stride 0 where broadcast) that meets the kernels' alignment rule: groups of 4
+// keys 8-byte aligned.  If the caller's does not, one copy of the un-broadcast bias with rows padded to a multiple of
+// 8 columns is made (the reference always copies: cnnl_contiguous, attention.cpp:660-663).
+at::Tensor bias_for_kernels(const at::Tensor& bias, at::ScalarType dt, int64_t B, int64_t Hq, int64_t Sq, int64_t Sk) {
+  TORCH_CHECK(bias.scalar_type() == dt, "bias must have the same dtype as query");
+  TORCH_CHECK(bias.is_cuda(), "bias must be on HIP device");
+  TORCH_CHECK(bias.dim() <= 4, "bias must have at most 4 dimensions");
+  at::Tensor bias_e = bias.expand({B, Hq, Sq, Sk});
+  const bool ok = Sk == 0 || (bias_e.stride(3) == 1 && bias_e.stride(0) % 4 == 0 && bias_e.stride(1) % 4 == 0 &&
+                              bias_e.stride(2) % 4 == 0 && reinterpret_cast<uintptr_t>(bias_e.data_ptr()) % 8 == 0);
+  if (!ok) {
+    const int64_t Skp = (Sk + 7) / 8 * 8;
+    at::Tensor b4 = bias;
+    while (b4.dim() < 4) b4 = b4.unsqueeze(0);
+    at::Tensor padded = at::empty({b4.size(0), b4.size(1), b4.size(2), Skp}, b4.options());
+    padded.narrow(3, 0, Sk).copy_(b4.expand({b4.size(0), b4.size(1), b4.size(2), Sk}));
+    bias_e = padded.narrow(3, 0, Sk).expand({B, Hq, Sq, Sk});
+  }
+  return bias_e;
 }
 }  // namespace
 
@@ -470,7 +481,6 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   TORCH_CHECK(!window_size.has_value() || *window_size <= 0, "efficient attention forward: sliding window is not supported");
   TORCH_CHECK(dropout_p == 0.0, "efficient attention forward: dropout_p > 0 is not supported by this build");
   TORCH_CHECK(custom_mask_type >= 0 && custom_mask_type <= 2, "custom_mask_type must be 0, 1 or 2");
-  check_no_gradient_required(query, key, value, bias);
   // mem_eff_fwd's checks (FlashAttention_internal.cpp:500-527)
   const auto dt = query.scalar_type();
   TORCH_CHECK(dt == at::kHalf || dt == at::kBFloat16, "FlashAttention only support fp16 and bf16 data type");
@@ -492,23 +502,8 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   at::Tensor output = at::empty({B, Sq, Hq, D}, q.options());
   at::Tensor lse = at::empty({B, Hq, Sq}, q.options().dtype(at::kFloat));
 
-  at::Tensor bias_e;  // [B, H, Sq, Sk] view (stride 0 where broadcast), 4-element groups 8-byte aligned
-  if (bias.has_value() && bias->defined()) {
-    TORCH_CHECK(bias->scalar_type() == dt, "bias must have the same dtype as query");
-    TORCH_CHECK(bias->is_cuda(), "bias must be on HIP device");
-    TORCH_CHECK(bias->dim() <= 4, "bias must have at most 4 dimensions");
-    bias_e = bias->expand({B, Hq, Sq, Sk});
-    const bool ok = Sk == 0 || (bias_e.stride(3) == 1 && bias_e.stride(0) % 4 == 0 && bias_e.stride(1) % 4 == 0 &&
-                                bias_e.stride(2) % 4 == 0 && reinterpret_cast<uintptr_t>(bias_e.data_ptr()) % 8 == 0);
-    if (!ok) {  // one copy of the un-broadcast bias with rows padded to a multiple of 8 columns (the reference always copies)
-      const int64_t Skp = (Sk + 7) / 8 * 8;
-      at::Tensor b4 = *bias;
-      while (b4.dim() < 4) b4 = b4.unsqueeze(0);
-      at::Tensor padded = at::empty({b4.size(0), b4.size(1), b4.size(2), Skp}, b4.options());
-      padded.narrow(3, 0, Sk).copy_(b4.expand({b4.size(0), b4.size(1), b4.size(2), Sk}));
-      bias_e = padded.narrow(3, 0, Sk).expand({B, Hq, Sq, Sk});
-    }
-  }
+  at::Tensor bias_e;
+  if (bias.has_value() && bias->defined()) bias_e = bias_for_kernels(*bias, dt, B, Hq, Sq, Sk);
 
   fa_fwd_params p{};
   p.q = q.data_ptr(); p.k = k.data_ptr(); p.v = v.data_ptr(); p.out = output.data_ptr();
@@ -556,13 +551,160 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> scaled_dot_product_ef
     bool compute_log_sumexp, double dropout_p, bool is_causal, std::optional<double> scale) {
   TORCH_CHECK(query.dim() == 4 && key.dim() == 4 && value.dim() == 4,
               "query, key and value must be 4-dimensional (batch, num_heads, seq_len, head_dim)");
-  check_no_gradient_required(query, key, value, attn_bias);  // the views made below do not carry requires_grad
   auto [out, lse, seed, offset, mq, mk] = efficient_attention_forward(
       query.transpose(1, 2), key.transpose(1, 2), value.transpose(1, 2), attn_bias, std::nullopt, std::nullopt,
       std::nullopt, std::nullopt, dropout_p, is_causal ? 1 : 0, compute_log_sumexp, scale, std::nullopt, std::nullopt);
   (void)mq;
   (void)mk;
   return std::make_tuple(out.transpose(1, 2), lse, seed, offset);
+}
+
+// ---- _efficient_attention_backward ----------------------------------------------------------------------------
+// cnnl__efficient_attention_backward (attention.cpp:579-727) + mem_eff_bwd (FlashAttention_internal.cpp:692-906):
+// inputs [B, S, H, D], the forward's bias and mask type, logsumexp [B, H, Sq].  No contiguous copies of q/k/v.
+// grad_bias: the reference allocates it (empty_like(bias) when bias_requires_grad, otherwise an uninitialised
+// [B*H, Sq, Sk], attention.cpp:664-671) but never passes it to the vendor call, so its contents are undefined there;
+// here it is computed when bias_requires_grad, in the shape of `bias`, and left undefined otherwise.
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> efficient_attention_backward(
+    const at::Tensor& grad_out_, const at::Tensor& query, const at::Tensor& key, const at::Tensor& value,
+    const std::optional<at::Tensor>& bias, const at::Tensor& out, const std::optional<at::Tensor>& cu_seqlens_q,
+    const std::optional<at::Tensor>& cu_seqlens_k, int64_t max_seqlen_q, int64_t max_seqlen_k,
+    const at::Tensor& logsumexp, double dropout_p, const at::Tensor& philox_seed, const at::Tensor& philox_offset,
+    int64_t custom_mask_type, bool bias_requires_grad, std::optional<double> scale,
+    std::optional<int64_t> num_splits_key, std::optional<int64_t> window_size, bool shared_storage_dqdkdv) {
+  (void)max_seqlen_q; (void)max_seqlen_k; (void)philox_seed; (void)philox_offset; (void)num_splits_key;
+  if (!grad_out_.defined()) return std::make_tuple(at::Tensor{}, at::Tensor{}, at::Tensor{}, at::Tensor{});  // :599-601
+  // the reference's shape checks (attention.cpp:602-625)
+  TORCH_CHECK(query.dim() == 4 && grad_out_.dim() == 4 && key.dim() == 4 && value.dim() == 4 && out.dim() == 4,
+              "grad_out, query, key, value and out must be 4-dimensional (batch, seq_len, num_heads, head_dim)");
+  TORCH_CHECK(query.size(0) == grad_out_.size(0) && query.size(0) == key.size(0) && query.size(0) == value.size(0),
+              "grad_out, query, key and value must have the same batch size");
+  TORCH_CHECK(key.size(1) == value.size(1), "key and value must have the same sequence length");
+  TORCH_CHECK(query.size(1) == grad_out_.size(1), "query and grad_out must have the same sequence length");
+  TORCH_CHECK(key.size(2) == value.size(2) && key.size(2) > 0 && query.size(2) % key.size(2) == 0,
+              "Number of heads in key/value must divide number of heads in query");
+  TORCH_CHECK(query.size(2) == grad_out_.size(2), "query and grad_out must have the same number of heads");
+  TORCH_CHECK(query.size(3) == key.size(3), "query and key must have the same head dimension");
+  TORCH_CHECK(value.size(3) == grad_out_.size(3) && value.size(3) == query.size(3),
+              "this build needs value.size(-1) == query.size(-1) == grad_out.size(-1)");
+  TORCH_CHECK(out.sizes() == grad_out_.sizes(), "out must have the shape of grad_out");
+  TORCH_CHECK(!(cu_seqlens_q.has_value() && cu_seqlens_q->defined()) && !(cu_seqlens_k.has_value() && cu_seqlens_k->defined()),
+              "efficient attention backward: cu_seqlens are not supported by this build (use _flash_attention_backward)");
+  TORCH_CHECK(!window_size.has_value() || *window_size <= 0, "efficient attention backward: sliding window is not supported");
+  TORCH_CHECK(dropout_p == 0.0, "efficient attention backward: dropout_p > 0 is not supported by this build");
+  TORCH_CHECK(custom_mask_type >= 0 && custom_mask_type <= 2, "custom_mask_type must be 0, 1 or 2");
+  // mem_eff_bwd's checks (FlashAttention_internal.cpp:714-758)
+  const auto dt = query.scalar_type();
+  TORCH_CHECK(dt == at::kHalf || dt == at::kBFloat16, "FlashAttention only support fp16 and bf16 data type");
+  TORCH_CHECK(key.scalar_type() == dt, "query and key must have the same dtype");
+  TORCH_CHECK(value.scalar_type() == dt, "query and value must have the same dtype");
+  TORCH_CHECK(out.scalar_type() == dt, "query and out must have the same dtype");
+  TORCH_CHECK(grad_out_.scalar_type() == dt, "query and dout must have the same dtype");
+  TORCH_CHECK(query.is_cuda() && key.is_cuda() && value.is_cuda(), "Input tensor must be on HIP device");
+  TORCH_CHECK(out.is_cuda(), "out tensor must be on HIP device");
+  TORCH_CHECK(grad_out_.is_cuda(), "dout tensor must be on HIP device");
+  TORCH_CHECK(logsumexp.is_cuda() && logsumexp.scalar_type() == at::kFloat, "softmax_lse tensor must be a float32 tensor on HIP device");
+  TORCH_CHECK(query.stride(-1) == 1 && key.stride(-1) == 1 && value.stride(-1) == 1,
+              "Input tensor must have contiguous last dimension");
+  const int64_t B = query.size(0), Sq = query.size(1), Hq = query.size(2), D = query.size(3);
+  const int64_t Sk = key.size(1), Hk = key.size(2);
+  TORCH_CHECK(B > 0, "batch size must be positive");
+  TORCH_CHECK(D <= 128, "FlashAttention backward only supports head dimension at most 128 in this build");
+  TORCH_CHECK(D % 8 == 0, "head dimension must be a multiple of 8");
+  TORCH_CHECK(Sq <= INT32_MAX && Sk <= INT32_MAX && B <= INT32_MAX, "sequence length too large");
+  TORCH_CHECK(logsumexp.dim() == 3 && logsumexp.size(0) == B && logsumexp.size(1) == Hq && logsumexp.size(2) >= Sq,
+              "logsumexp must have shape (batch_size, num_heads, seqlen_q): call the forward with compute_log_sumexp");
+
+  const c10::OptionalDeviceGuard guard(query.device());
+  const float softmax_scale = resolve_scale(query, scale);
+  auto fix = [](const at::Tensor& t) { return t.stride(-1) == 1 ? aligned_or_copy(t) : t.contiguous(); };
+  const at::Tensor q = aligned_or_copy(query), k = aligned_or_copy(key), v = aligned_or_copy(value);
+  const at::Tensor dout = fix(grad_out_), o = fix(out);  // the reference makes both contiguous (attention.cpp:646-650)
+  at::Tensor dq, dk, dv;
+  if (shared_storage_dqdkdv) {  // one [B, S, 3, H, D] allocation, the three gradients as its slices
+    TORCH_CHECK(Sq == Sk && Hq == Hk, "shared_storage_dqdkdv needs query and key of the same shape");
+    at::Tensor chunk = at::empty({B, Sq, 3, Hq, D}, q.options());
+    dq = chunk.select(2, 0); dk = chunk.select(2, 1); dv = chunk.select(2, 2);
+  } else {
+    dq = at::empty({B, Sq, Hq, D}, q.options());
+    dk = at::empty({B, Sk, Hk, D}, q.options());
+    dv = at::empty({B, Sk, Hk, D}, q.options());
+  }
+  const bool has_bias = bias.has_value() && bias->defined();
+  at::Tensor bias_e, dbias;
+  if (has_bias) bias_e = bias_for_kernels(*bias, dt, B, Hq, Sq, Sk);
+  const bool want_dbias = has_bias && bias_requires_grad;
+  if (want_dbias)  // rows padded to a multiple of 8 columns: every row start 16-byte aligned
+    dbias = at::empty({B, Hq, Sq, (Sk + 7) / 8 * 8}, q.options()).narrow(3, 0, Sk);
+
+  fa_bwd_params p{};
+  p.q = q.data_ptr(); p.k = k.data_ptr(); p.v = v.data_ptr(); p.out = o.data_ptr(); p.dout = dout.data_ptr();
+  p.lse = logsumexp.data_ptr<float>();
+  p.dq = dq.data_ptr(); p.dk = dk.data_ptr(); p.dv = dv.data_ptr();
+  fill_strides(q, false, p.q_stride_b, p.q_stride_s, p.q_stride_h);
+  fill_strides(k, false, p.k_stride_b, p.k_stride_s, p.k_stride_h);
+  fill_strides(v, false, p.v_stride_b, p.v_stride_s, p.v_stride_h);
+  fill_strides(o, false, p.o_stride_b, p.o_stride_s, p.o_stride_h);
+  fill_strides(dout, false, p.do_stride_b, p.do_stride_s, p.do_stride_h);
+  fill_strides(dq, false, p.dq_stride_b, p.dq_stride_s, p.dq_stride_h);
+  fill_strides(dk, false, p.dk_stride_b, p.dk_stride_s, p.dk_stride_h);
+  fill_strides(dv, false, p.dv_stride_b, p.dv_stride_s, p.dv_stride_h);
+  p.lse_stride_b = logsumexp.stride(0); p.lse_stride_h = logsumexp.stride(1); p.lse_stride_s = logsumexp.stride(2);
+  p.batch = static_cast<int32_t>(B);
+  p.heads_q = static_cast<int32_t>(Hq);
+  p.heads_k = static_cast<int32_t>(Hk);
+  p.seqlen_q = static_cast<int32_t>(Sq);
+  p.seqlen_k = static_cast<int32_t>(Sk);
+  p.head_dim = static_cast<int32_t>(D);
+  p.scale = softmax_scale;
+  p.dtype = dt == at::kBFloat16 ? FA_DTYPE_BF16 : FA_DTYPE_FP16;
+  p.is_causal = custom_mask_type == 1 ? FA_MASK_CAUSAL_TOP_LEFT
+                                      : (custom_mask_type == 2 ? FA_MASK_CAUSAL_BOTTOM_RIGHT : FA_MASK_NONE);
+  if (has_bias && Sk > 0) {
+    p.bias = bias_e.data_ptr();
+    p.bias_stride_b = bias_e.stride(0); p.bias_stride_h = bias_e.stride(1); p.bias_stride_q = bias_e.stride(2);
+    if (want_dbias) {
+      p.dbias = dbias.data_ptr();
+      p.dbias_stride_b = dbias.stride(0); p.dbias_stride_h = dbias.stride(1); p.dbias_stride_q = dbias.stride(2);
+    }
+  }
+  if (B * Sq * Hq == 0 || Sk == 0) {
+    dq.zero_(); dk.zero_(); dv.zero_();
+    if (want_dbias) dbias.zero_();
+  } else {
+    const size_t ws_bytes = fa_bwd_workspace_bytes(&p);
+    at::Tensor ws = at::empty({static_cast<int64_t>(ws_bytes > 0 ? ws_bytes : 16)}, q.options().dtype(at::kByte));
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
+    const int rc = fa_bwd_launch(&p, ws.data_ptr(), ws_bytes, stream);
+    TORCH_CHECK(rc == FA_OK, "fa_bwd_launch failed: ", fa_fwd_error_string(rc), " (rc=", rc, ")");
+    g_launches.fetch_add(1, std::memory_order_relaxed);
+  }
+  at::Tensor grad_bias;
+  if (want_dbias) {  // in the shape the caller's bias has: what was broadcast is summed
+    grad_bias = dbias;
+    if (bias->sizes() != dbias.sizes()) grad_bias = at::sum_to(dbias, bias->sizes());
+  }
+  return std::make_tuple(dq, dk, dv, grad_bias);
+}
+
+// ---- _scaled_dot_product_efficient_attention_backward ---------------------------------------------------------
+// cnnl__scaled_dot_product_efficient_attention_backward, attention.cpp:510-577: [B, H, S, D] in and out, causal from
+// the top-left corner (:547-549), the bias gradient asked for by grad_input_mask[3].
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> scaled_dot_product_efficient_attention_backward(
+    const at::Tensor& grad_out_, const at::Tensor& query, const at::Tensor& key, const at::Tensor& value,
+    const at::Tensor& attn_bias, const at::Tensor& out, const at::Tensor& logsumexp, const at::Tensor& philox_seed,
+    const at::Tensor& philox_offset, double dropout_p, std::array<bool, 4> grad_input_mask, bool is_causal,
+    std::optional<double> scale) {
+  if (!grad_out_.defined()) return std::make_tuple(at::Tensor{}, at::Tensor{}, at::Tensor{}, at::Tensor{});
+  TORCH_CHECK(query.dim() == 4 && key.dim() == 4 && value.dim() == 4 && grad_out_.dim() == 4 && out.dim() == 4,
+              "grad_out, query, key, value and out must be 4-dimensional (batch, num_heads, seq_len, head_dim)");
+  std::optional<at::Tensor> kernel_bias;  // an undefined tensor means "no bias" (attention.cpp:536-541)
+  if (attn_bias.defined()) kernel_bias = attn_bias;
+  auto [grad_q, grad_k, grad_v, grad_bias] = efficient_attention_backward(
+      grad_out_.transpose(1, 2), query.transpose(1, 2), key.transpose(1, 2), value.transpose(1, 2), kernel_bias,
+      out.transpose(1, 2), std::nullopt, std::nullopt, query.size(2), key.size(2), logsumexp, dropout_p, philox_seed,
+      philox_offset, is_causal ? 1 : 0, grad_input_mask[3], scale, std::nullopt, std::nullopt, false);
+  return std::make_tuple(grad_q.transpose(1, 2), grad_k.transpose(1, 2), grad_v.transpose(1, 2), grad_bias);
 }
 
 // ---- test hooks -----------------------------------------------------------------------------------------------
@@ -590,6 +732,9 @@ TORCH_LIBRARY_IMPL(aten, CUDA, m) {
   m.impl("_flash_attention_backward", TORCH_FN(torch_mlu_amd::flash_attention_backward));
   m.impl("_scaled_dot_product_efficient_attention", TORCH_FN(torch_mlu_amd::scaled_dot_product_efficient_attention));
   m.impl("_efficient_attention_forward", TORCH_FN(torch_mlu_amd::efficient_attention_forward));
+  m.impl("_scaled_dot_product_efficient_attention_backward",
+         TORCH_FN(torch_mlu_amd::scaled_dot_product_efficient_attention_backward));
+  m.impl("_efficient_attention_backward", TORCH_FN(torch_mlu_amd::efficient_attention_backward));
 }
 
 TORCH_LIBRARY(torch_mlu_amd, m) {

@@ -63,6 +63,11 @@ struct BArgs {
   float drop_rp;      // 1 / (1 - p)
   const int64_t* seed_ptr;    // the forward's philox_seed / philox_offset slots (device)
   const int64_t* offset_ptr;
+  int32_t causal_tl;          // causal mask aligned to the top-left corner (col <= row) instead of the bottom-right one
+  const unsigned char* bias;  // optional additive bias [b][h][row][col] through byte strides (dense mode only)
+  int64_t bias_sb, bias_sh, bias_sq;
+  unsigned char* dbias;       // optional gradient of the bias, same addressing
+  int64_t dbias_sb, dbias_sh, dbias_sq;
 };
 
 // One swizzle for tiles that are read both by rows (16 lanes = 16 consecutive rows, same logical chunk) and
@@ -87,7 +92,10 @@ struct TileIO {
 // ---------------------------------------------------------------------------------------------------------
 // dQ kernel
 // ---------------------------------------------------------------------------------------------------------
-template <typename T, int DP, bool DROP>
+// BIAS: the additive bias of this lane's query row is read straight from global memory into the score layout (8 bytes
+// = 4 consecutive keys per load, as in the forward); dS of the tile, already packed for the dQ product, is also what
+// the gradient of the bias is, and is stored from here (tiles the causal mask skips are stored as zeros).
+template <typename T, int DP, bool DROP, bool BIAS>
 __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
   using IO = TileIO<T, DP>;
   constexpr int CPR = IO::CPR, ROWB = IO::ROWB, TILE = IO::TILE, NI = IO::NI, RPI = IO::RPI, KS = IO::KS, MB = IO::MB;
@@ -141,7 +149,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
   const int nblk = (Lq + BM - 1) / BM;
   const int blk_first = (a.cu_q ? a.n_qslot : nblk) - 1 - pslot;
   if (blk_first < 0 || blk_first >= nblk) return;
-  const int off = Lk - Lq;
+  const int off = a.causal_tl ? 0 : Lk - Lq;
   const int D = a.head_dim;
   const int last_k = Lk - 1;
 
@@ -230,16 +238,66 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
   if constexpr (DROP)
     drop_row = drop_head_key((uint64_t)*a.seed_ptr, (uint64_t)*a.offset_ptr, (uint32_t)bh) ^ drop_row_term((uint32_t)row >> 1);
   const int drop_sh = 16 * (row & 1);
+  // bias / dBias of this lane's row, at its first key group (4 g)
+  const unsigned char* brow = nullptr;
+  unsigned char* dbrow = nullptr;
+  if constexpr (BIAS) {
+    const int64_t r = min(row, Lq - 1);
+    brow = a.bias + (int64_t)b * a.bias_sb + (int64_t)h * a.bias_sh + r * a.bias_sq + 8 * g;
+    if (a.dbias && row < Lq) dbrow = a.dbias + (int64_t)b * a.dbias_sb + (int64_t)h * a.dbias_sh + r * a.dbias_sq + 8 * g;
+  }
+  // chunk t of tile j holds dS of keys j BN + 32 (t >> 1) + 16 (t & 1) + 4 g + {0..3, 8..11} of this lane's row
+  auto store_dbias = [&](int j, int t, u32x4 w) {
+    if (!dbrow) return;
+    const int col = j * BN + 32 * (t >> 1) + 16 * (t & 1);
+    unsigned char* d = dbrow + col * 2;
+    if (j * BN + BN <= Lk) {
+      *(u32x2*)d = u32x2{w[0], w[1]};
+      *(u32x2*)(d + 16) = u32x2{w[2], w[3]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int e = 8 * (i >> 2) + (i & 3);
+        const uint32_t word = w[i >> 1];
+        if (col + 4 * g + e < Lk) *(unsigned short*)(d + e * 2) = (unsigned short)((i & 1) ? (word >> 16) : (word & 0xffffu));
+      }
+    }
+  };
 
   for (int j = 0; j < ntiles; ++j) {
     const int buf = j & 1;
     WAIT_VMCNT(0);
     __syncthreads();
     if (j + 1 < ntiles) issue_tile(j + 1, buf ^ 1);
-    if (a.is_causal && j * BN > wave_row_hi + off) continue;  // fully masked for this wavefront
+    if (a.is_causal && j * BN > wave_row_hi + off) {  // fully masked for this wavefront
+      if constexpr (BIAS) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) store_dbias(j, t, u32x4{0, 0, 0, 0});
+      }
+      continue;
+    }
 
     const unsigned char* kt = smem + buf * TILE;
     const unsigned char* vt = smem + 2 * TILE + buf * TILE;
+    // bias of a full tile: 8 loads of 4 keys each, issued now and consumed after the S / dP MFMAs
+    const bool full_tile = j * BN + BN <= Lk;
+    u32x2 braw[BIAS ? 8 : 1];
+    if constexpr (BIAS) {
+      if (full_tile) {
+        const unsigned char* bt = brow + (int64_t)j * (BN * 2);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) braw[i] = *(const u32x2*)(bt + (32 * (i >> 2) + 8 * (i & 3)) * 2);
+      } else {  // last, partial tile: element-wise, columns clamped to the last valid one (masked below anyway)
+        const unsigned short* be = (const unsigned short*)(brow + (int64_t)j * (BN * 2));
+        const int cmax = last_k - j * BN - 4 * g;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int e = 32 * (i >> 2) + 8 * (i & 3);
+          braw[i][0] = (uint32_t)be[min(e, cmax)] | ((uint32_t)be[min(e + 1, cmax)] << 16);
+          braw[i][1] = (uint32_t)be[min(e + 2, cmax)] | ((uint32_t)be[min(e + 3, cmax)] << 16);
+        }
+      }
+    }
     f32x16 s0, s1, p0, p1;
 #pragma unroll
     for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; p0[v] = 0.f; p1[v] = 0.f; }
@@ -288,13 +346,19 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
           const int e = 32 * (t >> 1) + 8 * (v >> 2) + (v & 3);
           const float sv = (t < 2) ? s0[v] : s1[v];
           float dpv = (t < 2) ? p0[v] : p1[v];
-          const float p = (e <= lim) ? fast_exp2(sv * c - lse2) : 0.f;
+          float xl = lse2;  // what is subtracted in the exponent: LSE - bias, in log2 units
+          if constexpr (BIAS) {
+            const uint32_t bw = braw[4 * (t >> 1) + (v >> 2)][(v & 3) >> 1];
+            xl = lse2 - Mma<T>::to_float((unsigned short)((v & 1) ? (bw >> 16) : (bw & 0xffffu))) * kLog2e;
+          }
+          const float p = (e <= lim) ? fast_exp2(sv * c - xl) : 0.f;
           if constexpr (DROP) dpv = (((word >> (8 * u)) & 0xffu) <= a.drop_thr) ? dpv * a.drop_rp : 0.f;
           ds[u] = p * (dpv - delta);
         }
         w[e2] = Mma<T>::pack2(ds[0], ds[1]);
       }
       dsb[t] = __builtin_bit_cast(s16x8, w);
+      if constexpr (BIAS) store_dbias(j, t, w);
     }
     // dQ^T += K^T dS^T; the transposed K fragments of chunk t + 1 are fetched while chunk t's MFMAs run
     {
@@ -318,6 +382,13 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+  }
+
+  if constexpr (BIAS) {  // key tiles beyond the causal bound of this block: dBias = 0
+    const int nall = (Lk + BN - 1) / BN;
+    for (int j = ntiles; j < nall; ++j)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) store_dbias(j, t, u32x4{0, 0, 0, 0});
   }
 
   if (row < Lq) {
@@ -346,7 +417,13 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
 // more); with head_dim <= 64 one launch produces both.
 constexpr int kDK = 1, kDV = 2;
 
-template <typename T, int DP, int WHAT, bool DROP>
+// BIAS: here a lane owns a key column and its registers run over query rows, while the bias is contiguous along keys.
+// A 32 x 32 block of it is therefore loaded as an MFMA A operand (a lane = one query row, 8 consecutive keys per
+// k-step: 8-byte loads) and multiplied by the identity: the product is the same block in the score layout, exact
+// (every output is one input times 1.0 plus zeros).  -inf entries are lowered to the most negative finite value
+// first, since -inf * 0 would turn the whole row into NaN; the exponential of either is 0.  The blocks of the next
+// (query head, query tile) are fetched one iteration ahead.
+template <typename T, int DP, int WHAT, bool DROP, bool BIAS>
 __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
   constexpr bool DO_K = (WHAT & kDK) != 0, DO_V = (WHAT & kDV) != 0;
   using IO = TileIO<T, DP>;
@@ -396,7 +473,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     lb = dlb = 0;
   }
   if (pslot * BKV >= Lk) return;
-  const int off = Lk - Lq;
+  const int off = a.causal_tl ? 0 : Lk - Lq;
   const int D = a.head_dim;
 
   const int dma_r = wave * RPI + lane / CPR;
@@ -482,6 +559,42 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
   };
   if (niter > 0) issue_iter(0, 0);
 
+  // ---- bias blocks of an iteration as A operands: [block of 32 query rows][k-step of 16 keys] ----
+  typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+  auto load_bias = [&](int it, u32x4 (&dst)[2][2]) {
+    const int hq = hk * a.group + it / nq;
+    const int jq = jq_begin + it % nq;
+    const unsigned char* bb = a.bias + (int64_t)b * a.bias_sb + (int64_t)hq * a.bias_sh;
+#pragma unroll
+    for (int qbk = 0; qbk < 2; ++qbk) {
+      const int64_t qr = min(jq * BQ + 32 * qbk + c32, Lq - 1);
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const int kvc = n0 + 32 * wave + 16 * ks + 8 * g;
+        const unsigned char* src = bb + qr * a.bias_sq + (int64_t)kvc * 2;
+        if (kvc + 8 <= Lk) {
+          const u32x2 lo = *(const u32x2*)src, hi = *(const u32x2*)(src + 8);
+          dst[qbk][ks] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        } else {
+          u32x4 w = {0, 0, 0, 0};
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (kvc + e < Lk) w[e >> 1] |= (uint32_t)((const unsigned short*)src)[e] << (16 * (e & 1));
+          dst[qbk][ks] = w;
+        }
+      }
+    }
+  };
+  u32x4 bnext[2][2];
+  s16x8 ident[2];  // B operand: rows 16 ks + 8 g + e of the 32 x 32 identity, column c32
+  if constexpr (BIAS) {
+    if (niter > 0) load_bias(0, bnext);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ident[ks][e] = (c32 == 16 * ks + 8 * g + e) ? (short)Mma<T>::kOne : (short)0;
+  }
+
   f32x16 dk[MB], dv[MB];
 #pragma unroll
   for (int i = 0; i < MB; ++i)
@@ -493,6 +606,19 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     WAIT_VMCNT(0);
     __syncthreads();
     if (it + 1 < niter) issue_iter(it + 1, buf ^ 1);
+    s16x8 bcur[2][2];
+    if constexpr (BIAS) {
+#pragma unroll
+      for (int qbk = 0; qbk < 2; ++qbk)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const u16x8 x = __builtin_bit_cast(u16x8, bnext[qbk][ks]);
+          const u16x8 lim8 = {Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax,
+                              Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax};
+          bcur[qbk][ks] = __builtin_bit_cast(s16x8, __builtin_elementwise_min(x, lim8));
+        }
+      if (it + 1 < niter) load_bias(it + 1, bnext);
+    }
     const int jq = jq_begin + it % nq;
     const int qlo = jq * BQ;
     // every (q, kv) of this tile masked for this wavefront: q + off < kv for all pairs
@@ -526,9 +652,13 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
         lv[q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
         if constexpr (DO_K) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
       }
-      f32x16 s, dp;
+      f32x16 s, dp, bacc;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; }
+      for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; bacc[v] = 0.f; }
+      if constexpr (BIAS) {
+        bacc = Mma<T>::m32(bcur[qbk][0], ident[0], bacc);
+        bacc = Mma<T>::m32(bcur[qbk][1], ident[1], bacc);
+      }
       {
         // Q (and dO) row fragments are fetched two k-steps ahead of the MFMAs that consume them
         s16x8 qa[2], da[2];
@@ -556,7 +686,11 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
 #pragma unroll
         for (int e2 = 0; e2 < 4; ++e2) {
           const int v = 8 * t + 2 * e2;  // v, v + 1: consecutive query rows
-          const float l0 = lv[v >> 2][v & 3] * kLog2e, l1 = lv[v >> 2][(v & 3) + 1] * kLog2e;
+          float l0 = lv[v >> 2][v & 3] * kLog2e, l1 = lv[v >> 2][(v & 3) + 1] * kLog2e;
+          if constexpr (BIAS) {
+            l0 -= bacc[v] * kLog2e;
+            l1 -= bacc[v + 1] * kLog2e;
+          }
           const float d0 = DO_K ? dl[v >> 2][v & 3] : 0.f, d1 = DO_K ? dl[v >> 2][(v & 3) + 1] : 0.f;
           float p0 = fast_exp2(s[v] * c - l0), p1 = fast_exp2(s[v + 1] * c - l1);
           if (need_mask) {
@@ -649,6 +783,21 @@ int bwd_validate(const fa_bwd_params* p) {
                              (((uintptr_t)p->philox_seed | (uintptr_t)p->philox_offset) & 7)))
     return FA_ERR_BAD_ARG;
   if (p->cu_seqlens_q && p->total_q < 0) return FA_ERR_BAD_ARG;
+  if (p->is_causal != FA_MASK_NONE && p->is_causal != FA_MASK_CAUSAL_BOTTOM_RIGHT && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT)
+    return FA_ERR_BAD_ARG;
+  if (p->dbias && !p->bias) return FA_ERR_BAD_ARG;
+  if (p->bias) {
+    if (((uintptr_t)p->bias & 7) || p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_q < 0 ||
+        ((p->bias_stride_b | p->bias_stride_h | p->bias_stride_q) & 3))
+      return FA_ERR_BAD_ARG;
+    if (p->cu_seqlens_q || p->dropout_p > 0.f) return FA_ERR_UNSUPPORTED;
+  }
+  if (p->dbias) {  // an output: aligned like the bias and not broadcast
+    if (((uintptr_t)p->dbias & 7) || ((p->dbias_stride_b | p->dbias_stride_h | p->dbias_stride_q) & 3)) return FA_ERR_BAD_ARG;
+    if (p->dbias_stride_q < p->seqlen_k || (p->seqlen_q > 1 && p->dbias_stride_q <= 0) ||
+        (p->heads_q > 1 && p->dbias_stride_h <= 0) || (p->batch > 1 && p->dbias_stride_b <= 0))
+      return FA_ERR_BAD_ARG;
+  }
   if (p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_UNSUPPORTED;
   if (p->head_dim > 128 || (p->head_dim & 7)) return FA_ERR_UNSUPPORTED;
   if (p->heads_q % p->heads_k) return FA_ERR_UNSUPPORTED;
@@ -679,14 +828,14 @@ size_t bwd_ws_bytes(const fa_bwd_params* p) {
   return (rows * p->heads_q * 4 + 15) & ~(size_t)15;
 }
 
-template <typename T, int DP, bool DROP>
+template <typename T, int DP, bool DROP, bool BIAS>
 int bwd_launch(const BArgs& a, hipStream_t st) {
   constexpr int lds_dq = 4 * 64 * DP * 2;
   constexpr int lds_dkv = 4 * 64 * DP * 2 + 4 * 256;
   constexpr bool split = DP > 64;  // head_dim 128: dK and dV as two launches
-  constexpr auto kq = fa_bwd_dq_kernel<T, DP, DROP>;
-  constexpr auto kkv = fa_bwd_dkv_kernel<T, DP, split ? kDK : (kDK | kDV), DROP>;
-  constexpr auto kv2 = fa_bwd_dkv_kernel<T, DP, kDV, DROP>;
+  constexpr auto kq = fa_bwd_dq_kernel<T, DP, DROP, BIAS>;
+  constexpr auto kkv = fa_bwd_dkv_kernel<T, DP, split ? kDK : (kDK | kDV), DROP, BIAS>;
+  constexpr auto kv2 = fa_bwd_dkv_kernel<T, DP, kDV, DROP, BIAS>;
   if (!ensure_dynamic_lds<kq>(lds_dq) || !ensure_dynamic_lds<kkv>(lds_dkv) || (split && !ensure_dynamic_lds<kv2>(lds_dkv)))
     return FA_ERR_LAUNCH;
   const int64_t gq = (int64_t)a.batch * a.heads_q * a.n_qslot;
@@ -745,7 +894,12 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   }
   a.batch = p->batch; a.heads_q = p->heads_q; a.heads_k = p->heads_k; a.group = p->heads_q / p->heads_k;
   a.seqlen_q = p->seqlen_q; a.seqlen_k = p->seqlen_k; a.head_dim = p->head_dim;
-  a.is_causal = p->is_causal ? 1 : 0;
+  a.is_causal = p->is_causal != FA_MASK_NONE ? 1 : 0;
+  a.causal_tl = p->is_causal == FA_MASK_CAUSAL_TOP_LEFT ? 1 : 0;
+  a.bias = (const unsigned char*)p->bias;
+  a.bias_sb = p->bias_stride_b * 2; a.bias_sh = p->bias_stride_h * 2; a.bias_sq = p->bias_stride_q * 2;
+  a.dbias = (unsigned char*)p->dbias;
+  a.dbias_sb = p->dbias_stride_b * 2; a.dbias_sh = p->dbias_stride_h * 2; a.dbias_sq = p->dbias_stride_q * 2;
   a.n_qslot = (p->seqlen_q + 127) / 128;
   a.n_kslot = (p->seqlen_k + 127) / 128;
   a.blockmajor_q = a.is_causal && (int64_t)p->batch * p->heads_q * a.n_qslot < 8 * 256;
@@ -761,12 +915,17 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   const int dp = p->head_dim <= 64 ? 64 : 128;
   if (p->dropout_p > 0.f) {
     if (p->dtype == FA_DTYPE_BF16)
-      return dp == 64 ? bwd_launch<__bf16, 64, true>(a, st) : bwd_launch<__bf16, 128, true>(a, st);
-    return dp == 64 ? bwd_launch<_Float16, 64, true>(a, st) : bwd_launch<_Float16, 128, true>(a, st);
+      return dp == 64 ? bwd_launch<__bf16, 64, true, false>(a, st) : bwd_launch<__bf16, 128, true, false>(a, st);
+    return dp == 64 ? bwd_launch<_Float16, 64, true, false>(a, st) : bwd_launch<_Float16, 128, true, false>(a, st);
+  }
+  if (p->bias) {
+    if (p->dtype == FA_DTYPE_BF16)
+      return dp == 64 ? bwd_launch<__bf16, 64, false, true>(a, st) : bwd_launch<__bf16, 128, false, true>(a, st);
+    return dp == 64 ? bwd_launch<_Float16, 64, false, true>(a, st) : bwd_launch<_Float16, 128, false, true>(a, st);
   }
   if (p->dtype == FA_DTYPE_BF16)
-    return dp == 64 ? bwd_launch<__bf16, 64, false>(a, st) : bwd_launch<__bf16, 128, false>(a, st);
-  return dp == 64 ? bwd_launch<_Float16, 64, false>(a, st) : bwd_launch<_Float16, 128, false>(a, st);
+    return dp == 64 ? bwd_launch<__bf16, 64, false, false>(a, st) : bwd_launch<__bf16, 128, false, false>(a, st);
+  return dp == 64 ? bwd_launch<_Float16, 64, false, false>(a, st) : bwd_launch<_Float16, 128, false, false>(a, st);
 }
 
 }  // extern "C"

@@ -41,6 +41,9 @@ struct Mma<__bf16> {
     f32x2 f = {a, b};
     return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
   }
+  static __device__ __forceinline__ float to_float(unsigned short bits) { return __builtin_bit_cast(float, (unsigned)bits << 16); }
+  static constexpr unsigned short kOne = 0x3f80;     // 1.0
+  static constexpr unsigned short kNegMax = 0xff7f;  // the most negative finite value; -inf is the next bit pattern
 };
 template <>
 struct Mma<_Float16> {
@@ -54,6 +57,9 @@ struct Mma<_Float16> {
     f32x2 f = {a, b};
     return __builtin_bit_cast(unsigned, __builtin_convertvector(f, f16x2));
   }
+  static __device__ __forceinline__ float to_float(unsigned short bits) { return (float)__builtin_bit_cast(_Float16, bits); }
+  static constexpr unsigned short kOne = 0x3c00;
+  static constexpr unsigned short kNegMax = 0xfbff;
 };
 
 // 16-byte global -> LDS DMA.  Lane i of the wavefront writes LDS bytes [lds_wave_base + 16 i, +16); the global

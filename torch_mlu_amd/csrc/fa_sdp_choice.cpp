@@ -6,7 +6,7 @@
 // (sdp_utils.h:475-524: device series, "split condition", "valid data ratio") and the xformers-derived priority order
 // (sdp_utils.cpp:8-53): on MI355X the flash kernels of this build are preferred whenever they are eligible — they
 // take GQA, head dims up to 256, and single-query decode (split-KV) —, then its mem-efficient entry points (additive
-// attn_mask, top-left causal on non-square problems; inference only), and everything else is left to PyTorch's own
+// attn_mask, top-left causal on non-square problems), and everything else is left to PyTorch's own
 // choice among its remaining backends.
 #include <ATen/ATen.h>
 #include <ATen/Context.h>
@@ -195,15 +195,18 @@ bool check_head_dim_size_mem_efficient(const sdp_params& p, bool debug) {
   return true;
 }
 
-// Not in the reference (its mem-efficient path has a backward and dropout): what this build's does not implement.
+// Not in the reference (its mem-efficient path takes dropout, and its backward is the vendor's): what this build's
+// does not implement.
 bool check_this_build_mem_efficient(const sdp_params& p, bool debug) {
   if (p.dropout > 0.0) {
     if (debug) TORCH_WARN("The mem-efficient kernels of this build do not implement dropout (dropout_p must be 0).");
     return false;
   }
   const bool mask_grad = p.attn_mask.has_value() && p.attn_mask->defined() && p.attn_mask->requires_grad();
-  if (input_requires_grad(p) || (at::GradMode::is_enabled() && mask_grad)) {
-    if (debug) TORCH_WARN("The mem-efficient entry points of this build have no backward; a gradient is required.");
+  if ((input_requires_grad(p) || (at::GradMode::is_enabled() && mask_grad)) && p.query.size(-1) > 128) {
+    if (debug)
+      TORCH_WARN("The backward of this build stops at head dimension 128; a gradient is required and query.size(-1) is ",
+                 p.query.size(-1), ".");
     return false;
   }
   if (p.attn_mask.has_value() && p.attn_mask->defined()) {
