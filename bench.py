@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the flash-attention forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop|cfg2_mask_bwd] [--no-extras] [--no-cpu-baseline]
 
 A "step" is one call of the registered op on one batch of seeded synthetic input that is already resident in HBM.
 The headline workload is BASELINE.json configs[1] (causal prefill, bf16 MHA, B=4 H=32 S=4096 D=128); the other
@@ -115,6 +115,25 @@ def make_workload(name, dev):
         return dict(call=call, check=check, flops=4 * B * H * S * S * D, bytes_kv=2 * B * H * S * D * 2,
                     desc=f"non-causal prefill with additive [B,1,S,S] mask bf16 B={B} H={H} S={S} D={D}", dtype="bf16",
                     bound="mfma", kernel="fa_tile_kernel<bias>")
+    if name == "cfg2_mask_bwd":
+        # the backward of cfg2_mask (the mask takes no gradient: what an attn_mask built from padding looks like)
+        B, H, S, D = 4, 32, 4096, 128
+        q, k, v, do = (seeded((B, H, S, D), 1 + i, bf).to(dev) for i in range(4))
+        bias = seeded((B, 1, S, S), 9, bf, std=1.0).to(dev)
+        bias_e = bias.expand(B, H, S, S)
+        out, lse, ps, po = aten._scaled_dot_product_efficient_attention(q, k, v, bias_e, True)
+
+        def call():
+            return aten._scaled_dot_product_efficient_attention_backward(do, q, k, v, bias_e, out, lse, ps, po, 0.0,
+                                                                         [True, True, True, False], False)
+
+        def check():
+            return _check_grads(q, k, v, do, call(), [(0, 0), (B - 1, H - 1)], causal=False, bias=bias)
+
+        return dict(call=call, check=check, flops=10 * B * H * S * S * D, bytes_kv=2 * B * H * S * D * 2,
+                    desc=f"backward of non-causal prefill with additive [B,1,S,S] mask bf16 B={B} H={H} S={S} D={D}",
+                    dtype="bf16", bound="mfma",
+                    kernel="fa_bwd_dq_kernel<bias> + fa_bwd_dkv_kernel<dK, bias> + fa_bwd_dkv_kernel<dV, bias>")
     if name == "cfg4":
         g = torch.Generator().manual_seed(3)
         lens = torch.randint(256, 2049, (16,), generator=g).tolist()
@@ -199,9 +218,9 @@ def _check_heads(q, k, v, out, lse, causal, heads, bias=None, keep=None, dropout
     return eo, el
 
 
-def _check_grads(q, k, v, do, grads, heads):
+def _check_grads(q, k, v, do, grads, heads, causal=True, bias=None):
     """max-abs error of dQ / of dK and dV on sampled (batch, head) pairs against autograd through fp32 math on the
-    device (causal, MHA).  Returned in the (out, lse) slots of the bench record: (dQ error, max of dK and dV error)."""
+    device (MHA).  Returned in the (out, lse) slots of the bench record: (dQ error, max of dK and dV error)."""
     Sq, Sk, D = q.shape[2], k.shape[2], q.shape[3]
     r = torch.arange(Sq, device=q.device)[:, None]
     c = torch.arange(Sk, device=q.device)[None, :]
@@ -209,7 +228,10 @@ def _check_grads(q, k, v, do, grads, heads):
     for b, h in heads:
         qq, kk, vv = (t[b, h].float().clone().requires_grad_() for t in (q, k, v))
         s = (qq @ kk.T) / math.sqrt(D)
-        s = s.masked_fill(c > r + Sk - Sq, float("-inf"))
+        if bias is not None:
+            s = s + bias[b, 0].float()
+        if causal:
+            s = s.masked_fill(c > r + Sk - Sq, float("-inf"))
         (torch.softmax(s, -1) @ vv).backward(do[b, h].float())
         eq = max(eq, (grads[0][b, h].float() - qq.grad).abs().max().item())
         ekv = max(ekv, (grads[1][b, h].float() - kk.grad).abs().max().item(),
@@ -277,7 +299,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "copy1g"])
+    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "copy1g"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -322,7 +344,7 @@ def main():
     main_r = run(args.config, args.steps, args.warmup)
     extras = []
     if not args.no_extras:
-        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask", "cfg2_drop"):
+        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd"):
             if name != args.config:
                 extras.append(run(name, args.steps, args.warmup))
 
@@ -343,7 +365,8 @@ def main():
         "config": {"workload": main_r["workload"], "name": args.config,
                    "entry": {"cfg4": "aten::_flash_attention_forward",
                              "cfg2_bwd": "aten::_scaled_dot_product_flash_attention_backward",
-                             "cfg2_mask": "aten::_scaled_dot_product_efficient_attention"}.get(
+                             "cfg2_mask": "aten::_scaled_dot_product_efficient_attention",
+                             "cfg2_mask_bwd": "aten::_scaled_dot_product_efficient_attention_backward"}.get(
                                  args.config, "aten::_scaled_dot_product_flash_attention")},
         "roofline": main_r["roofline"],
         "parity": dict({k: v for k, v in main_r.items() if k.startswith("max_abs_err")},

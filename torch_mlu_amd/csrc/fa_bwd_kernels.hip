@@ -279,7 +279,8 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
 
     const unsigned char* kt = smem + buf * TILE;
     const unsigned char* vt = smem + 2 * TILE + buf * TILE;
-    // bias of a full tile: 8 loads of 4 keys each, issued now and consumed after the S / dP MFMAs
+    // bias of this tile: 8 loads of 4 keys each (a partial last tile: element-wise, columns clamped to the last valid
+    // one, masked below anyway), issued now and consumed after the S / dP MFMAs
     const bool full_tile = j * BN + BN <= Lk;
     u32x2 braw[BIAS ? 8 : 1];
     if constexpr (BIAS) {
@@ -287,7 +288,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
         const unsigned char* bt = brow + (int64_t)j * (BN * 2);
 #pragma unroll
         for (int i = 0; i < 8; ++i) braw[i] = *(const u32x2*)(bt + (32 * (i >> 2) + 8 * (i & 3)) * 2);
-      } else {  // last, partial tile: element-wise, columns clamped to the last valid one (masked below anyway)
+      } else {
         const unsigned short* be = (const unsigned short*)(brow + (int64_t)j * (BN * 2));
         const int cmax = last_k - j * BN - 4 * g;
 #pragma unroll
@@ -421,8 +422,8 @@ constexpr int kDK = 1, kDV = 2;
 // A 32 x 32 block of it is therefore loaded as an MFMA A operand (a lane = one query row, 8 consecutive keys per
 // k-step: 8-byte loads) and multiplied by the identity: the product is the same block in the score layout, exact
 // (every output is one input times 1.0 plus zeros).  -inf entries are lowered to the most negative finite value
-// first, since -inf * 0 would turn the whole row into NaN; the exponential of either is 0.  The blocks of the next
-// (query head, query tile) are fetched one iteration ahead.
+// first, since -inf * 0 would turn the whole row into NaN; the exponential of either is 0.  A block's loads are issued
+// ahead of its S / dP MFMAs and consumed after them.
 template <typename T, int DP, int WHAT, bool DROP, bool BIAS>
 __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
   constexpr bool DO_K = (WHAT & kDK) != 0, DO_V = (WHAT & kDV) != 0;
@@ -559,36 +560,31 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
   };
   if (niter > 0) issue_iter(0, 0);
 
-  // ---- bias blocks of an iteration as A operands: [block of 32 query rows][k-step of 16 keys] ----
+  // ---- one 32 x 32 bias block (block qbk of iteration it) as A operands: [k-step of 16 keys] ----
   typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
-  auto load_bias = [&](int it, u32x4 (&dst)[2][2]) {
+  auto load_bias = [&](int it, int qbk, u32x4 (&dst)[2]) {
     const int hq = hk * a.group + it / nq;
     const int jq = jq_begin + it % nq;
-    const unsigned char* bb = a.bias + (int64_t)b * a.bias_sb + (int64_t)hq * a.bias_sh;
+    const int64_t qr = min(jq * BQ + 32 * qbk + c32, Lq - 1);
+    const unsigned char* src0 = a.bias + (int64_t)b * a.bias_sb + (int64_t)hq * a.bias_sh + qr * a.bias_sq;
 #pragma unroll
-    for (int qbk = 0; qbk < 2; ++qbk) {
-      const int64_t qr = min(jq * BQ + 32 * qbk + c32, Lq - 1);
+    for (int ks = 0; ks < 2; ++ks) {
+      const int kvc = n0 + 32 * wave + 16 * ks + 8 * g;
+      const unsigned char* src = src0 + (int64_t)kvc * 2;
+      if (kvc + 8 <= Lk) {
+        const u32x2 lo = *(const u32x2*)src, hi = *(const u32x2*)(src + 8);
+        dst[ks] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      } else {
+        u32x4 w = {0, 0, 0, 0};
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const int kvc = n0 + 32 * wave + 16 * ks + 8 * g;
-        const unsigned char* src = bb + qr * a.bias_sq + (int64_t)kvc * 2;
-        if (kvc + 8 <= Lk) {
-          const u32x2 lo = *(const u32x2*)src, hi = *(const u32x2*)(src + 8);
-          dst[qbk][ks] = u32x4{lo[0], lo[1], hi[0], hi[1]};
-        } else {
-          u32x4 w = {0, 0, 0, 0};
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (kvc + e < Lk) w[e >> 1] |= (uint32_t)((const unsigned short*)src)[e] << (16 * (e & 1));
-          dst[qbk][ks] = w;
-        }
+        for (int e = 0; e < 8; ++e)
+          if (kvc + e < Lk) w[e >> 1] |= (uint32_t)((const unsigned short*)src)[e] << (16 * (e & 1));
+        dst[ks] = w;
       }
     }
   };
-  u32x4 bnext[2][2];
   s16x8 ident[2];  // B operand: rows 16 ks + 8 g + e of the 32 x 32 identity, column c32
   if constexpr (BIAS) {
-    if (niter > 0) load_bias(0, bnext);
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
@@ -606,19 +602,6 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     WAIT_VMCNT(0);
     __syncthreads();
     if (it + 1 < niter) issue_iter(it + 1, buf ^ 1);
-    s16x8 bcur[2][2];
-    if constexpr (BIAS) {
-#pragma unroll
-      for (int qbk = 0; qbk < 2; ++qbk)
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-          const u16x8 x = __builtin_bit_cast(u16x8, bnext[qbk][ks]);
-          const u16x8 lim8 = {Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax,
-                              Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax};
-          bcur[qbk][ks] = __builtin_bit_cast(s16x8, __builtin_elementwise_min(x, lim8));
-        }
-      if (it + 1 < niter) load_bias(it + 1, bnext);
-    }
     const int jq = jq_begin + it % nq;
     const int qlo = jq * BQ;
     // every (q, kv) of this tile masked for this wavefront: q + off < kv for all pairs
@@ -646,19 +629,22 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     for (int qbk = 0; qbk < 2; ++qbk) {  // two blocks of 32 query rows
       // LSE and delta of this lane's 16 rows (register v <-> row 32 qbk + 8 (v >> 2) + 4 g + (v & 3)), fetched ahead
       // of the MFMAs that hide their latency
+      // (with a bias the registers are needed elsewhere and the two vectors are read after the MFMAs; in halves
+      // where the dK accumulators of head_dim 128 leave no room)
+      constexpr bool HALVES = BIAS && DO_K && DP > 64;
       f32x4 lv[4], dl[4];
+      if constexpr (!BIAS) {
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        lv[q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
-        if constexpr (DO_K) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
+        for (int q4 = 0; q4 < 4; ++q4) {
+          lv[q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
+          if constexpr (DO_K) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
+        }
       }
       f32x16 s, dp, bacc;
 #pragma unroll
       for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; bacc[v] = 0.f; }
-      if constexpr (BIAS) {
-        bacc = Mma<T>::m32(bcur[qbk][0], ident[0], bacc);
-        bacc = Mma<T>::m32(bcur[qbk][1], ident[1], bacc);
-      }
+      u32x4 braw[2];  // this block's bias, requested now, used after the S / dP MFMAs
+      if constexpr (BIAS) load_bias(it, qbk, braw);
       {
         // Q (and dO) row fragments are fetched two k-steps ahead of the MFMAs that consume them
         s16x8 qa[2], da[2];
@@ -679,10 +665,38 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+      if constexpr (BIAS) {
+        // the bias through the matrix unit into the score layout
+        s16x8 bcur[2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const u16x8 x = __builtin_bit_cast(u16x8, braw[ks]);
+          const u16x8 lim8 = {Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax,
+                              Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax, Mma<T>::kNegMax};
+          bcur[ks] = __builtin_bit_cast(s16x8, __builtin_elementwise_min(x, lim8));
+        }
+        bacc = Mma<T>::m32(bcur[0], ident[0], bacc);
+        bacc = Mma<T>::m32(bcur[1], ident[1], bacc);
+        if constexpr (!HALVES) {
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            lv[q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
+            if constexpr (DO_K) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
+          }
+        }
+      }
       s16x8 pb[2], dsb[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         u32x4 wp, wd;
+        if constexpr (HALVES) {  // LSE and delta of this half's 8 rows only, to keep the register count down
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int q4 = 2 * t; q4 < 2 * t + 2; ++q4) {
+            lv[q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
+            if constexpr (DO_K) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
+          }
+        }
 #pragma unroll
         for (int e2 = 0; e2 < 4; ++e2) {
           const int v = 8 * t + 2 * e2;  // v, v + 1: consecutive query rows
