@@ -8,7 +8,7 @@
  *   cnnlCreate/SetFlashAttentionDescriptor + CnnlTensorDescriptor::set x8 (:131-180)  -> fa_fwd_params (one POD struct)
  *   cnnlGetFlashAttentionForwardWorkspaceSize_v2 (:215-228)                         -> fa_fwd_workspace_bytes
  *   cnnlFlashAttentionForward_v2 (:231-258)                                         -> fa_fwd_launch
- *   cnnlGetFlashAttentionGeneratedRandomNumbers (:181-197)                          -> not needed: dropout_p must be 0
+ *   cnnlGetFlashAttentionGeneratedRandomNumbers (:181-197)                          -> not needed: one (seed, offset) pair per call
  *
  * Plain C: pointers, sizes and strides only.  No torch types, no exceptions, no allocation, no
  * host/device synchronisation, no global mutable state: the library may be dlopen()ed from any

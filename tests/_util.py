@@ -60,3 +60,37 @@ def out_close(got, want, dtype, tol=None):
 
 def default_scale(d):
     return 1.0 / math.sqrt(d)
+
+
+def algorithm_rounding_error(q, k, v, dout, dtype, is_causal=False, causal_top_left=False, scale=None, attn_bias=None,
+                             dropout_p=0.0, dropout_mask=None):
+    """What the two roundings every flash backward makes cost, per gradient (dq, dk, dv, dbias): delta = rowsum(dO o O)
+    is formed from the forward's output O as stored in `dtype`, and P, dS enter the matrix products rounded to
+    `dtype`.  Everything else is exact here (float64), so the result is the error floor of the algorithm on these
+    inputs, against which a kernel's own error can be judged (the reference's tests judge theirs against the error
+    of low-precision math in the same spirit, test_scaled_dot_product_attention.py:188-204)."""
+    import oracle
+
+    def rnd(x):
+        return torch.from_numpy(np.ascontiguousarray(x)).to(dtype).double().numpy()
+
+    qn, kn, vn, don = (t.double().numpy() for t in (q, k, v, dout))
+    B, Hq, Sq, D = qn.shape
+    Hk, Sk = kn.shape[1], kn.shape[2]
+    g = Hq // Hk
+    sc = (1.0 / math.sqrt(D)) if scale is None else float(scale)
+    kw = dict(is_causal=is_causal, causal_top_left=causal_top_left, scale=scale, attn_bias=attn_bias,
+              dropout_p=dropout_p, dropout_mask=dropout_mask)
+    want = oracle.sdpa_backward_oracle(q, k, v, dout, return_dbias=True, **kw)
+    out, p, _ = oracle.attention_ref(qn.transpose(0, 2, 1, 3), kn.transpose(0, 2, 1, 3), vn.transpose(0, 2, 1, 3),
+                                     scale=scale, causal=is_causal, causal_top_left=causal_top_left,
+                                     attn_bias=attn_bias, dropout_p=dropout_p, dropout_mask=dropout_mask)
+    m = np.ones_like(p) if dropout_mask is None else np.asarray(dropout_mask, dtype=np.float64)
+    r = 1.0 / (1.0 - dropout_p)
+    kr, vr = np.repeat(kn, g, axis=1), np.repeat(vn, g, axis=1)
+    delta = (don * rnd(out)).sum(-1, keepdims=True)
+    ds = rnd(p * (np.matmul(don, vr.transpose(0, 1, 3, 2)) * m * r - delta))
+    dq = sc * np.matmul(ds, kr)
+    dk = (sc * np.matmul(ds.transpose(0, 1, 3, 2), qn)).reshape(B, Hk, g, Sk, D).sum(2)
+    dv = np.matmul(rnd(p * m * r).transpose(0, 1, 3, 2), don).reshape(B, Hk, g, Sk, D).sum(2)
+    return tuple(float(np.abs(a - w).max()) if a.size else 0.0 for a, w in zip((dq, dk, dv, ds), want))

@@ -162,6 +162,8 @@ def test_bwd_validate_accepts_good_params_and_sizes_delta_scratch():
                      bias_stride_q=256, dbias=0xd000, dbias_stride_b=8 * 128 * 256, dbias_stride_h=128 * 256,
                      dbias_stride_q=256)
     assert L.fa_bwd_validate(ctypes.byref(full)) == capi.FA_OK
+    full.dropout_p, full.philox_seed, full.philox_offset = 0.1, 0xe000, 0xe008     # bias and dropout together
+    assert L.fa_bwd_validate(ctypes.byref(full)) == capi.FA_OK
 
 
 @pytest.mark.parametrize("over,rc", [
@@ -183,8 +185,6 @@ def test_bwd_validate_accepts_good_params_and_sizes_delta_scratch():
     (dict(dbias=0xd000, dbias_stride_q=256), capi.FA_ERR_BAD_ARG),          # a bias gradient without a bias
     (dict(bias=0xc000, bias_stride_q=256, dbias=0xd000, dbias_stride_q=0), capi.FA_ERR_BAD_ARG),   # broadcast output
     (dict(bias=0xc000, bias_stride_q=256, dbias=0xd000, dbias_stride_q=256, dbias_stride_h=0), capi.FA_ERR_BAD_ARG),
-    (dict(bias=0xc000, bias_stride_q=256, dropout_p=0.1, philox_seed=0xe000, philox_offset=0xe008),
-     capi.FA_ERR_UNSUPPORTED),
     (dict(bias=0xc000, bias_stride_q=256, cu_seqlens_q=0xa000, cu_seqlens_k=0xb000, total_q=200), capi.FA_ERR_UNSUPPORTED),
 ])
 def test_bwd_validate_rejects(over, rc):

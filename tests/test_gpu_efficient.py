@@ -111,8 +111,8 @@ def test_efficient_attention_forward_op_layout_and_mask_types():
 
 def test_errors():
     q, k, v = (t.to(DEV) for t in _qkv(1, 2, 2, 16, 16, 64, HF))
-    with pytest.raises(RuntimeError, match="dropout"):
-        aten._scaled_dot_product_efficient_attention(q, k, v, None, False, 0.1)
+    with pytest.raises(RuntimeError, match="dropout_p must be in"):
+        aten._scaled_dot_product_efficient_attention(q, k, v, None, False, 1.0)
     with pytest.raises(RuntimeError, match="same dtype as query"):
         aten._scaled_dot_product_efficient_attention(q, k, v, torch.zeros(16, 16, device=DEV), False)
     with pytest.raises(RuntimeError, match="only support fp16 and bf16"):

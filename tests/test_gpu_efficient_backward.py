@@ -274,8 +274,8 @@ def test_backward_op_errors():
     args = lambda **o: aten._efficient_attention_backward(
         o.get("do", do), q, k, v, o.get("bias"), out, o.get("cu"), o.get("cu"), mq, mk, o.get("lse", lse),
         o.get("p", 0.0), seed, offset, o.get("cmt", 0), False)
-    with pytest.raises(RuntimeError, match="dropout"):
-        args(p=0.2)
+    with pytest.raises(RuntimeError, match="dropout_p must be in"):
+        args(p=1.5)
     with pytest.raises(RuntimeError, match="cu_seqlens are not supported"):
         args(cu=torch.zeros(2, dtype=torch.int32, device=DEV))
     with pytest.raises(RuntimeError, match="custom_mask_type"):
@@ -330,3 +330,90 @@ def test_training_non_square_causal_through_plain_sdpa():
     want = oracle.sdpa_backward_oracle(q, k, v, do, is_causal=True, causal_top_left=True)
     for name, t, w in zip(("dq", "dk", "dv"), (qd, kd, vd), want):
         _close(name, t.grad, w, HF)
+
+
+# ---- dropout on the mem-efficient path (with and without a bias) ------------------------------------------------------
+def _keep(seed, offset, B, Hq, Sq, Sk, p):
+    return np.stack([np.stack([oracle.dropout_keep_mask(seed, offset, b * Hq + h, Sq, Sk, p) for h in range(Hq)])
+                     for b in range(B)])
+
+
+@pytest.mark.parametrize("dtype,D", [(BF, 128), (HF, 64), (BF, 32)])
+@pytest.mark.parametrize("mask", ["none", "tl"])
+def test_bias_with_dropout_through_c_abi(dtype, D, mask):
+    """Bias and dropout together, forward and backward, against the oracle fed with this build's keep-mask (the
+    reference tests' criterion for dropout, test_scaled_dot_product_attention.py:1049-1070)."""
+    for i, (B, Hq, Hk, Sq, Sk, p) in enumerate([(2, 4, 2, 130, 131, 0.1), (1, 2, 2, 257, 65, 0.5), (1, 4, 1, 70, 333, 0.25)]):
+        print(f"case {i} D={D} {dtype} mask={mask}", flush=True)
+        q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, dtype, 1000 + 10 * i)
+        fb = _bias((B, Hq, Sq, Sk), dtype, 1005 + i, holes=0.1)
+        qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
+        bd = fb.to(DEV)[..., :Sk]
+        seed, offset = 0x0BAD_CAFE_1234_0000 + i, 8 * (i + 3)
+        rng = torch.zeros(2, dtype=torch.int64, device=DEV)
+        out, lse = capi.fa_forward_dense(qd, kd, vd, is_causal=MASKS[mask], bias=bd, dropout_p=p, philox_seed=seed,
+                                         philox_offset=offset, rng_out=rng)
+        assert rng.tolist() == [seed, offset]
+        keep = _keep(seed, offset, B, Hq, Sq, Sk, p)
+        okw = dict(is_causal=mask != "none", causal_top_left=mask == "tl", attn_bias=fb[..., :Sk].double().numpy(),
+                   dropout_p=p, dropout_mask=keep)
+        ro, rl = oracle.sdpa_oracle(q, k, v, **okw)
+        got_o = out.float().cpu().double().numpy()
+        assert np.isfinite(got_o).all()
+        assert np.abs(got_o - ro).max() <= 2 * EPS[dtype] * max(1.0, float(np.abs(ro).max()))
+        fin = np.isfinite(rl)
+        assert np.abs(lse.cpu().numpy()[fin] - rl[fin]).max() <= 2e-3
+        got = capi.fa_backward_dense(dod, qd, kd, vd, out, lse, is_causal=MASKS[mask], bias=bd, want_dbias=True,
+                                     dropout_p=p, rng=rng)
+        want = oracle.sdpa_backward_oracle(q, k, v, do, return_dbias=True, **okw)
+        for name, g, w in zip(("dq", "dk", "dv", "dbias"), got, want):
+            _close(name, g, w, dtype)
+
+
+def test_efficient_ops_with_dropout_return_state_and_train():
+    """_scaled_dot_product_efficient_attention with dropout_p > 0: the Philox pair comes back as int64 device scalars,
+    the backward op regenerates the mask from them; same generator state, same result."""
+    B, H, Sq, Sk, D, p = 2, 4, 120, 168, 64, 0.3
+    q, k, v, do = _inputs(B, H, H, Sq, Sk, D, HF, 1100)
+    bias = _bias((B, 1, Sq, Sk), HF, 1101)[..., :Sk].contiguous()
+    qd, kd, vd, dod, bd = (t.to(DEV) for t in (q, k, v, do, bias))
+    be = bd.expand(B, H, Sq, Sk)
+    torch.manual_seed(77)
+    out, lse, seed, offset = aten._scaled_dot_product_efficient_attention(qd, kd, vd, be, True, p, False)
+    assert seed.is_cuda and seed.dtype == torch.int64 and seed.dim() == 0 and seed.item() == 77
+    keep = _keep(seed.item(), offset.item(), B, H, Sq, Sk, p)
+    okw = dict(attn_bias=bias.double().numpy(), dropout_p=p, dropout_mask=keep)
+    ro, _ = oracle.sdpa_oracle(q, k, v, **okw)
+    assert np.abs(out.float().cpu().double().numpy() - ro).max() <= 2 * EPS[HF] * max(1.0, float(np.abs(ro).max()))
+    gq, gk, gv, gb = aten._scaled_dot_product_efficient_attention_backward(
+        dod, qd, kd, vd, be, out, lse, seed, offset, p, [True, True, True, True], False)
+    want = oracle.sdpa_backward_oracle(q, k, v, do, return_dbias=True, **okw)
+    for name, g, w in zip(("dq", "dk", "dv", "dbias"), (gq, gk, gv, gb), want):
+        _close(name, g, w, HF)
+    torch.manual_seed(77)
+    out2 = aten._scaled_dot_product_efficient_attention(qd, kd, vd, be, True, p, False)[0]
+    out3 = aten._scaled_dot_product_efficient_attention(qd, kd, vd, be, True, p, False)[0]
+    assert torch.equal(out2, out) and not torch.equal(out3, out)
+
+
+def test_plain_sdpa_with_mask_and_dropout_trains_on_this_build():
+    """Padding mask + attention dropout, the encoder-training combination: one forward and one backward launch of this
+    build; the mean over many masks approaches the undropped result."""
+    B, H, S, D = 2, 4, 96, 64
+    q, k, v, _ = _inputs(B, H, H, S, S, D, BF, 1200)
+    qd, kd, vd = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    pad = torch.ones(B, 1, 1, S, dtype=torch.bool, device=DEV)
+    pad[0, ..., 70:] = False
+    assert torch._fused_sdp_choice(qd, kd, vd, pad, 0.1, False) == SDPBackend.EFFICIENT_ATTENTION
+    n0 = torch_mlu_amd.launch_count()
+    out = F.scaled_dot_product_attention(qd, kd, vd, attn_mask=pad, dropout_p=0.1)
+    out.float().sum().backward()
+    assert torch_mlu_amd.launch_count() == n0 + 2
+    assert all(torch.isfinite(t.grad).all().item() for t in (qd, kd, vd))
+    assert float(kd.grad[0, :, 70:].abs().max()) == 0.0 and float(vd.grad[0, :, 70:].abs().max()) == 0.0
+    with torch.no_grad():
+        acc = torch.zeros_like(out, dtype=torch.float32)
+        for _ in range(64):
+            acc += F.scaled_dot_product_attention(qd, kd, vd, attn_mask=pad, dropout_p=0.1).float()
+        ref = F.scaled_dot_product_attention(qd, kd, vd, attn_mask=pad).float()
+    assert (acc / 64 - ref).abs().mean().item() < 0.02

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import oracle
-from tests._util import LSE_TOL, lse_close, out_close, seeded
+from tests._util import LSE_TOL, algorithm_rounding_error, lse_close, out_close, seeded
 from torch_mlu_amd import capi
 
 pytestmark = pytest.mark.gpu
@@ -40,7 +40,7 @@ def _draw(rng):
     return dict(B=rng.choice([1, 2, 3]), Hq=Hq, Hk=Hk, Sq=Sq, Sk=Sk, D=D, dtype=rng.choice([BF, HF]),
                 mask=rng.choice([capi.FA_MASK_NONE, capi.FA_MASK_CAUSAL_BOTTOM_RIGHT, capi.FA_MASK_CAUSAL_TOP_LEFT]),
                 scale=rng.choice([None, None, 0.3, -0.11]), layout=rng.choice(["bhsd", "bshd", "wide"]),
-                extra=rng.choice(["none", "none", "bias", "dropout"]))
+                extra=rng.choice(["none", "none", "bias", "dropout", "bias+dropout"]))
 
 
 @pytest.mark.parametrize("chunk", range(6))
@@ -56,16 +56,16 @@ def test_dense_sweep(chunk):
         qd, kd, vd, dod = (_layout(t.to(DEV), c["layout"]) for t in (q, k, v, do))
         kw, okw = dict(is_causal=c["mask"], scale=c["scale"]), dict(
             is_causal=c["mask"] != 0, causal_top_left=c["mask"] == capi.FA_MASK_CAUSAL_TOP_LEFT, scale=c["scale"])
-        rng_t = None
-        if c["extra"] == "bias":
+        rng_t, bias_d = None, None
+        if "bias" in c["extra"]:
             bshape = rng.choice([(B, Hq, Sq, Sk), (B, 1, Sq, Sk), (1, Hq, 1, Sk), (1, 1, Sq, Sk)])
             full = seeded(bshape[:-1] + ((Sk + 7) // 8 * 8,), 77 + case, dtype, std=1.5)
             if rng.random() < 0.5:                        # a boolean-style mask: some -inf entries
                 drop = torch.rand(full.shape, generator=torch.Generator().manual_seed(case)) < 0.2
                 full = full.masked_fill(drop, float("-inf"))
-            kw["bias"] = full.to(DEV)[..., :Sk]
+            bias_d = kw["bias"] = full.to(DEV)[..., :Sk]
             okw["attn_bias"] = full[..., :Sk].double().numpy()
-        elif c["extra"] == "dropout":
+        if "dropout" in c["extra"]:
             p = rng.choice([0.1, 0.35, 0.8])
             seed, offset = rng.getrandbits(63), 4 * rng.getrandbits(40)
             rng_t = torch.zeros(2, dtype=torch.int64, device=DEV)
@@ -79,18 +79,20 @@ def test_dense_sweep(chunk):
         assert np.isfinite(got).all(), tag
         out_close(got, ro, dtype, tol=2 * EPS[dtype] * max(1.0, float(np.abs(ro).max())))
         lse_close(lse.cpu().numpy(), rl, tol=2e-3 if dtype == BF else LSE_TOL)
-        # backward: flash entry points only (no bias, bottom-right or no mask), head_dim <= 128
-        if D <= 128 and c["extra"] != "bias" and c["mask"] != capi.FA_MASK_CAUSAL_TOP_LEFT:
-            bkw = dict(is_causal=c["mask"] != 0, scale=c["scale"])
+        # backward (head_dim <= 128), with the gradient of the bias where there is one
+        if D <= 128:
+            bkw = dict(is_causal=c["mask"], scale=c["scale"], bias=bias_d, want_dbias=bias_d is not None)
             if rng_t is not None:
                 bkw.update(dropout_p=kw["dropout_p"], rng=rng_t)
             grads = capi.fa_backward_dense(dod, qd, kd, vd, out, lse, **bkw)
-            want = oracle.sdpa_backward_oracle(q, k, v, do, **{k_: v_ for k_, v_ in okw.items() if k_ != "causal_top_left"})
-            for name, g, w in zip(("dq", "dk", "dv"), grads, want):
+            want = oracle.sdpa_backward_oracle(q, k, v, do, return_dbias=bias_d is not None, **okw)
+            # bar: what the algorithm's own roundings cost on these inputs, plus 2 ulp at the gradient's magnitude
+            floor = algorithm_rounding_error(q, k, v, do, dtype, **okw)
+            for name, g, w, fl in zip(("dq", "dk", "dv", "dbias"), grads, want, floor):
                 g = g.float().cpu().double().numpy()
                 assert np.isfinite(g).all(), (tag, name)
                 err = float(np.abs(g - w).max()) if g.size else 0.0
-                assert err <= 2.0 * EPS[dtype] * max(float(np.abs(w).max()), 0.25), (tag, name, err)
+                assert err <= fl + 2.0 * EPS[dtype] * max(float(np.abs(w).max()), 0.25), (tag, name, err, fl)
 
 
 @pytest.mark.parametrize("chunk", range(3))

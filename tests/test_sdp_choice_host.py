@@ -88,7 +88,8 @@ def test_mem_efficient_constraints():
     q2, k2, v2 = _qkv((2, 4, 16, 64), size_k=(2, 4, 40, 64))
     assert "HIP device" in mem_reason(q2, k2, v2, None, 0.0, True)         # non-square causal is fine here (top-left)
     assert "boolean mask or have the dtype of query" in mem_reason(q, k, v, torch.zeros(16, 16))
-    assert "dropout" in mem_reason(q, k, v, None, 0.1)
+    assert "HIP device" in mem_reason(q, k, v, None, 0.1)                  # dropout is fine, with or without a mask
+    assert "HIP device" in mem_reason(q, k, v, mask, 0.1)
     assert "Mem efficient attention requires query.size(-1)==key.size(-1)==value.size(-1)" in mem_reason(*_qkv((2, 2, 3, 12)))
     assert "4 dimensional" in mem_reason(*_qkv((2, 3, 8)))
     assert "HIP device" in mem_reason(q.clone().requires_grad_(), k, v)   # a gradient is fine up to head_dim 128 ...

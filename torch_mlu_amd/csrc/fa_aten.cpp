@@ -127,6 +127,19 @@ void fill_strides(const at::Tensor& t, bool packed, int64_t& sb, int64_t& ss, in
 
 }  // namespace
 
+// One (seed, offset) pair of the default generator's Philox state for a call with dropout, taken under the generator's
+// mutex (FlashAttention_internal.cpp:198-210).  The increment only has to keep later consumers off this offset.
+static void take_philox_state(int64_t seqlen_q, int64_t seqlen_k, uint64_t& seed, uint64_t& offset) {
+  TORCH_CHECK(c10::hip::currentStreamCaptureStatusMayInitCtx() == c10::hip::CaptureStatus::None,
+              "attention forward: dropout under graph capture is not supported by this build");
+  auto* gen = at::get_generator_or_default<at::CUDAGeneratorImpl>(std::nullopt, at::cuda::detail::getDefaultCUDAGenerator());
+  std::lock_guard<std::mutex> lock(gen->mutex_);
+  const uint64_t increment = 4 * static_cast<uint64_t>((seqlen_q * seqlen_k + 1023) / 1024 + 1);
+  const at::PhiloxCudaState st = gen->philox_cuda_state(increment);
+  seed = st.seed_.val;
+  offset = st.offset_.val;
+}
+
 // ---- _flash_attention_forward ---------------------------------------------------------------------------------
 // cnnl__flash_attention_forward, attention.cpp:161-203.  cum_seq given: packed [T, H, D] inputs (the reference's
 // only mode); absent: dense [B, S, H, D] inputs (installed-PyTorch extension of the schema).
@@ -199,17 +212,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> flash_att
   at::Tensor offset_t = at::empty({}, q.options().dtype(at::kLong));
   at::Tensor debug_attn_mask = at::empty({0}, q.options());
   if (dropout_p > 0.0) {
-    TORCH_CHECK(c10::hip::currentStreamCaptureStatusMayInitCtx() == c10::hip::CaptureStatus::None,
-                "flash attention forward: dropout under graph capture is not supported by this build");
-    auto* gen = at::get_generator_or_default<at::CUDAGeneratorImpl>(std::nullopt, at::cuda::detail::getDefaultCUDAGenerator());
-    {
-      std::lock_guard<std::mutex> lock(gen->mutex_);
-      // one call consumes one (seed, offset) pair; the increment only has to keep later consumers off this offset
-      const uint64_t increment = 4 * static_cast<uint64_t>((seqlen_q * seqlen_k + 1023) / 1024 + 1);
-      const at::PhiloxCudaState st = gen->philox_cuda_state(increment);
-      p.philox_seed = st.seed_.val;
-      p.philox_offset = st.offset_.val;
-    }
+    take_philox_state(seqlen_q, seqlen_k, p.philox_seed, p.philox_offset);
     p.dropout_p = static_cast<float>(dropout_p);
     p.rng_seed_out = seed_t.data_ptr<int64_t>();
     p.rng_offset_out = offset_t.data_ptr<int64_t>();
@@ -479,7 +482,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
               "efficient attention forward: cu_seqlens are not supported by this build (use _flash_attention_forward)");
   TORCH_CHECK(!(seqlen_k.has_value() && seqlen_k->defined()), "efficient attention forward: seqlen_k is not supported");
   TORCH_CHECK(!window_size.has_value() || *window_size <= 0, "efficient attention forward: sliding window is not supported");
-  TORCH_CHECK(dropout_p == 0.0, "efficient attention forward: dropout_p > 0 is not supported by this build");
+  TORCH_CHECK(dropout_p >= 0.0 && dropout_p < 1.0, "efficient attention forward: dropout_p must be in [0, 1), got ", dropout_p);
   TORCH_CHECK(custom_mask_type >= 0 && custom_mask_type <= 2, "custom_mask_type must be 0, 1 or 2");
   // mem_eff_fwd's checks (FlashAttention_internal.cpp:500-527)
   const auto dt = query.scalar_type();
@@ -528,6 +531,15 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
     p.bias = bias_e.data_ptr();
     p.bias_stride_b = bias_e.stride(0); p.bias_stride_h = bias_e.stride(1); p.bias_stride_q = bias_e.stride(2);
   }
+  // the two Philox numbers of a call with dropout live on the device, stored there by the kernel (as in the flash op)
+  at::Tensor seed_t = at::empty({}, q.options().dtype(at::kLong));
+  at::Tensor offset_t = at::empty({}, q.options().dtype(at::kLong));
+  if (dropout_p > 0.0) {
+    take_philox_state(Sq, Sk, p.philox_seed, p.philox_offset);
+    p.dropout_p = static_cast<float>(dropout_p);
+    p.rng_seed_out = seed_t.data_ptr<int64_t>();
+    p.rng_offset_out = offset_t.data_ptr<int64_t>();
+  }
   if (B * Sq * Hq > 0) {
     const size_t ws_bytes = fa_fwd_workspace_bytes(&p);
     at::Tensor ws;
@@ -537,8 +549,6 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
     TORCH_CHECK(rc == FA_OK, "fa_fwd_launch failed: ", fa_fwd_error_string(rc), " (rc=", rc, ")");
     g_launches.fetch_add(1, std::memory_order_relaxed);
   }
-  at::Tensor seed_t = at::empty({}, q.options().dtype(at::kLong));
-  at::Tensor offset_t = at::empty({}, q.options().dtype(at::kLong));
   if (!compute_log_sumexp) lse = at::empty({B, Hq, 0}, q.options().dtype(at::kFloat));
   return std::make_tuple(output, lse, seed_t, offset_t, c10::SymInt(Sq), c10::SymInt(Sk));
 }
@@ -572,7 +582,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> efficient_attention_b
     const at::Tensor& logsumexp, double dropout_p, const at::Tensor& philox_seed, const at::Tensor& philox_offset,
     int64_t custom_mask_type, bool bias_requires_grad, std::optional<double> scale,
     std::optional<int64_t> num_splits_key, std::optional<int64_t> window_size, bool shared_storage_dqdkdv) {
-  (void)max_seqlen_q; (void)max_seqlen_k; (void)philox_seed; (void)philox_offset; (void)num_splits_key;
+  (void)max_seqlen_q; (void)max_seqlen_k; (void)num_splits_key;
   if (!grad_out_.defined()) return std::make_tuple(at::Tensor{}, at::Tensor{}, at::Tensor{}, at::Tensor{});  // :599-601
   // the reference's shape checks (attention.cpp:602-625)
   TORCH_CHECK(query.dim() == 4 && grad_out_.dim() == 4 && key.dim() == 4 && value.dim() == 4 && out.dim() == 4,
@@ -591,7 +601,13 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> efficient_attention_b
   TORCH_CHECK(!(cu_seqlens_q.has_value() && cu_seqlens_q->defined()) && !(cu_seqlens_k.has_value() && cu_seqlens_k->defined()),
               "efficient attention backward: cu_seqlens are not supported by this build (use _flash_attention_backward)");
   TORCH_CHECK(!window_size.has_value() || *window_size <= 0, "efficient attention backward: sliding window is not supported");
-  TORCH_CHECK(dropout_p == 0.0, "efficient attention backward: dropout_p > 0 is not supported by this build");
+  TORCH_CHECK(dropout_p >= 0.0 && dropout_p < 1.0, "efficient attention backward: dropout_p must be in [0, 1), got ", dropout_p);
+  if (dropout_p > 0.0)
+    TORCH_CHECK(philox_seed.defined() && philox_offset.defined() && philox_seed.is_cuda() && philox_offset.is_cuda() &&
+                    philox_seed.scalar_type() == at::kLong && philox_offset.scalar_type() == at::kLong &&
+                    philox_seed.numel() == 1 && philox_offset.numel() == 1,
+                "efficient attention backward: philox_seed and philox_offset must be the int64 device scalars the "
+                "forward returned");
   TORCH_CHECK(custom_mask_type >= 0 && custom_mask_type <= 2, "custom_mask_type must be 0, 1 or 2");
   // mem_eff_bwd's checks (FlashAttention_internal.cpp:714-758)
   const auto dt = query.scalar_type();
@@ -660,6 +676,11 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> efficient_attention_b
   p.dtype = dt == at::kBFloat16 ? FA_DTYPE_BF16 : FA_DTYPE_FP16;
   p.is_causal = custom_mask_type == 1 ? FA_MASK_CAUSAL_TOP_LEFT
                                       : (custom_mask_type == 2 ? FA_MASK_CAUSAL_BOTTOM_RIGHT : FA_MASK_NONE);
+  if (dropout_p > 0.0) {
+    p.dropout_p = static_cast<float>(dropout_p);
+    p.philox_seed = philox_seed.data_ptr<int64_t>();
+    p.philox_offset = philox_offset.data_ptr<int64_t>();
+  }
   if (has_bias && Sk > 0) {
     p.bias = bias_e.data_ptr();
     p.bias_stride_b = bias_e.stride(0); p.bias_stride_h = bias_e.stride(1); p.bias_stride_q = bias_e.stride(2);

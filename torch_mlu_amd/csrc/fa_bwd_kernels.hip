@@ -804,7 +804,7 @@ int bwd_validate(const fa_bwd_params* p) {
     if (((uintptr_t)p->bias & 7) || p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_q < 0 ||
         ((p->bias_stride_b | p->bias_stride_h | p->bias_stride_q) & 3))
       return FA_ERR_BAD_ARG;
-    if (p->cu_seqlens_q || p->dropout_p > 0.f) return FA_ERR_UNSUPPORTED;
+    if (p->cu_seqlens_q) return FA_ERR_UNSUPPORTED;
   }
   if (p->dbias) {  // an output: aligned like the bias and not broadcast
     if (((uintptr_t)p->dbias & 7) || ((p->dbias_stride_b | p->dbias_stride_h | p->dbias_stride_q) & 3)) return FA_ERR_BAD_ARG;
@@ -927,6 +927,11 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   a.offset_ptr = p->philox_offset;
   hipStream_t st = (hipStream_t)stream;
   const int dp = p->head_dim <= 64 ? 64 : 128;
+  if (p->dropout_p > 0.f && p->bias) {
+    if (p->dtype == FA_DTYPE_BF16)
+      return dp == 64 ? bwd_launch<__bf16, 64, true, true>(a, st) : bwd_launch<__bf16, 128, true, true>(a, st);
+    return dp == 64 ? bwd_launch<_Float16, 64, true, true>(a, st) : bwd_launch<_Float16, 128, true, true>(a, st);
+  }
   if (p->dropout_p > 0.f) {
     if (p->dtype == FA_DTYPE_BF16)
       return dp == 64 ? bwd_launch<__bf16, 64, true, false>(a, st) : bwd_launch<__bf16, 128, true, false>(a, st);

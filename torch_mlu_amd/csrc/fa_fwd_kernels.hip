@@ -820,7 +820,7 @@ int validate(const fa_fwd_params* p) {
   if (p->is_causal < FA_MASK_NONE || p->is_causal > FA_MASK_CAUSAL_TOP_LEFT) return FA_ERR_BAD_ARG;
   if (p->reserved2 != 0 || !(p->dropout_p >= 0.f && p->dropout_p < 1.f)) return FA_ERR_BAD_ARG;
   if (p->dropout_p > 0.f) {
-    if (p->bias || p->kernel == FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
+    if (p->kernel == FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
     if (p->dropout_mask && (p->cu_seqlens_q || ((uintptr_t)p->dropout_mask & 3))) return FA_ERR_UNSUPPORTED;
     if (((uintptr_t)p->rng_seed_out | (uintptr_t)p->rng_offset_out) & 7) return FA_ERR_BAD_ARG;
   }
@@ -953,6 +953,11 @@ int dispatch(const KArgs& a, int kern, hipStream_t st) {
     return launch_splitkv<T, 256>(a, st);
   }
   if (a.drop_thr < 255u) {  // dropout_p > 0
+    if (a.bias) {
+      if (dp == 64) return launch_tile<T, 64, 2, true, true>(a, st);
+      if (dp == 128) return launch_tile<T, 128, 2, true, true>(a, st);
+      return launch_tile<T, 256, 1, true, true>(a, st);
+    }
     if (dp == 64) return launch_tile<T, 64, 2, false, true>(a, st);
     if (dp == 128) return launch_tile<T, 128, 2, false, true>(a, st);
     return launch_tile<T, 256, 1, false, true>(a, st);

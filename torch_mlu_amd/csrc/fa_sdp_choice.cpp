@@ -195,13 +195,8 @@ bool check_head_dim_size_mem_efficient(const sdp_params& p, bool debug) {
   return true;
 }
 
-// Not in the reference (its mem-efficient path takes dropout, and its backward is the vendor's): what this build's
-// does not implement.
+// Not in the reference (its backward is the vendor's): what this build's does not implement.
 bool check_this_build_mem_efficient(const sdp_params& p, bool debug) {
-  if (p.dropout > 0.0) {
-    if (debug) TORCH_WARN("The mem-efficient kernels of this build do not implement dropout (dropout_p must be 0).");
-    return false;
-  }
   const bool mask_grad = p.attn_mask.has_value() && p.attn_mask->defined() && p.attn_mask->requires_grad();
   if ((input_requires_grad(p) || (at::GradMode::is_enabled() && mask_grad)) && p.query.size(-1) > 128) {
     if (debug)
