@@ -99,7 +99,8 @@ typedef struct fa_bwd_params {
 /* Host-only validation: FA_OK or a negative code (FA_ERR_UNSUPPORTED for head_dim > 128). */
 int fa_bwd_validate(const fa_bwd_params* p);
 
-/* Bytes of device scratch fa_bwd_launch needs (delta = rowsum(dO o O), fp32 per query row and head); 0 if invalid. */
+/* Bytes of device scratch fa_bwd_launch needs (-rowsum(dO o O) and LSE log2(e), two fp32 per query row and head);
+   0 if invalid. */
 size_t fa_bwd_workspace_bytes(const fa_bwd_params* p);
 
 /* Enqueue the backward pass on `stream`; `workspace` must hold fa_bwd_workspace_bytes(p) bytes, 16-byte aligned. */

@@ -153,10 +153,10 @@ def test_bwd_validate_accepts_good_params_and_sizes_delta_scratch():
     L = capi.lib()
     p = _good_bwd()
     assert L.fa_bwd_validate(ctypes.byref(p)) == capi.FA_OK
-    assert L.fa_bwd_workspace_bytes(ctypes.byref(p)) == 2 * 128 * 8 * 4      # fp32 per (batch, row, query head)
+    assert L.fa_bwd_workspace_bytes(ctypes.byref(p)) == 2 * (2 * 128 * 8 * 4)   # two fp32 per (batch, row, query head)
     packed = _good_bwd(cu_seqlens_q=0xa000, cu_seqlens_k=0xb000, total_q=200)
     assert L.fa_bwd_validate(ctypes.byref(packed)) == capi.FA_OK
-    assert L.fa_bwd_workspace_bytes(ctypes.byref(packed)) == 200 * 8 * 4
+    assert L.fa_bwd_workspace_bytes(ctypes.byref(packed)) == 2 * (200 * 8 * 4)
     # the mem-efficient backward's additions: mask aligned top-left, a (broadcast) bias, its gradient
     full = _good_bwd(is_causal=capi.FA_MASK_CAUSAL_TOP_LEFT, bias=0xc000, bias_stride_b=0, bias_stride_h=0,
                      bias_stride_q=256, dbias=0xd000, dbias_stride_b=8 * 128 * 256, dbias_stride_h=128 * 256,

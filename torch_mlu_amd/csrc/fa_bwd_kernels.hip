@@ -8,7 +8,8 @@
 //   fa_bwd_dq_kernel   — one workgroup = 128 query rows of one (sequence, head), loops over K/V tiles of 64 rows.
 //                        Per lane one query row (as in the forward): S^T = K Q^T, dP^T = V dO^T,
 //                        P^T = exp2(S^T c - LSE), dS^T = P^T o (dP^T - delta), dQ^T += K^T dS^T.
-//                        Also computes delta = rowsum(dO o O) for its rows and stores it for the second kernel.
+//                        Also computes delta = rowsum(dO o O) for its rows and stores -delta and LSE log2(e) for the
+//                        second kernel (which then starts its dP accumulators from -delta and needs no rescaling of LSE).
 //   fa_bwd_dkv_kernel  — one workgroup = 128 key rows of one (sequence, kv head), loops over the query heads of the
 //                        GQA group and over Q/dO tiles of 64 rows.  Per lane one key row: S = Q K^T, dP = dO V^T,
 //                        P, dS as above, dV^T += dO^T P, dK^T += Q^T dS.
@@ -37,7 +38,8 @@ struct BArgs {
   unsigned char* dq;
   unsigned char* dk;
   unsigned char* dv;
-  float* delta;  // dense [B][Hq][Sq], packed [Hq][total_q]
+  float* delta;  // workspace, dense [B][Hq][Sq], packed [Hq][total_q]: -rowsum(dO o O), written by the dQ kernel
+  float* lse2;   // workspace, same shape: LSE * log2(e)
   const int32_t* cu_q;
   const int32_t* cu_k;
   int64_t q_sb, q_ss, q_sh;  // byte strides
@@ -225,7 +227,10 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
   }
   const float lse2 =
       (row < Lq) ? a.lse[lb + (int64_t)h * a.lse_sh + (int64_t)(q0 + row) * a.lse_ss] * kLog2e : INFINITY;
-  if (row < Lq && g == 0) a.delta[dlb + (int64_t)h * a.dl_sh + (q0 + row)] = delta;
+  if (row < Lq && g == 0) {
+    a.delta[dlb + (int64_t)h * a.dl_sh + (q0 + row)] = -delta;
+    a.lse2[dlb + (int64_t)h * a.dl_sh + (q0 + row)] = lse2;
+  }
 
   f32x16 acc[MB];
 #pragma unroll
@@ -464,14 +469,14 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
   int q0 = 0, k0 = 0, Lq = a.seqlen_q, Lk = a.seqlen_k;
   int64_t qb = (int64_t)b * a.q_sb, kb = (int64_t)b * a.k_sb, vb = (int64_t)b * a.v_sb, dob = (int64_t)b * a.do_sb;
   int64_t dkb = (int64_t)b * a.dk_sb, dvb = (int64_t)b * a.dv_sb;
-  int64_t lb = (int64_t)b * a.lse_sb, dlb = (int64_t)b * a.dl_sb;
+  int64_t dlb = (int64_t)b * a.dl_sb;
   if (a.cu_q) {
     q0 = a.cu_q[b];
     Lq = a.cu_q[b + 1] - q0;
     k0 = a.cu_k[b];
     Lk = a.cu_k[b + 1] - k0;
     qb = kb = vb = dob = dkb = dvb = 0;
-    lb = dlb = 0;
+    dlb = 0;
   }
   if (pslot * BKV >= Lk) return;
   const int off = a.causal_tl ? 0 : Lk - Lq;
@@ -549,11 +554,9 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     for (int i = 0; i < NI; ++i)
       dma16s(dt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * do_ss + lc * 16,
              lds0 + 2 * TILE + buf * TILE + i * 4096);
-    if (wave < (DO_K ? 2 : 1)) {  // wavefront 0: LSE of the 64 rows, wavefront 1: delta (4 bytes per lane)
+    if (wave < (DO_K ? 2 : 1)) {  // wavefront 0: LSE log2(e) of the 64 rows, wavefront 1: -delta (4 bytes per lane)
       const int r = min(lane, rmax);
-      const float* src = (wave == 0)
-                             ? a.lse + lb + (int64_t)hq * a.lse_sh + (int64_t)(q0 + jq * BQ + r) * a.lse_ss
-                             : a.delta + dlb + (int64_t)hq * a.dl_sh + (q0 + jq * BQ + r);
+      const float* src = ((wave == 0) ? a.lse2 : a.delta) + dlb + (int64_t)hq * a.dl_sh + (q0 + jq * BQ + r);
       const unsigned dst = ldsv + (wave * 2 + buf) * 256;
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(dst), "v"(src) : "m0");
     }
@@ -632,17 +635,17 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
       // (with a bias the registers are needed elsewhere and the two vectors are read after the MFMAs; in halves
       // where the dK accumulators of head_dim 128 leave no room)
       constexpr bool HALVES = BIAS && DO_K && DP > 64;
+      // without dropout the dP accumulators start from -delta of their rows, so that the MFMAs deliver dP - delta
+      constexpr bool DELTA_INIT = DO_K && !DROP;
       f32x4 lv[4], dl[4];
-      if constexpr (!BIAS) {
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          lv[q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
-          if constexpr (DO_K) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
-        }
+      for (int q4 = 0; q4 < 4; ++q4) {
+        if constexpr (!BIAS) lv[q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
+        if constexpr (DO_K && (!BIAS || DELTA_INIT)) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
       }
       f32x16 s, dp, bacc;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; bacc[v] = 0.f; }
+      for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = DELTA_INIT ? dl[v >> 2][v & 3] : 0.f; bacc[v] = 0.f; }
       u32x4 braw[2];  // this block's bias, requested now, used after the S / dP MFMAs
       if constexpr (BIAS) load_bias(it, qbk, braw);
       {
@@ -681,7 +684,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
 #pragma unroll
           for (int q4 = 0; q4 < 4; ++q4) {
             lv[q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
-            if constexpr (DO_K) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
+            if constexpr (DO_K && !DELTA_INIT) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
           }
         }
       }
@@ -694,18 +697,20 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
 #pragma unroll
           for (int q4 = 2 * t; q4 < 2 * t + 2; ++q4) {
             lv[q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
-            if constexpr (DO_K) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
+            if constexpr (DO_K && !DELTA_INIT) dl[q4] = *(const f32x4*)(del_t + 32 * qbk + 8 * q4 + 4 * g);
           }
         }
 #pragma unroll
         for (int e2 = 0; e2 < 4; ++e2) {
           const int v = 8 * t + 2 * e2;  // v, v + 1: consecutive query rows
-          float l0 = lv[v >> 2][v & 3] * kLog2e, l1 = lv[v >> 2][(v & 3) + 1] * kLog2e;
+          float l0 = lv[v >> 2][v & 3], l1 = lv[v >> 2][(v & 3) + 1];
           if constexpr (BIAS) {
             l0 -= bacc[v] * kLog2e;
             l1 -= bacc[v + 1] * kLog2e;
           }
-          const float d0 = DO_K ? dl[v >> 2][v & 3] : 0.f, d1 = DO_K ? dl[v >> 2][(v & 3) + 1] : 0.f;
+          // minus delta of the two rows (already inside dp when the accumulators started from it)
+          const float d0 = (DO_K && !DELTA_INIT) ? dl[v >> 2][v & 3] : 0.f;
+          const float d1 = (DO_K && !DELTA_INIT) ? dl[v >> 2][(v & 3) + 1] : 0.f;
           float p0 = fast_exp2(s[v] * c - l0), p1 = fast_exp2(s[v + 1] * c - l1);
           if (need_mask) {
             const int qc = 32 * qbk + 8 * (v >> 2) + (v & 3);  // ql - 4 g
@@ -724,7 +729,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
             dp1 = k1 ? dp1 * a.drop_rp : 0.f;
           }
           if constexpr (DO_V) wp[e2] = Mma<T>::pack2(pv0, pv1);
-          if constexpr (DO_K) wd[e2] = Mma<T>::pack2(p0 * (dp0 - d0), p1 * (dp1 - d1));
+          if constexpr (DO_K) wd[e2] = Mma<T>::pack2(p0 * (dp0 + d0), p1 * (dp1 + d1));
         }
         pb[t] = __builtin_bit_cast(s16x8, wp);
         dsb[t] = __builtin_bit_cast(s16x8, wd);
@@ -837,10 +842,12 @@ int bwd_validate(const fa_bwd_params* p) {
   return FA_OK;
 }
 
-size_t bwd_ws_bytes(const fa_bwd_params* p) {
+// two fp32 planes per (row, head): -delta and LSE log2(e)
+size_t bwd_ws_plane(const fa_bwd_params* p) {
   const size_t rows = p->cu_seqlens_q ? (size_t)p->total_q : (size_t)p->batch * p->seqlen_q;
   return (rows * p->heads_q * 4 + 15) & ~(size_t)15;
 }
+size_t bwd_ws_bytes(const fa_bwd_params* p) { return 2 * bwd_ws_plane(p); }
 
 template <typename T, int DP, bool DROP, bool BIAS>
 int bwd_launch(const BArgs& a, hipStream_t st) {
@@ -891,6 +898,7 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   a.o = (const unsigned char*)p->out; a.dout = (const unsigned char*)p->dout; a.lse = p->lse;
   a.dq = (unsigned char*)p->dq; a.dk = (unsigned char*)p->dk; a.dv = (unsigned char*)p->dv;
   a.delta = (float*)workspace;
+  a.lse2 = (float*)((unsigned char*)workspace + bwd_ws_plane(p));
   a.cu_q = p->cu_seqlens_q; a.cu_k = p->cu_seqlens_k;
   a.q_sb = p->q_stride_b * 2; a.q_ss = p->q_stride_s * 2; a.q_sh = p->q_stride_h * 2;
   a.k_sb = p->k_stride_b * 2; a.k_ss = p->k_stride_s * 2; a.k_sh = p->k_stride_h * 2;
