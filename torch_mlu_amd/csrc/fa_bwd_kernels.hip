@@ -24,6 +24,13 @@
 #include "fa_bwd.h"
 #include "fa_device.h"
 
+// ring depths of the two operand prefetch loops of the dK/dV kernel, by what the instantiation computes
+#ifndef FA_RS
+#define FA_RS(DO_K, DO_V) ((DO_K) ? 2 : 4)
+#endif
+#ifndef FA_RT
+#define FA_RT(DO_K, DO_V) ((DO_K) && (DO_V) ? 2 : 4)
+#endif
 namespace {
 
 using namespace fa;
@@ -649,21 +656,22 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
       u32x4 braw[2];  // this block's bias, requested now, used after the S / dP MFMAs
       if constexpr (BIAS) load_bias(it, qbk, braw);
       {
-        // Q (and dO) row fragments are fetched two k-steps ahead of the MFMAs that consume them
-        s16x8 qa[2], da[2];
+        // Q (and dO) row fragments are fetched RS k-steps ahead of the MFMAs that consume them (a ring of RS slots)
+        constexpr int RS = FA_RS(DO_K, DO_V) < KS ? FA_RS(DO_K, DO_V) : KS;
+        s16x8 qa[RS], da[RS];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+        for (int ks = 0; ks < RS; ++ks) {
           qa[ks] = *(const s16x8*)(qt + kaddr[ks] + qbk * 32 * ROWB);
           if constexpr (DO_K) da[ks] = *(const s16x8*)(dt + kaddr[ks] + qbk * 32 * ROWB);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          s = Mma<T>::m32(qa[ks & 1], kf[ks], s);
-          if constexpr (DO_K) dp = Mma<T>::m32(da[ks & 1], vf[ks], dp);
-          if (ks + 2 < KS) {
-            qa[ks & 1] = *(const s16x8*)(qt + kaddr[ks + 2] + qbk * 32 * ROWB);
-            if constexpr (DO_K) da[ks & 1] = *(const s16x8*)(dt + kaddr[ks + 2] + qbk * 32 * ROWB);
+          s = Mma<T>::m32(qa[ks % RS], kf[ks], s);
+          if constexpr (DO_K) dp = Mma<T>::m32(da[ks % RS], vf[ks], dp);
+          if (ks + RS < KS) {
+            qa[ks % RS] = *(const s16x8*)(qt + kaddr[ks + RS] + qbk * 32 * ROWB);
+            if constexpr (DO_K) da[ks % RS] = *(const s16x8*)(dt + kaddr[ks + RS] + qbk * 32 * ROWB);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -736,25 +744,29 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
       }
       // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 32 query rows of this block)
       {
-        // transposed dO / Q fragments of step i + 1 are fetched while step i's MFMAs run (step = (t, mb))
+        // transposed dO / Q fragments are fetched RT - 1 steps ahead of their MFMAs (a ring of RT slots; step = (t, mb))
         auto tfrag = [&](const unsigned char* tile, int i) {
           const int ro = (32 * qbk + 16 * (i / MB)) * ROWB;
           const s16x4 lo = lds_read_tr(tile + taddr[0][i % MB] + ro);
           const s16x4 hi = lds_read_tr(tile + taddr[1][i % MB] + ro);
           return s16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         };
-        s16x8 dav[2], qav[2];
-        if constexpr (DO_V) dav[0] = tfrag(dt, 0);
-        if constexpr (DO_K) qav[0] = tfrag(qt, 0);
+        constexpr int RT = FA_RT(DO_K, DO_V) < 2 * MB ? FA_RT(DO_K, DO_V) : 2 * MB;
+        s16x8 dav[RT], qav[RT];
+#pragma unroll
+        for (int i = 0; i < RT - 1; ++i) {
+          if constexpr (DO_V) dav[i] = tfrag(dt, i);
+          if constexpr (DO_K) qav[i] = tfrag(qt, i);
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 2 * MB; ++i) {
-          if (i + 1 < 2 * MB) {
-            if constexpr (DO_V) dav[(i + 1) & 1] = tfrag(dt, i + 1);
-            if constexpr (DO_K) qav[(i + 1) & 1] = tfrag(qt, i + 1);
+          if (i + RT - 1 < 2 * MB) {
+            if constexpr (DO_V) dav[(i + RT - 1) % RT] = tfrag(dt, i + RT - 1);
+            if constexpr (DO_K) qav[(i + RT - 1) % RT] = tfrag(qt, i + RT - 1);
           }
-          if constexpr (DO_V) dv[i % MB] = Mma<T>::m32(dav[i & 1], pb[i / MB], dv[i % MB]);
-          if constexpr (DO_K) dk[i % MB] = Mma<T>::m32(qav[i & 1], dsb[i / MB], dk[i % MB]);
+          if constexpr (DO_V) dv[i % MB] = Mma<T>::m32(dav[i % RT], pb[i / MB], dv[i % MB]);
+          if constexpr (DO_K) dk[i % MB] = Mma<T>::m32(qav[i % RT], dsb[i / MB], dk[i % MB]);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
