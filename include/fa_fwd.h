@@ -116,6 +116,11 @@ typedef struct fa_fwd_params {
   void* dropout_mask;      /* device or NULL: debug output, dense [batch][heads_q][seqlen_q][seqlen_k] elements of
                               `dtype`, +1 kept / -1 dropped, positions outside a sequence or masked left untouched
                               (dense mode only) */
+  /* optional (NULL = all of them): device int32[batch]; only the first min(seqused_k[b], its length) keys of sequence b
+     exist — a KV cache that is allocated to seqlen_k rows but filled to a per-sequence length (the `seqused_k` of
+     aten::_flash_attention_forward, the `seqlen_k` of aten::_efficient_attention_forward).  The causal mask aligns to
+     the used length.  Forward only: the backward has no such argument. */
+  const int32_t* seqused_k;
 } fa_fwd_params;
 
 #define FA_MAX_SPLITS 64

@@ -99,8 +99,6 @@ def test_unsupported_features_are_refused_loudly():
         f(q, k, v, None, None, 8, 8, 0.0, False, False, window_size_left=4)
     with pytest.raises(RuntimeError, match="alibi_slopes is not supported"):
         f(q, k, v, None, None, 8, 8, 0.0, False, False, alibi_slopes=torch.zeros(4))
-    with pytest.raises(RuntimeError, match="seqused_k is not supported"):
-        f(q, k, v, None, None, 8, 8, 0.0, False, False, seqused_k=torch.zeros(2, dtype=torch.int32))
 
 
 def test_sdp_kernel_context_restores_flags():

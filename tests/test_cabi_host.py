@@ -204,6 +204,14 @@ def test_bwd_null_and_short_workspace():
 
 
 # ---- additive bias and mask alignment ------------------------------------------------------------------------------
+def test_seqused_k_pointer_is_validated():
+    L = capi.lib()
+    p = _good(seqused_k=0xf000)
+    assert L.fa_fwd_validate(ctypes.byref(p)) == capi.FA_OK
+    p = _good(seqused_k=0xf002)                      # int32 entries: 4-byte aligned
+    assert L.fa_fwd_validate(ctypes.byref(p)) == capi.FA_ERR_BAD_ARG
+
+
 def test_bias_and_mask_mode_validation_and_plan():
     L = capi.lib()
     good = _good(bias=0x7000, bias_stride_b=0, bias_stride_h=128 * 256, bias_stride_q=256, is_causal=0)

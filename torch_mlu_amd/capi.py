@@ -84,6 +84,7 @@ class FaFwdParams(ctypes.Structure):
         ("rng_seed_out", ctypes.c_void_p),
         ("rng_offset_out", ctypes.c_void_p),
         ("dropout_mask", ctypes.c_void_p),
+        ("seqused_k", ctypes.c_void_p),
     ]
 
 
@@ -164,7 +165,7 @@ def make_params(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Te
                 is_causal=False, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
                 bias: Optional[torch.Tensor] = None, dropout_p: float = 0.0, philox_seed: int = 0,
                 philox_offset: int = 0, rng_out: Optional[torch.Tensor] = None,
-                dropout_mask: Optional[torch.Tensor] = None) -> FaFwdParams:
+                dropout_mask: Optional[torch.Tensor] = None, seqused_k: Optional[torch.Tensor] = None) -> FaFwdParams:
     """Fill a params struct.  `is_causal`: False / True (bottom-right aligned) or one of the FA_MASK_* codes; `bias`:
     a [B, Hq, Sq, Sk] view (dense mode; stride 0 where broadcast) of the inputs' dtype.
 
@@ -215,6 +216,7 @@ def make_params(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Te
     p.rng_seed_out = rng_out[0:].data_ptr() if rng_out is not None else None
     p.rng_offset_out = rng_out[1:].data_ptr() if rng_out is not None else None
     p.dropout_mask = dropout_mask.data_ptr() if dropout_mask is not None else None
+    p.seqused_k = seqused_k.data_ptr() if seqused_k is not None else None
     return p
 
 
@@ -233,12 +235,14 @@ def fa_forward_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, is_ca
                      scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
                      bias: Optional[torch.Tensor] = None, dropout_p: float = 0.0, philox_seed: int = 0,
                      philox_offset: int = 0, rng_out: Optional[torch.Tensor] = None,
-                     dropout_mask: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                     dropout_mask: Optional[torch.Tensor] = None, seqused_k: Optional[torch.Tensor] = None
+                     ) -> Tuple[torch.Tensor, torch.Tensor]:
     """q [B, Hq, Sq, D], k/v [B, Hk, Sk, D] (any strides, contiguous last dim) -> out [B, Hq, Sq, D] (stored
     [B, Sq, Hq, D] like the reference's dense wrapper, attention.cpp:146-148), lse [B, Hq, Sq] fp32.
     `bias`: anything that expands to [B, Hq, Sq, Sk]; `is_causal` may also be FA_MASK_CAUSAL_TOP_LEFT.
     Dropout: `dropout_p`, the two numbers that define the mask, `rng_out` (int64[2] on the device, receives them) and
-    `dropout_mask` (zero-initialised [B, Hq, Sq, Sk] of q's dtype, receives +1 kept / -1 dropped)."""
+    `dropout_mask` (zero-initialised [B, Hq, Sq, Sk] of q's dtype, receives +1 kept / -1 dropped).
+    `seqused_k`: int32 [B] on the device, how many of the Sk key rows of each sequence exist."""
     B, Hq, Sq, D = q.shape
     if bias is not None:
         bias = bias.expand(B, Hq, Sq, k.shape[2])
@@ -246,7 +250,8 @@ def fa_forward_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, is_ca
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
     p = make_params(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), out, lse, scale=scale,
                     is_causal=is_causal, kernel=kernel, num_splits=num_splits, bias=bias, dropout_p=dropout_p,
-                    philox_seed=philox_seed, philox_offset=philox_offset, rng_out=rng_out, dropout_mask=dropout_mask)
+                    philox_seed=philox_seed, philox_offset=philox_offset, rng_out=rng_out, dropout_mask=dropout_mask,
+                    seqused_k=seqused_k)
     launch(p, q.device)
     return out.transpose(1, 2), lse
 
@@ -255,7 +260,8 @@ def fa_forward_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seql
                       cu_seqlens_k: torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, *, is_causal: bool = False,
                       scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
                       dropout_p: float = 0.0, philox_seed: int = 0, philox_offset: int = 0,
-                      rng_out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                      rng_out: Optional[torch.Tensor] = None, seqused_k: Optional[torch.Tensor] = None
+                      ) -> Tuple[torch.Tensor, torch.Tensor]:
     """q [Tq, Hq, D], k/v [Tk, Hk, D], cu_seqlens int32 [B+1] on the device -> out [Tq, Hq, D], lse [Hq, Tq]."""
     Tq, Hq, D = q.shape
     out = torch.empty((Tq, Hq, D), dtype=q.dtype, device=q.device)
@@ -263,7 +269,7 @@ def fa_forward_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seql
     p = make_params(q, k, v, out, lse, cu_seqlens_q=cu_seqlens_q, cu_seqlens_k=cu_seqlens_k,
                     max_seqlen_q=max_seqlen_q, max_seqlen_k=max_seqlen_k, scale=scale, is_causal=is_causal,
                     kernel=kernel, num_splits=num_splits, dropout_p=dropout_p, philox_seed=philox_seed,
-                    philox_offset=philox_offset, rng_out=rng_out)
+                    philox_offset=philox_offset, rng_out=rng_out, seqused_k=seqused_k)
     launch(p, q.device)
     return out, lse
 

@@ -9,8 +9,9 @@
 //   registration                              codegen/templates/RegisterMLU.cpp:185-187 (TORCH_LIBRARY_IMPL)
 //
 // Differences from the reference, all forced by the installed PyTorch or by the no-copy design:
-//   * the schemas are the installed PyTorch's (optional cum_seq, window/alibi/seqused arguments that must be
-//     unset); the tuple positions and meanings are the reference's (codegen/mlu_functions.yaml:1313,1315);
+//   * the schemas are the installed PyTorch's (optional cum_seq; window and alibi arguments that must be unset;
+//     seqused_k = per-sequence fill level of a KV cache, honoured); the tuple positions and meanings are the
+//     reference's (codegen/mlu_functions.yaml:1313,1315);
 //   * Q/K/V are never copied: their strides go to the launcher (the reference makes up to three transposing
 //     copies at attention.cpp:124-129);
 //   * Hq may be a multiple of Hkv at the dense op too (the inner launcher already allowed it,
@@ -129,6 +130,18 @@ void fill_strides(const at::Tensor& t, bool packed, int64_t& sb, int64_t& ss, in
 
 // One (seed, offset) pair of the default generator's Philox state for a call with dropout, taken under the generator's
 // mutex (FlashAttention_internal.cpp:198-210).  The increment only has to keep later consumers off this offset.
+// `seqused_k` / `seqlen_k`: int32 [batch] on the device.  The backward ops have no such argument, so a call that will
+// be differentiated is refused here rather than differentiated wrongly later.
+static at::Tensor checked_seqused_k(const at::Tensor& t, int64_t batch, const at::Tensor& q, const at::Tensor& k,
+                                    const at::Tensor& v, const char* name) {
+  TORCH_CHECK(t.scalar_type() == at::kInt, name, " must have dtype int32");
+  TORCH_CHECK(t.is_cuda(), name, " must be on HIP device");
+  TORCH_CHECK(t.dim() == 1 && t.size(0) == batch, name, " must have shape (batch_size)");
+  TORCH_CHECK(!(at::GradMode::is_enabled() && (q.requires_grad() || k.requires_grad() || v.requires_grad())), name,
+              " is for inference: the backward ops cannot take it");
+  return t.contiguous();
+}
+
 static void take_philox_state(int64_t seqlen_q, int64_t seqlen_k, uint64_t& seed, uint64_t& offset) {
   TORCH_CHECK(c10::hip::currentStreamCaptureStatusMayInitCtx() == c10::hip::CaptureStatus::None,
               "attention forward: dropout under graph capture is not supported by this build");
@@ -156,7 +169,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> flash_att
   TORCH_CHECK(!window_size_left.has_value() || *window_size_left < 0, "flash attention forward: sliding window is not supported");
   TORCH_CHECK(!window_size_right.has_value() || *window_size_right < 0 || (is_causal && *window_size_right == 0),
               "flash attention forward: sliding window is not supported");
-  TORCH_CHECK(!(seqused_k.has_value() && seqused_k->defined()), "flash attention forward: seqused_k is not supported");
+  const bool has_used = seqused_k.has_value() && seqused_k->defined();
   TORCH_CHECK(!(alibi_slopes.has_value() && alibi_slopes->defined()), "flash attention forward: alibi_slopes is not supported");
 
   Packed pk{packed ? &*cum_seq_q : nullptr, packed ? &*cum_seq_k : nullptr, max_q, max_k};
@@ -204,6 +217,11 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> flash_att
   p.is_causal = is_causal ? 1 : 0;
   p.kernel = FA_KERNEL_AUTO;
   p.num_splits = 0;
+  at::Tensor used;  // per-sequence count of the key rows that exist (a KV cache filled to different lengths)
+  if (has_used) {
+    used = checked_seqused_k(*seqused_k, batch, query, key, value, "seqused_k");
+    p.seqused_k = used.data_ptr<int32_t>();
+  }
 
   // p == 0: the reference returns two uninitialised 0-d int64 tensors (FlashAttention_internal.cpp:211-213); p > 0:
   // the generator's Philox state, advanced under its mutex (:198-210) — here the kernel stores the two numbers into
@@ -480,7 +498,6 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   TORCH_CHECK(value.size(3) == query.size(3), "this build needs value.size(-1) == query.size(-1)");
   TORCH_CHECK(!(cu_seqlens_q.has_value() && cu_seqlens_q->defined()) && !(cu_seqlens_k.has_value() && cu_seqlens_k->defined()),
               "efficient attention forward: cu_seqlens are not supported by this build (use _flash_attention_forward)");
-  TORCH_CHECK(!(seqlen_k.has_value() && seqlen_k->defined()), "efficient attention forward: seqlen_k is not supported");
   TORCH_CHECK(!window_size.has_value() || *window_size <= 0, "efficient attention forward: sliding window is not supported");
   TORCH_CHECK(dropout_p >= 0.0 && dropout_p < 1.0, "efficient attention forward: dropout_p must be in [0, 1), got ", dropout_p);
   TORCH_CHECK(custom_mask_type >= 0 && custom_mask_type <= 2, "custom_mask_type must be 0, 1 or 2");
@@ -527,6 +544,11 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   p.is_causal = custom_mask_type == 1 ? FA_MASK_CAUSAL_TOP_LEFT
                                       : (custom_mask_type == 2 ? FA_MASK_CAUSAL_BOTTOM_RIGHT : FA_MASK_NONE);
   p.kernel = FA_KERNEL_AUTO;
+  at::Tensor used;
+  if (seqlen_k.has_value() && seqlen_k->defined()) {
+    used = checked_seqused_k(*seqlen_k, B, query, key, value, "seqlen_k");
+    p.seqused_k = used.data_ptr<int32_t>();
+  }
   if (bias_e.defined() && Sk > 0) {
     p.bias = bias_e.data_ptr();
     p.bias_stride_b = bias_e.stride(0); p.bias_stride_h = bias_e.stride(1); p.bias_stride_q = bias_e.stride(2);

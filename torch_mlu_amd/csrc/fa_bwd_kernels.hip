@@ -25,6 +25,13 @@
 #include "fa_device.h"
 
 // ring depths of the two operand prefetch loops of the dK/dV kernel, by what the instantiation computes
+// ring depths of the two operand prefetch loops of the dQ kernel
+#ifndef FA_RQ
+#define FA_RQ 2
+#endif
+#ifndef FA_RA
+#define FA_RA 2
+#endif
 #ifndef FA_RS
 #define FA_RS(DO_K, DO_V) ((DO_K) ? 2 : 4)
 #endif
@@ -315,26 +322,26 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; p0[v] = 0.f; p1[v] = 0.f; }
     {
-      // K and V fragments are fetched one k-step ahead of the MFMAs that consume them
-      s16x8 fr[2][4];
-      fr[0][0] = *(const s16x8*)(kt + kaddr[0]);
-      fr[0][1] = *(const s16x8*)(kt + kaddr[0] + 32 * ROWB);
-      fr[0][2] = *(const s16x8*)(vt + kaddr[0]);
-      fr[0][3] = *(const s16x8*)(vt + kaddr[0] + 32 * ROWB);
+      // K and V fragments are fetched RQ - 1 k-steps ahead of the MFMAs that consume them (a ring of RQ slots)
+      constexpr int RQ = FA_RQ;
+      s16x8 fr[RQ][4];
+      auto load_fr = [&](int ks) {
+        fr[ks % RQ][0] = *(const s16x8*)(kt + kaddr[ks]);
+        fr[ks % RQ][1] = *(const s16x8*)(kt + kaddr[ks] + 32 * ROWB);
+        fr[ks % RQ][2] = *(const s16x8*)(vt + kaddr[ks]);
+        fr[ks % RQ][3] = *(const s16x8*)(vt + kaddr[ks] + 32 * ROWB);
+      };
+#pragma unroll
+      for (int ks = 0; ks < RQ - 1; ++ks) load_fr(ks);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        if (ks + 1 < KS) {
-          fr[(ks + 1) & 1][0] = *(const s16x8*)(kt + kaddr[ks + 1]);
-          fr[(ks + 1) & 1][1] = *(const s16x8*)(kt + kaddr[ks + 1] + 32 * ROWB);
-          fr[(ks + 1) & 1][2] = *(const s16x8*)(vt + kaddr[ks + 1]);
-          fr[(ks + 1) & 1][3] = *(const s16x8*)(vt + kaddr[ks + 1] + 32 * ROWB);
-        }
-        s0 = Mma<T>::m32(fr[ks & 1][0], qf[ks], s0);
-        s1 = Mma<T>::m32(fr[ks & 1][1], qf[ks], s1);
-        p0 = Mma<T>::m32(fr[ks & 1][2], dof[ks], p0);
-        p1 = Mma<T>::m32(fr[ks & 1][3], dof[ks], p1);
-        __builtin_amdgcn_sched_barrier(0);  // keep the loads of step ks + 1 ahead of these MFMAs
+        if (ks + RQ - 1 < KS) load_fr(ks + RQ - 1);
+        s0 = Mma<T>::m32(fr[ks % RQ][0], qf[ks], s0);
+        s1 = Mma<T>::m32(fr[ks % RQ][1], qf[ks], s1);
+        p0 = Mma<T>::m32(fr[ks % RQ][2], dof[ks], p0);
+        p1 = Mma<T>::m32(fr[ks % RQ][3], dof[ks], p1);
+        __builtin_amdgcn_sched_barrier(0);  // keep the loads of the later steps ahead of these MFMAs
       }
     }
     // P^T = exp2(S^T c - LSE), dS^T = P^T (dP^T - delta); masked positions contribute nothing
@@ -380,18 +387,21 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
         const s16x4 hi = lds_read_tr(kt + taddr[1][mb] + (16 * t) * ROWB);
         return s16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       };
-      s16x8 ka[2][MB];
+      constexpr int RA = FA_RA;
+      s16x8 ka[RA][MB];
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) ka[0][mb] = kfrag(mb, 0);
+      for (int t = 0; t < RA - 1; ++t)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) ka[t][mb] = kfrag(mb, t);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        if (t + 1 < 4) {
+        if (t + RA - 1 < 4) {
 #pragma unroll
-          for (int mb = 0; mb < MB; ++mb) ka[(t + 1) & 1][mb] = kfrag(mb, t + 1);
+          for (int mb = 0; mb < MB; ++mb) ka[(t + RA - 1) % RA][mb] = kfrag(mb, t + RA - 1);
         }
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) acc[mb] = Mma<T>::m32(ka[t & 1][mb], dsb[t], acc[mb]);
+        for (int mb = 0; mb < MB; ++mb) acc[mb] = Mma<T>::m32(ka[t % RA][mb], dsb[t], acc[mb]);
         __builtin_amdgcn_sched_barrier(0);
       }
     }

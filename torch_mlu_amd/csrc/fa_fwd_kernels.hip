@@ -55,6 +55,7 @@ struct KArgs {
   float scale_log2;   // |scale| * log2(e)
   float scale_abs;    // |scale| (bias path)
   int32_t causal_tl;  // causal mask aligned to the top-left corner (col <= row) instead of the bottom-right one
+  const int32_t* seqused_k;   // optional: keys of sequence b beyond seqused_k[b] do not exist
   const unsigned char* bias;  // optional additive bias, dense mode: [b][h][row][col] through byte strides
   int64_t bias_sb, bias_sh, bias_sq;
   uint32_t drop_thr;  // dropout: an element is kept iff its byte <= drop_thr
@@ -154,6 +155,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     qb = kb = vb = ob = 0;
     lb = 0;
   }
+  if (a.seqused_k) Lk = min(Lk, max(a.seqused_k[b], 0));
   // query blocks owned by this workgroup: paired (causal, dense) -> the heavy block nblk-1-p and the light block p,
   // so that every workgroup of a sequence has the same number of tiles; unpaired -> one block, heavy blocks first
   // (packed: counted down from the longest possible sequence so that equal slots mean equal block indices)
@@ -535,6 +537,7 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
     qb = kb = vb = ob = 0;
     lb = (int64_t)q0 * a.lse_ss;
   }
+  if (a.seqused_k) Lk = min(Lk, max(a.seqused_k[b], 0));
   const int D = a.head_dim;
   const int group = a.group;
   const int h0 = hk * group;
@@ -824,6 +827,7 @@ int validate(const fa_fwd_params* p) {
     if (p->dropout_mask && (p->cu_seqlens_q || ((uintptr_t)p->dropout_mask & 3))) return FA_ERR_UNSUPPORTED;
     if (((uintptr_t)p->rng_seed_out | (uintptr_t)p->rng_offset_out) & 7) return FA_ERR_BAD_ARG;
   }
+  if ((uintptr_t)p->seqused_k & 3) return FA_ERR_BAD_ARG;
   if (p->bias) {
     if (((uintptr_t)p->bias & 7) || p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_q < 0 ||
         ((p->bias_stride_b | p->bias_stride_h | p->bias_stride_q) & 3))
@@ -889,6 +893,7 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   a.n_splits = ns;
   a.is_causal = p->is_causal ? 1 : 0;
   a.causal_tl = p->is_causal == FA_MASK_CAUSAL_TOP_LEFT ? 1 : 0;
+  a.seqused_k = p->seqused_k;
   a.bias = (const unsigned char*)p->bias;
   a.bias_sb = p->bias_stride_b * 2; a.bias_sh = p->bias_stride_h * 2; a.bias_sq = p->bias_stride_q * 2;
   a.neg_scale = p->scale < 0.f ? 1 : 0;
