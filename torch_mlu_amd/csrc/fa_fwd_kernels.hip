@@ -97,7 +97,9 @@ constexpr float kLazyLog2 = 8.0f;
 // groups of 4 consecutive keys = 8 bytes) and the softmax then runs on scores already in the log2 domain.
 // DROP: dropout on the probabilities.  The row sums (and LSE) are those of the undropped probabilities; dropped
 // entries are zeroed in the P operand of the PV product and 1 / (1 - p) is folded into the final normalisation.
-template <typename T, int DP, int MINB, bool BIAS, bool DROP = false>
+// DMASK (with DROP): also write the keep-mask out for tests; a variant of its own because the extra stores cost
+// registers (30 spilled at head_dim 128) that the plain dropout kernel does not have to pay.
+template <typename T, int DP, int MINB, bool BIAS, bool DROP = false, bool DMASK = false>
 __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   constexpr int CPR = DP / 8;          // 16-byte chunks per row
   constexpr int ROWB = DP * 2;         // bytes per LDS row
@@ -275,7 +277,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   const int drop_sh = 16 * (row & 1);
   const unsigned char* brow = nullptr;  // this lane's bias row, at its first key group (4 g)
   unsigned char* drow = nullptr;  // this lane's row of the debug mask
-  if constexpr (DROP)
+  if constexpr (DROP && DMASK)
     if (a.dmask) drow = a.dmask + (((int64_t)b * a.heads_q + h) * a.seqlen_q + min(row, Lq - 1)) * (int64_t)a.seqlen_k * 2;
   if constexpr (BIAS)
     brow = a.bias + (int64_t)b * a.bias_sb + (int64_t)h * a.bias_sh + (int64_t)min(row, Lq - 1) * a.bias_sq + 8 * g;
@@ -428,7 +430,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
           const uint32_t cp_const = 16 * (t >> 1) + 4 * (v >> 2) + ((v & 3) >> 1);
           const uint32_t word = drop_mix(drop_tile ^ cp_const) >> drop_sh;
           const bool k0 = (word & 0xffu) <= a.drop_thr, k1 = ((word >> 8) & 0xffu) <= a.drop_thr;
-          if (a.dmask) {
+          if (DMASK && a.dmask) {
             const int col = j * BN + 32 * (t >> 1) + 8 * (v >> 2) + 4 * g + (v & 3);
             if (row < Lq && col + 1 <= min(last_k, causal_row_lim)) {
               *(unsigned*)(drow + (int64_t)col * 2) = Mma<T>::pack2(k0 ? 1.f : -1.f, k1 ? 1.f : -1.f);
@@ -918,10 +920,10 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   return a;
 }
 
-template <typename T, int DP, int MINB, bool BIAS, bool DROP = false>
+template <typename T, int DP, int MINB, bool BIAS, bool DROP = false, bool DMASK = false>
 int launch_tile(KArgs a, hipStream_t st) {
   constexpr int lds = 4 * 64 * DP * 2;
-  constexpr auto kfn = fa_tile_kernel<T, DP, MINB, BIAS, DROP>;
+  constexpr auto kfn = fa_tile_kernel<T, DP, MINB, BIAS, DROP, DMASK>;
   if (!ensure_dynamic_lds<kfn>(lds)) return FA_ERR_LAUNCH;
   const int nblk = (a.seqlen_q + 127) / 128;
   a.pair = (DP != 256 && !a.cu_q && a.is_causal && nblk >= 2 && (int64_t)a.batch * a.heads_q * ((nblk + 1) / 2) >= 1024) ? 1 : 0;
@@ -956,6 +958,16 @@ int dispatch(const KArgs& a, int kern, hipStream_t st) {
     if (dp == 64) return launch_splitkv<T, 64>(a, st);
     if (dp == 128) return launch_splitkv<T, 128>(a, st);
     return launch_splitkv<T, 256>(a, st);
+  }
+  if (a.drop_thr < 255u && a.dmask) {  // dropout_p > 0 and the keep-mask is wanted (tests)
+    if (a.bias) {
+      if (dp == 64) return launch_tile<T, 64, 2, true, true, true>(a, st);
+      if (dp == 128) return launch_tile<T, 128, 2, true, true, true>(a, st);
+      return launch_tile<T, 256, 1, true, true, true>(a, st);
+    }
+    if (dp == 64) return launch_tile<T, 64, 2, false, true, true>(a, st);
+    if (dp == 128) return launch_tile<T, 128, 2, false, true, true>(a, st);
+    return launch_tile<T, 256, 1, false, true, true>(a, st);
   }
   if (a.drop_thr < 255u) {  // dropout_p > 0
     if (a.bias) {
