@@ -30,12 +30,12 @@ PEAK_HBM_GBS = 8000.0
 # their commands are recorded under profiles/.  Counters cannot be read from inside a timed run, so these are the
 # recorded values (None: not profiled).
 TRAFFIC_BYTES = {
-    "cfg2": int((512.7 + 130.0) * 2 ** 20),
+    "cfg2": int((515.9 + 130.0) * 2 ** 20),
     "cfg5": int(2.0021 * 2 ** 30 + 4.25 * 2 ** 20),
-    "cfg2_bwd": int((1746.7 + 386.1) * 2 ** 20),  # the three launches of one backward together
-    "cfg2_mask": int(3.05 * 2 ** 30 + 227.9 * 2 ** 20),
-    "cfg2_drop": int((629.9 + 195.0) * 2 ** 20),
-    "cfg2_mask_bwd": int((3.32 + 4.41 + 2.40) * 2 ** 30 + (150.7 + 136.0 + 130.7) * 2 ** 20),  # three launches
+    "cfg2_bwd": int((1746.1 + 388.1) * 2 ** 20),  # the three launches of one backward together
+    "cfg2_mask": int(3.68 * 2 ** 30 + 223.6 * 2 ** 20),
+    "cfg2_drop": int((512.8 + 130.0) * 2 ** 20),
+    "cfg2_mask_bwd": int((3.44 + 4.43 + 2.40) * 2 ** 30 + (151.1 + 133.5 + 130.7) * 2 ** 20),  # three launches
 }
 
 
