@@ -178,10 +178,21 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
   if (lc * 8 >= D) lc = 0;
   const unsigned k_ss = (unsigned)a.k_ss, v_ss = (unsigned)a.v_ss;
   const unsigned lds0 = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + wave * 1024;
+  // per-lane byte offsets of a full tile's first DMA block; the later blocks only move the scalar base
+  const unsigned koff0 = (unsigned)dma_r * k_ss + lc * 16, voff0 = (unsigned)dma_r * v_ss + lc * 16;
   auto issue_tile = [&](int j, int buf) {
     const int rmax = last_k - j * BN;
     const unsigned char* kt = kp + (uint64_t)(unsigned)(j * BN) * k_ss;
     const unsigned char* vt = vp + (uint64_t)(unsigned)(j * BN) * v_ss;
+    if (rmax >= BN - 1) {  // the whole tile lies inside the sequence: scalar address arithmetic only
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        dma16s(kt + (uint64_t)(unsigned)(i * 4 * RPI) * k_ss, koff0, lds0 + buf * TILE + i * 4096);
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        dma16s(vt + (uint64_t)(unsigned)(i * 4 * RPI) * v_ss, voff0, lds0 + 2 * TILE + buf * TILE + i * 4096);
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NI; ++i)
       dma16s(kt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * k_ss + lc * 16, lds0 + buf * TILE + i * 4096);
@@ -557,6 +568,8 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     }
   }
 
+  // per-lane byte offsets of a full tile's first DMA block; the later blocks only move the scalar base
+  const unsigned qoff0 = (unsigned)dma_r * q_ss + lc * 16, dooff0 = (unsigned)dma_r * do_ss + lc * 16;
   // ---- DMA of a (query head, query tile): Q rows, dO rows, LSE and delta of the 64 rows ----
   auto issue_iter = [&](int it, int buf) {
     const int hq = hk * a.group + it / nq;
@@ -564,13 +577,22 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     const int rmax = Lq - 1 - jq * BQ;
     const unsigned char* qt = a.q + qb + (int64_t)(q0 + jq * BQ) * a.q_ss + (int64_t)hq * a.q_sh;
     const unsigned char* dt = a.dout + dob + (int64_t)(q0 + jq * BQ) * a.do_ss + (int64_t)hq * a.do_sh;
+    if (rmax >= BQ - 1) {  // the whole tile lies inside the sequence: scalar address arithmetic only
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
-      dma16s(qt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * q_ss + lc * 16, lds0 + buf * TILE + i * 4096);
+      for (int i = 0; i < NI; ++i)
+        dma16s(qt + (uint64_t)(unsigned)(i * 4 * RPI) * q_ss, qoff0, lds0 + buf * TILE + i * 4096);
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
-      dma16s(dt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * do_ss + lc * 16,
-             lds0 + 2 * TILE + buf * TILE + i * 4096);
+      for (int i = 0; i < NI; ++i)
+        dma16s(dt + (uint64_t)(unsigned)(i * 4 * RPI) * do_ss, dooff0, lds0 + 2 * TILE + buf * TILE + i * 4096);
+    } else {
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        dma16s(qt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * q_ss + lc * 16, lds0 + buf * TILE + i * 4096);
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        dma16s(dt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * do_ss + lc * 16,
+               lds0 + 2 * TILE + buf * TILE + i * 4096);
+    }
     if (wave < (DO_K ? 2 : 1)) {  // wavefront 0: LSE log2(e) of the 64 rows, wavefront 1: -delta (4 bytes per lane)
       const int r = min(lane, rmax);
       const float* src = ((wave == 0) ? a.lse2 : a.delta) + dlb + (int64_t)hq * a.dl_sh + (q0 + jq * BQ + r);
