@@ -356,8 +356,19 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
       }
     }
     // P^T = exp2(S^T c - LSE), dS^T = P^T (dP^T - delta); masked positions contribute nothing
+    // masked positions (beyond the sequence, above the causal diagonal) get a score whose exponential is 0; only the
+    // diagonal and tail tiles run this
     const bool need_mask = (j * BN + BN > Lk) || (a.is_causal && j * BN + BN - 1 > wave_row_lo + off);
-    const int lim = need_mask ? min(last_k, causal_row_lim) - j * BN - 4 * g : 0x7fffffff;
+    if (need_mask) {
+      const int lim = min(last_k, causal_row_lim) - j * BN - 4 * g;  // element index e is visible iff e <= lim
+      const float gone = (c < 0.f) ? INFINITY : -INFINITY;           // times c: -inf (c is never 0)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int e = 8 * (v >> 2) + (v & 3);
+        if (e > lim) s0[v] = gone;
+        if (32 + e > lim) s1[v] = gone;
+      }
+    }
     const uint32_t drop_tile = DROP ? (drop_row ^ drop_col_term((uint32_t)(j * (BN / 2) + 2 * g))) : 0u;
     s16x8 dsb[4];
 #pragma unroll
@@ -374,7 +385,6 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
           const int v = 8 * (t & 1) + 2 * e2 + u;
-          const int e = 32 * (t >> 1) + 8 * (v >> 2) + (v & 3);
           const float sv = (t < 2) ? s0[v] : s1[v];
           float dpv = (t < 2) ? p0[v] : p1[v];
           float xl = lse2;  // what is subtracted in the exponent: LSE - bias, in log2 units
@@ -382,7 +392,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
             const uint32_t bw = braw[4 * (t >> 1) + (v >> 2)][(v & 3) >> 1];
             xl = lse2 - Mma<T>::to_float((unsigned short)((v & 1) ? (bw >> 16) : (bw & 0xffffu))) * kLog2e;
           }
-          const float p = (e <= lim) ? fast_exp2(sv * c - xl) : 0.f;
+          const float p = fast_exp2(sv * c - xl);
           if constexpr (DROP) dpv = (((word >> (8 * u)) & 0xffu) <= a.drop_thr) ? dpv * a.drop_rp : 0.f;
           ds[u] = p * (dpv - delta);
         }
@@ -972,6 +982,7 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   a.blockmajor_k = a.is_causal && (int64_t)p->batch * p->heads_k * a.n_kslot < 8 * 256;
   a.scale = p->scale;
   a.scale_log2 = p->scale * kLog2e;
+  if (a.scale_log2 == 0.f) a.scale_log2 = 1e-30f;  // scale 0: uniform probabilities, and -inf * c stays -inf
   const float p_keep = 1.f - p->dropout_p;
   a.drop_thr = (uint32_t)floorf(p_keep * 255.f);
   a.drop_rp = 1.f / p_keep;
