@@ -779,7 +779,10 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
             dp1 = k1 ? dp1 * a.drop_rp : 0.f;
           }
           if constexpr (DO_V) wp[e2] = Mma<T>::pack2(pv0, pv1);
-          if constexpr (DO_K) wd[e2] = Mma<T>::pack2(p0 * (dp0 + d0), p1 * (dp1 + d1));
+          if constexpr (DO_K) {
+            if constexpr (DELTA_INIT) wd[e2] = Mma<T>::pack2(p0 * dp0, p1 * dp1);
+            else wd[e2] = Mma<T>::pack2(p0 * (dp0 + d0), p1 * (dp1 + d1));
+          }
         }
         pb[t] = __builtin_bit_cast(s16x8, wp);
         dsb[t] = __builtin_bit_cast(s16x8, wd);
