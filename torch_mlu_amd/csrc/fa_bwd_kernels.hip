@@ -184,7 +184,9 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
     const int rmax = last_k - j * BN;
     const unsigned char* kt = kp + (uint64_t)(unsigned)(j * BN) * k_ss;
     const unsigned char* vt = vp + (uint64_t)(unsigned)(j * BN) * v_ss;
-    if (rmax >= BN - 1) {  // the whole tile lies inside the sequence: scalar address arithmetic only
+    // the whole tile lies inside the sequence: scalar address arithmetic only (not in the bias variants, which have no
+    // registers to spare for the two offsets)
+    if (!BIAS && rmax >= BN - 1) {
 #pragma unroll
       for (int i = 0; i < NI; ++i)
         dma16s(kt + (uint64_t)(unsigned)(i * 4 * RPI) * k_ss, koff0, lds0 + buf * TILE + i * 4096);
@@ -358,9 +360,10 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
     // P^T = exp2(S^T c - LSE), dS^T = P^T (dP^T - delta); masked positions contribute nothing
     // masked positions (beyond the sequence, above the causal diagonal) get a score whose exponential is 0; only the
     // diagonal and tail tiles run this
+    // (the bias variant, short of registers, selects per element in the loop below instead)
     const bool need_mask = (j * BN + BN > Lk) || (a.is_causal && j * BN + BN - 1 > wave_row_lo + off);
-    if (need_mask) {
-      const int lim = min(last_k, causal_row_lim) - j * BN - 4 * g;  // element index e is visible iff e <= lim
+    const int lim = need_mask ? min(last_k, causal_row_lim) - j * BN - 4 * g : 0x7fffffff;  // element e visible iff e <= lim
+    if (!BIAS && need_mask) {
       const float gone = (c < 0.f) ? INFINITY : -INFINITY;           // times c: -inf (c is never 0)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
@@ -392,7 +395,8 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
             const uint32_t bw = braw[4 * (t >> 1) + (v >> 2)][(v & 3) >> 1];
             xl = lse2 - Mma<T>::to_float((unsigned short)((v & 1) ? (bw >> 16) : (bw & 0xffffu))) * kLog2e;
           }
-          const float p = fast_exp2(sv * c - xl);
+          float p = fast_exp2(sv * c - xl);
+          if constexpr (BIAS) p = (32 * (t >> 1) + 8 * (v >> 2) + (v & 3) <= lim) ? p : 0.f;
           if constexpr (DROP) dpv = (((word >> (8 * u)) & 0xffu) <= a.drop_thr) ? dpv * a.drop_rp : 0.f;
           ds[u] = p * (dpv - delta);
         }
@@ -587,7 +591,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     const int rmax = Lq - 1 - jq * BQ;
     const unsigned char* qt = a.q + qb + (int64_t)(q0 + jq * BQ) * a.q_ss + (int64_t)hq * a.q_sh;
     const unsigned char* dt = a.dout + dob + (int64_t)(q0 + jq * BQ) * a.do_ss + (int64_t)hq * a.do_sh;
-    if (rmax >= BQ - 1) {  // the whole tile lies inside the sequence: scalar address arithmetic only
+    if (!BIAS && rmax >= BQ - 1) {  // the whole tile lies inside the sequence: scalar address arithmetic only
 #pragma unroll
       for (int i = 0; i < NI; ++i)
         dma16s(qt + (uint64_t)(unsigned)(i * 4 * RPI) * q_ss, qoff0, lds0 + buf * TILE + i * 4096);
