@@ -417,3 +417,29 @@ def test_plain_sdpa_with_mask_and_dropout_trains_on_this_build():
             acc += F.scaled_dot_product_attention(qd, kd, vd, attn_mask=pad, dropout_p=0.1).float()
         ref = F.scaled_dot_product_attention(qd, kd, vd, attn_mask=pad).float()
     assert (acc / 64 - ref).abs().mean().item() < 0.02
+
+
+def test_packed_sequences_with_top_left_mask():
+    """The mask modes are per sequence in packed mode too: forward and backward of ragged sequences with the causal
+    mask aligned top-left, against the dense oracle on each sequence."""
+    lens_q, lens_k = [40, 130, 1, 64], [100, 70, 5, 64]
+    Hq, Hk, D = 4, 2, 64
+    cu_q = np.concatenate([[0], np.cumsum(lens_q)]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)
+    Tq, Tk = int(cu_q[-1]), int(cu_k[-1])
+    q, k, v, do = (seeded((Tq, Hq, D), 1300, HF), seeded((Tk, Hk, D), 1301, HF), seeded((Tk, Hk, D), 1302, HF),
+                   seeded((Tq, Hq, D), 1303, HF))
+    qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
+    cq, ck = torch.from_numpy(cu_q).to(DEV), torch.from_numpy(cu_k).to(DEV)
+    out, lse = capi.fa_forward_packed(qd, kd, vd, cq, ck, max(lens_q), max(lens_k), is_causal=capi.FA_MASK_CAUSAL_TOP_LEFT)
+    grads = capi.fa_backward_packed(dod, qd, kd, vd, out, lse, cq, ck, max(lens_q), max(lens_k),
+                                    is_causal=capi.FA_MASK_CAUSAL_TOP_LEFT)
+    for b in range(4):
+        qs, ks = slice(cu_q[b], cu_q[b + 1]), slice(cu_k[b], cu_k[b + 1])
+        args = [t.transpose(0, 1)[None] for t in (q[qs], k[ks], v[ks])]
+        ro, rl = oracle.sdpa_oracle(*args, is_causal=True, causal_top_left=True)
+        assert np.abs(out[qs].float().cpu().numpy() - ro[0].transpose(1, 0, 2)).max() <= 5e-3
+        assert np.abs(lse[:, qs].cpu().numpy() - rl[0]).max() <= 1e-3
+        want = oracle.sdpa_backward_oracle(*args, do[qs].transpose(0, 1)[None], is_causal=True, causal_top_left=True)
+        for name, g, w, sl in zip(("dq", "dk", "dv"), grads, want, (qs, ks, ks)):
+            _close(name, g[sl].transpose(0, 1)[None], w, HF)

@@ -347,7 +347,7 @@ def fa_backward_packed(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_
     p.batch, p.heads_q, p.heads_k = cu_seqlens_q.numel() - 1, Hq, k.shape[1]
     p.seqlen_q, p.seqlen_k, p.head_dim, p.total_q = max_seqlen_q, max_seqlen_k, D, Tq
     p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
-    p.dtype, p.is_causal, p.reserved = _dtype_code(q.dtype), 1 if is_causal else 0, 0
+    p.dtype, p.is_causal, p.reserved = _dtype_code(q.dtype), int(is_causal), 0
     _set_dropout(p, dropout_p, rng)
     _launch_bwd(p, q.device)
     return dq, dk, dv
