@@ -70,7 +70,7 @@ typedef struct fa_bwd_params {
   int32_t heads_k;
   int32_t seqlen_q;  /* dense: rows per sequence; packed: max over sequences */
   int32_t seqlen_k;
-  int32_t head_dim;  /* multiple of 8, 8..128 */
+  int32_t head_dim;  /* multiple of 8, 8..256 (FlashAttention_internal.cpp:355-357) */
   int64_t total_q;   /* packed: rows of q (sizes the delta scratch); dense: ignored */
 
   float scale;
@@ -96,7 +96,7 @@ typedef struct fa_bwd_params {
   int64_t dbias_stride_b, dbias_stride_h, dbias_stride_q;
 } fa_bwd_params;
 
-/* Host-only validation: FA_OK or a negative code (FA_ERR_UNSUPPORTED for head_dim > 128). */
+/* Host-only validation: FA_OK or a negative code (FA_ERR_UNSUPPORTED for head_dim > 256). */
 int fa_bwd_validate(const fa_bwd_params* p);
 
 /* Bytes of device scratch fa_bwd_launch needs (-rowsum(dO o O) and LSE log2(e), two fp32 per query row and head);

@@ -175,7 +175,7 @@ def test_bwd_validate_accepts_good_params_and_sizes_delta_scratch():
     (dict(batch=0), capi.FA_ERR_BAD_ARG),
     (dict(reserved=3), capi.FA_ERR_BAD_ARG),
     (dict(cu_seqlens_k=0xb000), capi.FA_ERR_BAD_ARG),
-    (dict(head_dim=136), capi.FA_ERR_UNSUPPORTED),      # the reference's backward stops at 128 as well
+    (dict(head_dim=264), capi.FA_ERR_UNSUPPORTED),      # "FlashAttention backward only supports head dimension at most 256"
     (dict(head_dim=100), capi.FA_ERR_UNSUPPORTED),
     (dict(dtype=3), capi.FA_ERR_UNSUPPORTED),
     (dict(heads_k=3), capi.FA_ERR_UNSUPPORTED),

@@ -219,13 +219,7 @@ def test_dense_backward_op_layout_contract():
 
 
 def test_backward_errors():
-    q, k, v, do = (t.to(DEV) for t in _inputs(1, 2, 2, 64, 64, 256, BF, 1300))
-    out, lse, cq, ck, mq, mk, seed, offset, _ = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, 0.0, False,
-                                                                                                  False)
-    with pytest.raises(RuntimeError, match="head dimension at most 128"):
-        torch.ops.aten._scaled_dot_product_flash_attention_backward(do, q, k, v, out, lse, cq, ck, mq, mk, 0.0, False,
-                                                                    seed, offset)
-    q, k, v, do = (t[..., :64].contiguous() for t in (q, k, v, do))
+    q, k, v, do = (t.to(DEV) for t in _inputs(1, 2, 2, 64, 64, 64, BF, 1300))
     out, lse, cq, ck, mq, mk, seed, offset, _ = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, 0.0, False,
                                                                                                   False)
     with pytest.raises(RuntimeError, match="dropout_p must be in"):
@@ -260,3 +254,32 @@ def test_full_size_causal_prefill_properties_and_sampled_heads():
         sl = (slice(bi, bi + 1), slice(hi, hi + 1))
         _check_grads((dq[sl], dk[sl], dv[sl]), q[sl].cpu(), k[sl].cpu(), v[sl].cpu(), do[sl].cpu(), True, None,
                      reference_rule=False)
+
+
+@pytest.mark.parametrize("dtype", [BF, HF])
+@pytest.mark.parametrize("D", [136, 160, 192, 256])
+def test_head_dims_above_128(dtype, D):
+    """The reference's backward takes head dimensions up to 256 and its test grid uses 128 and 256
+    (FlashAttention_internal.cpp:355-357, test_scaled_dot_product_attention.py:938-969)."""
+    for i, (B, Hq, Hk, Sq, Sk, causal) in enumerate([(1, 2, 2, 64, 64, False), (2, 4, 2, 130, 200, True),
+                                                     (1, 2, 1, 257, 129, True), (1, 1, 1, 1, 17, False)]):
+        q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, dtype, 1400 + 7 * i)
+        _check_grads(_fwd_bwd_capi(q, k, v, do, causal), q, k, v, do, causal, None, reference_rule=(i == 1))
+
+
+def test_reference_backward_grid_head_dim_256():
+    """One corner of the reference's backward grid at head_dim 256 (B=4, H=4, Sq=512, Sk=1024, fp16, scale 1/D, causal and
+    not), through the registered ops and autograd."""
+    B, H, Sq, Sk, D = 4, 4, 512, 1024, 256
+    q, k, v, do = _inputs(B, H, H, Sq, Sk, D, HF, 1500)
+    for causal in (False, True):
+        if causal and Sq != Sk:
+            kk, vv = k[:, :, :Sq].contiguous(), v[:, :, :Sq].contiguous()     # F.sdpa's causal needs square here
+        else:
+            kk, vv = k, v
+        qd, kd, vd = (t.to(DEV).requires_grad_() for t in (q, kk, vv))
+        n0 = torch_mlu_amd.launch_count()
+        out = F.scaled_dot_product_attention(qd, kd, vd, is_causal=causal, scale=1.0 / D)
+        out.backward(do.to(DEV))
+        assert torch_mlu_amd.launch_count() == n0 + 2
+        _check_grads((qd.grad, kd.grad, vd.grad), q, kk, vv, do, causal, 1.0 / D, reference_rule=False)

@@ -286,9 +286,9 @@ def test_backward_op_errors():
         args(do=do.to(BF))
     with pytest.raises(RuntimeError, match="same dtype as query"):
         args(bias=torch.zeros(16, 16, device=DEV))
-    q256 = torch.zeros(1, 16, 2, 256, dtype=HF, device=DEV)
-    with pytest.raises(RuntimeError, match="at most 128"):
-        aten._efficient_attention_backward(q256, q256, q256, q256, None, q256, None, None, 16, 16,
+    q264 = torch.zeros(1, 16, 2, 264, dtype=HF, device=DEV)
+    with pytest.raises(RuntimeError, match="at most 256"):
+        aten._efficient_attention_backward(q264, q264, q264, q264, None, q264, None, None, 16, 16,
                                            torch.zeros(1, 2, 16, device=DEV), 0.0, seed, offset, 0, False)
 
 

@@ -353,7 +353,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> flash_attention_backward(
   TORCH_CHECK(out.scalar_type() == query.scalar_type(), "query and out must have the same dtype");
   TORCH_CHECK(grad_out.sizes() == query.sizes() && out.sizes() == query.sizes(), "dout and out must have the shape of query");
   TORCH_CHECK(logsumexp.scalar_type() == at::kFloat && logsumexp.is_cuda(), "logsumexp must be a float32 tensor on the device");
-  TORCH_CHECK(query.size(-1) <= 128, "FlashAttention backward only supports head dimension at most 128 in this build");
+  TORCH_CHECK(query.size(-1) <= 256, "FlashAttention backward only supports head dimension at most 256");  // :355-357
 
   const c10::OptionalDeviceGuard guard(query.device());
   const float softmax_scale = resolve_scale(query, scale);
@@ -647,7 +647,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> efficient_attention_b
   const int64_t B = query.size(0), Sq = query.size(1), Hq = query.size(2), D = query.size(3);
   const int64_t Sk = key.size(1), Hk = key.size(2);
   TORCH_CHECK(B > 0, "batch size must be positive");
-  TORCH_CHECK(D <= 128, "FlashAttention backward only supports head dimension at most 128 in this build");
+  TORCH_CHECK(D <= 256, "FlashAttention backward only supports head dimension at most 256");
   TORCH_CHECK(D % 8 == 0, "head dimension must be a multiple of 8");
   TORCH_CHECK(Sq <= INT32_MAX && Sk <= INT32_MAX && B <= INT32_MAX, "sequence length too large");
   TORCH_CHECK(logsumexp.dim() == 3 && logsumexp.size(0) == B && logsumexp.size(1) == Hq && logsumexp.size(2) >= Sq,

@@ -103,6 +103,9 @@ struct TileIO {
   static constexpr int RPI = 64 / CPR;
   static constexpr int KS = DP / 16;
   static constexpr int MB = DP / 32;
+  // consecutive DMA instructions of a wavefront are 4 RPI rows apart; the swizzle repeats every 16 rows, so at
+  // head_dim 256 (8 rows apart) even and odd instructions need their own chunk index
+  static constexpr int NV = (4 * RPI) % 16 == 0 ? 1 : 2;
 };
 
 // ---------------------------------------------------------------------------------------------------------
@@ -112,9 +115,10 @@ struct TileIO {
 // = 4 consecutive keys per load, as in the forward); dS of the tile, already packed for the dQ product, is also what
 // the gradient of the bias is, and is stored from here (tiles the causal mask skips are stored as zeros).
 template <typename T, int DP, bool DROP, bool BIAS>
-__global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
+__global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const BArgs a) {
   using IO = TileIO<T, DP>;
   constexpr int CPR = IO::CPR, ROWB = IO::ROWB, TILE = IO::TILE, NI = IO::NI, RPI = IO::RPI, KS = IO::KS, MB = IO::MB;
+  constexpr int NV = IO::NV;
   constexpr int BM = 128, BN = 64;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // K0 K1 V0 V1
 
@@ -174,12 +178,21 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
 
   // ---- DMA: rows clamped to the last valid one, logical chunk un-swizzled on the global side ----
   const int dma_r = wave * RPI + lane / CPR;
-  int lc = (lane % CPR) ^ swzU<DP>(dma_r);  // invariant under the per-instruction row step (multiple of 16)
-  if (lc * 8 >= D) lc = 0;
+  int lcv[NV];  // logical chunk this lane fetches, per instruction parity (see TileIO::NV)
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    lcv[n] = (lane % CPR) ^ swzU<DP>(dma_r + n * 4 * RPI);
+    if (lcv[n] * 8 >= D) lcv[n] = 0;
+  }
   const unsigned k_ss = (unsigned)a.k_ss, v_ss = (unsigned)a.v_ss;
   const unsigned lds0 = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + wave * 1024;
   // per-lane byte offsets of a full tile's first DMA block; the later blocks only move the scalar base
-  const unsigned koff0 = (unsigned)dma_r * k_ss + lc * 16, voff0 = (unsigned)dma_r * v_ss + lc * 16;
+  unsigned koff0[NV], voff0[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    koff0[n] = (unsigned)dma_r * k_ss + lcv[n] * 16;
+    voff0[n] = (unsigned)dma_r * v_ss + lcv[n] * 16;
+  }
   auto issue_tile = [&](int j, int buf) {
     const int rmax = last_k - j * BN;
     const unsigned char* kt = kp + (uint64_t)(unsigned)(j * BN) * k_ss;
@@ -189,18 +202,18 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BArgs a) {
     if (!BIAS && rmax >= BN - 1) {
 #pragma unroll
       for (int i = 0; i < NI; ++i)
-        dma16s(kt + (uint64_t)(unsigned)(i * 4 * RPI) * k_ss, koff0, lds0 + buf * TILE + i * 4096);
+        dma16s(kt + (uint64_t)(unsigned)(i * 4 * RPI) * k_ss, koff0[i % NV], lds0 + buf * TILE + i * 4096);
 #pragma unroll
       for (int i = 0; i < NI; ++i)
-        dma16s(vt + (uint64_t)(unsigned)(i * 4 * RPI) * v_ss, voff0, lds0 + 2 * TILE + buf * TILE + i * 4096);
+        dma16s(vt + (uint64_t)(unsigned)(i * 4 * RPI) * v_ss, voff0[i % NV], lds0 + 2 * TILE + buf * TILE + i * 4096);
       return;
     }
 #pragma unroll
     for (int i = 0; i < NI; ++i)
-      dma16s(kt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * k_ss + lc * 16, lds0 + buf * TILE + i * 4096);
+      dma16s(kt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * k_ss + lcv[i % NV] * 16, lds0 + buf * TILE + i * 4096);
 #pragma unroll
     for (int i = 0; i < NI; ++i)
-      dma16s(vt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * v_ss + lc * 16, lds0 + 2 * TILE + buf * TILE + i * 4096);
+      dma16s(vt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * v_ss + lcv[i % NV] * 16, lds0 + 2 * TILE + buf * TILE + i * 4096);
   };
 
   const float c = a.scale_log2;
@@ -472,10 +485,11 @@ constexpr int kDK = 1, kDV = 2;
 // first, since -inf * 0 would turn the whole row into NaN; the exponential of either is 0.  A block's loads are issued
 // ahead of its S / dP MFMAs and consumed after them.
 template <typename T, int DP, int WHAT, bool DROP, bool BIAS>
-__global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
+__global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const BArgs a) {
   constexpr bool DO_K = (WHAT & kDK) != 0, DO_V = (WHAT & kDV) != 0;
   using IO = TileIO<T, DP>;
   constexpr int CPR = IO::CPR, ROWB = IO::ROWB, TILE = IO::TILE, NI = IO::NI, RPI = IO::RPI, KS = IO::KS, MB = IO::MB;
+  constexpr int NV = IO::NV;
   constexpr int BKV = 128, BQ = 64;
   constexpr int VEC = 4 * TILE;  // Q0 Q1 dO0 dO1 | lse[2][64] delta[2][64]
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -525,8 +539,12 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
   const int D = a.head_dim;
 
   const int dma_r = wave * RPI + lane / CPR;
-  int lc = (lane % CPR) ^ swzU<DP>(dma_r);
-  if (lc * 8 >= D) lc = 0;
+  int lcv[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    lcv[n] = (lane % CPR) ^ swzU<DP>(dma_r + n * 4 * RPI);
+    if (lcv[n] * 8 >= D) lcv[n] = 0;
+  }
   const unsigned q_ss = (unsigned)a.q_ss, do_ss = (unsigned)a.do_ss;
   const unsigned lds0 = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + wave * 1024;
   const unsigned ldsv = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + VEC;
@@ -583,7 +601,12 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
   }
 
   // per-lane byte offsets of a full tile's first DMA block; the later blocks only move the scalar base
-  const unsigned qoff0 = (unsigned)dma_r * q_ss + lc * 16, dooff0 = (unsigned)dma_r * do_ss + lc * 16;
+  unsigned qoff0[NV], dooff0[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    qoff0[n] = (unsigned)dma_r * q_ss + lcv[n] * 16;
+    dooff0[n] = (unsigned)dma_r * do_ss + lcv[n] * 16;
+  }
   // ---- DMA of a (query head, query tile): Q rows, dO rows, LSE and delta of the 64 rows ----
   auto issue_iter = [&](int it, int buf) {
     const int hq = hk * a.group + it / nq;
@@ -594,17 +617,17 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dkv_kernel(const BArgs a) {
     if (!BIAS && rmax >= BQ - 1) {  // the whole tile lies inside the sequence: scalar address arithmetic only
 #pragma unroll
       for (int i = 0; i < NI; ++i)
-        dma16s(qt + (uint64_t)(unsigned)(i * 4 * RPI) * q_ss, qoff0, lds0 + buf * TILE + i * 4096);
+        dma16s(qt + (uint64_t)(unsigned)(i * 4 * RPI) * q_ss, qoff0[i % NV], lds0 + buf * TILE + i * 4096);
 #pragma unroll
       for (int i = 0; i < NI; ++i)
-        dma16s(dt + (uint64_t)(unsigned)(i * 4 * RPI) * do_ss, dooff0, lds0 + 2 * TILE + buf * TILE + i * 4096);
+        dma16s(dt + (uint64_t)(unsigned)(i * 4 * RPI) * do_ss, dooff0[i % NV], lds0 + 2 * TILE + buf * TILE + i * 4096);
     } else {
 #pragma unroll
       for (int i = 0; i < NI; ++i)
-        dma16s(qt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * q_ss + lc * 16, lds0 + buf * TILE + i * 4096);
+        dma16s(qt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * q_ss + lcv[i % NV] * 16, lds0 + buf * TILE + i * 4096);
 #pragma unroll
       for (int i = 0; i < NI; ++i)
-        dma16s(dt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * do_ss + lc * 16,
+        dma16s(dt, (unsigned)min(dma_r + i * 4 * RPI, rmax) * do_ss + lcv[i % NV] * 16,
                lds0 + 2 * TILE + buf * TILE + i * 4096);
     }
     if (wave < (DO_K ? 2 : 1)) {  // wavefront 0: LSE log2(e) of the 64 rows, wavefront 1: -delta (4 bytes per lane)
@@ -879,7 +902,7 @@ int bwd_validate(const fa_bwd_params* p) {
       return FA_ERR_BAD_ARG;
   }
   if (p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_UNSUPPORTED;
-  if (p->head_dim > 128 || (p->head_dim & 7)) return FA_ERR_UNSUPPORTED;
+  if (p->head_dim > 256 || (p->head_dim & 7)) return FA_ERR_UNSUPPORTED;
   if (p->heads_q % p->heads_k) return FA_ERR_UNSUPPORTED;
   const uintptr_t al = (uintptr_t)p->q | (uintptr_t)p->k | (uintptr_t)p->v | (uintptr_t)p->out | (uintptr_t)p->dout |
                        (uintptr_t)p->dq | (uintptr_t)p->dk | (uintptr_t)p->dv;
@@ -936,6 +959,21 @@ int bwd_launch(const BArgs& a, hipStream_t st) {
     }
   }
   return FA_OK;
+}
+
+template <typename T, int DP>
+int bwd_dispatch_dp(const BArgs& a, hipStream_t st, bool drop, bool bias) {
+  if (drop && bias) return bwd_launch<T, DP, true, true>(a, st);
+  if (drop) return bwd_launch<T, DP, true, false>(a, st);
+  if (bias) return bwd_launch<T, DP, false, true>(a, st);
+  return bwd_launch<T, DP, false, false>(a, st);
+}
+
+template <typename T>
+int bwd_dispatch(const BArgs& a, hipStream_t st, int dp, bool drop, bool bias) {
+  if (dp == 64) return bwd_dispatch_dp<T, 64>(a, st, drop, bias);
+  if (dp == 128) return bwd_dispatch_dp<T, 128>(a, st, drop, bias);
+  return bwd_dispatch_dp<T, 256>(a, st, drop, bias);
 }
 
 }  // namespace
@@ -996,25 +1034,10 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   a.seed_ptr = p->philox_seed;
   a.offset_ptr = p->philox_offset;
   hipStream_t st = (hipStream_t)stream;
-  const int dp = p->head_dim <= 64 ? 64 : 128;
-  if (p->dropout_p > 0.f && p->bias) {
-    if (p->dtype == FA_DTYPE_BF16)
-      return dp == 64 ? bwd_launch<__bf16, 64, true, true>(a, st) : bwd_launch<__bf16, 128, true, true>(a, st);
-    return dp == 64 ? bwd_launch<_Float16, 64, true, true>(a, st) : bwd_launch<_Float16, 128, true, true>(a, st);
-  }
-  if (p->dropout_p > 0.f) {
-    if (p->dtype == FA_DTYPE_BF16)
-      return dp == 64 ? bwd_launch<__bf16, 64, true, false>(a, st) : bwd_launch<__bf16, 128, true, false>(a, st);
-    return dp == 64 ? bwd_launch<_Float16, 64, true, false>(a, st) : bwd_launch<_Float16, 128, true, false>(a, st);
-  }
-  if (p->bias) {
-    if (p->dtype == FA_DTYPE_BF16)
-      return dp == 64 ? bwd_launch<__bf16, 64, false, true>(a, st) : bwd_launch<__bf16, 128, false, true>(a, st);
-    return dp == 64 ? bwd_launch<_Float16, 64, false, true>(a, st) : bwd_launch<_Float16, 128, false, true>(a, st);
-  }
-  if (p->dtype == FA_DTYPE_BF16)
-    return dp == 64 ? bwd_launch<__bf16, 64, false, false>(a, st) : bwd_launch<__bf16, 128, false, false>(a, st);
-  return dp == 64 ? bwd_launch<_Float16, 64, false, false>(a, st) : bwd_launch<_Float16, 128, false, false>(a, st);
+  const int dp = p->head_dim <= 64 ? 64 : (p->head_dim <= 128 ? 128 : 256);
+  const bool drop = p->dropout_p > 0.f, bias = p->bias != nullptr;
+  if (p->dtype == FA_DTYPE_BF16) return bwd_dispatch<__bf16>(a, st, dp, drop, bias);
+  return bwd_dispatch<_Float16>(a, st, dp, drop, bias);
 }
 
 }  // extern "C"

@@ -96,11 +96,9 @@ bool check_for_attn_mask(const sdp_params& p, bool debug) {
 
 bool check_head_dim_size(const sdp_params& p, bool debug) {
   const int64_t dq = p.query.size(-1), dk = p.key.size(-1), dv = p.value.size(-1);
-  const int64_t dmax = input_requires_grad(p) ? 128 : 256;  // this build's backward stops at 128
-  if (!(dq == dk && dq == dv && dq <= dmax && dq >= 8 && dq % 8 == 0)) {
+  if (!(dq == dk && dq == dv && dq <= 256 && dq >= 8 && dq % 8 == 0)) {
     if (debug)
-      TORCH_WARN("Flash attention requires q,k,v to have the same last dimension, at most ", dmax,
-                 input_requires_grad(p) ? " when a gradient is required." : ".",
+      TORCH_WARN("Flash attention requires q,k,v to have the same last dimension, at most 256.",
                  " Flash attention requires last dimension of inputs to be divisible by 8.", " Got Query.size(-1): ", dq,
                  ", Key.size(-1): ", dk, ", Value.size(-1): ", dv, " instead.");
     return false;
@@ -195,15 +193,8 @@ bool check_head_dim_size_mem_efficient(const sdp_params& p, bool debug) {
   return true;
 }
 
-// Not in the reference (its backward is the vendor's): what this build's does not implement.
+// Not in the reference: what the mem-efficient entry points of this build need beyond the shared constraints.
 bool check_this_build_mem_efficient(const sdp_params& p, bool debug) {
-  const bool mask_grad = p.attn_mask.has_value() && p.attn_mask->defined() && p.attn_mask->requires_grad();
-  if ((input_requires_grad(p) || (at::GradMode::is_enabled() && mask_grad)) && p.query.size(-1) > 128) {
-    if (debug)
-      TORCH_WARN("The backward of this build stops at head dimension 128; a gradient is required and query.size(-1) is ",
-                 p.query.size(-1), ".");
-    return false;
-  }
   if (p.attn_mask.has_value() && p.attn_mask->defined()) {
     const auto mt = p.attn_mask->scalar_type();
     if ((mt != at::kBool && mt != p.query.scalar_type()) || p.attn_mask->dim() > 4 || !p.attn_mask->is_cuda() ||
