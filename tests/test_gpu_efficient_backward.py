@@ -443,3 +443,92 @@ def test_packed_sequences_with_top_left_mask():
         want = oracle.sdpa_backward_oracle(*args, do[qs].transpose(0, 1)[None], is_causal=True, causal_top_left=True)
         for name, g, w, sl in zip(("dq", "dk", "dv"), grads, want, (qs, ks, ks)):
             _close(name, g[sl].transpose(0, 1)[None], w, HF)
+
+
+# ---- the reference's own mem-efficient tests (test_scaled_dot_product_attention.py:1288-1727), restated ----------------
+def _math_sdpa_grads(q, k, v, mask, do, scale, dtype):
+    """out and gradients of plain-torch math attention on the device in `dtype` (float32: the reference's `*_ref`; the
+    inputs' dtype: its `*_lp_ref`)."""
+    qq, kk, vv, mm = (t.detach().to(dtype).requires_grad_() for t in (q, k, v, mask))
+    s = torch.matmul(qq, kk.transpose(-1, -2)) * (scale if scale is not None else 1.0 / math.sqrt(q.shape[-1])) + mm
+    out = torch.matmul(torch.softmax(s, -1), vv)
+    out.backward(do.to(dtype))
+    return out.detach(), qq.grad, kk.grad, vv.grad, mm.grad
+
+
+@pytest.mark.parametrize("dtype", [HF, BF])
+@pytest.mark.parametrize("B,Sq,Sk,D,l1", [(4, 512, 1024, 128, False), (4, 1024, 512, 256, True), (8, 512, 512, 128, True),
+                                          (4, 2048, 512, 256, False)])
+def test_reference_memory_efficient_backward_grid(dtype, B, Sq, Sk, D, l1):
+    """A slice of the reference's grid (:1372-1727): H = 4, head_dim 128 and 256, scale None or 1/D, a full random mask that
+    requires a gradient, inputs uniform in [0, 1); its acceptance rule — within fudge x the error of the same math in the
+    low precision (fudge 4 for dQ, 2 otherwise) — against float32 math on the device."""
+    H, scale = 4, (1.0 / D if l1 else None)
+    g = torch.Generator().manual_seed(B * Sq + Sk + D)
+    q, k, v, do = (torch.rand(B, H, s, D, generator=g).to(dtype).to(DEV) for s in (Sq, Sk, Sk, Sq))
+    mask = torch.rand(B, H, Sq, Sk, generator=g).to(dtype).to(DEV)
+    qd, kd, vd, md = (t.clone().requires_grad_() for t in (q, k, v, mask))
+    n0 = torch_mlu_amd.launch_count()
+    with torch_mlu_amd.backends.sdp_kernel(enable_mem_efficient=True, enable_flash=False, enable_math=False):
+        out = F.scaled_dot_product_attention(qd, kd, vd, md, dropout_p=0.0, is_causal=False, scale=scale)
+    out.backward(do)
+    assert torch_mlu_amd.launch_count() == n0 + 2
+    ref = _math_sdpa_grads(q, k, v, mask, do, scale, torch.float32)
+    lp = _math_sdpa_grads(q, k, v, mask, do, scale, dtype)
+    for name, got, r, l, fudge in zip(("out", "dq", "dk", "dv", "dmask"), (out, qd.grad, kd.grad, vd.grad, md.grad), ref,
+                                      lp, (2.0, 4.0, 2.0, 2.0, 4.0)):
+        atol, rtol = oracle.get_tolerances(r.cpu().numpy(), l.float().cpu().numpy(), NAME[dtype], fudge)
+        assert torch.allclose(got.float(), r, atol=atol, rtol=rtol), (name, (got.float() - r).abs().max().item(), atol, rtol)
+
+
+def test_reference_mask_variants_train():
+    """Masks of 1 to 4 dimensions with the efficient backend forced, forward and backward (:1288-1321); here with the
+    gradients checked against the oracle on a smaller problem."""
+    B, H, Sq, Sk, D = 2, 3, 96, 96, 128
+    q, k, v, do = _inputs(B, H, H, Sq, Sk, D, HF, 1600)
+    for shp in ((Sk,), (Sq, Sk), (H, Sq, Sk), (B, H, Sq, Sk)):
+        mask = seeded(shp, 1601 + len(shp), HF, std=1.0)
+        qd, kd, vd = (t.to(DEV).requires_grad_() for t in (q, k, v))
+        with torch_mlu_amd.backends.sdp_kernel(enable_mem_efficient=True, enable_flash=False, enable_math=False):
+            out = F.scaled_dot_product_attention(qd, kd, vd, mask.to(DEV))
+        out.backward(do.to(DEV))
+        want = oracle.sdpa_backward_oracle(q, k, v, do, attn_bias=mask.double().numpy())
+        for name, t, w in zip(("dq", "dk", "dv"), (qd, kd, vd), want):
+            _close(name, t.grad, w, HF)
+
+
+def test_reference_non_contiguous_mask():
+    """A mask that is one row seen through strides (0, 0, 0, 1) (:1323-1346)."""
+    B, H, Sq, Sk, D = 2, 4, 130, 260, 128
+    q, k, v, do = _inputs(B, H, H, Sq, Sk, D, HF, 1700)
+    base = seeded((B, H, Sq, Sk), 1701, HF, std=1.0)
+    mask = torch.as_strided(base.to(DEV), (B, H, Sq, Sk), (0, 0, 0, 1))
+    qd, kd, vd = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    with torch_mlu_amd.backends.sdp_kernel(enable_mem_efficient=True, enable_flash=False, enable_math=False):
+        out = F.scaled_dot_product_attention(qd, kd, vd, mask)
+    out.backward(do.to(DEV))
+    row = base.reshape(-1)[:Sk].double().numpy()[None, None, None, :]
+    ro, _ = oracle.sdpa_oracle(q, k, v, attn_bias=row)
+    assert np.abs(out.detach().float().cpu().numpy() - ro).max() <= 5e-3
+    want = oracle.sdpa_backward_oracle(q, k, v, do, attn_bias=row)
+    for name, t, w in zip(("dq", "dk", "dv"), (qd, kd, vd), want):
+        _close(name, t.grad, w, HF)
+
+
+def test_reference_long_sequence_mask():
+    """8192 x 8192 mask for 32 heads (4 GiB in fp16), forward and backward (:1349-1370); one head checked against float32
+    math on the device."""
+    B, H, S, D = 1, 32, 8192, 128
+    g = torch.Generator(device=DEV).manual_seed(5)
+    q, k, v, do = ((torch.randn(B, H, S, D, generator=g, device=DEV) * 0.5).to(HF) for _ in range(4))
+    mask = torch.randn(B, H, S, S, generator=g, device=DEV, dtype=HF)
+    qd, kd, vd = (t.clone().requires_grad_() for t in (q, k, v))
+    with torch_mlu_amd.backends.sdp_kernel(enable_mem_efficient=True, enable_flash=False, enable_math=False):
+        out = F.scaled_dot_product_attention(qd, kd, vd, mask)
+    out.backward(do)
+    h = 17
+    ref = _math_sdpa_grads(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], mask[:, h:h + 1], do[:, h:h + 1], None, torch.float32)
+    for name, got, r in zip(("out", "dq", "dk", "dv"), (out, qd.grad, kd.grad, vd.grad), ref):
+        err = (got[:, h:h + 1].float() - r).abs().max().item()
+        assert err <= 2 * EPS[HF] * max(r.abs().max().item(), 0.25), (name, err)
+    assert all(torch.isfinite(t.grad).all().item() for t in (qd, kd, vd))
