@@ -283,3 +283,72 @@ def test_reference_backward_grid_head_dim_256():
         out.backward(do.to(DEV))
         assert torch_mlu_amd.launch_count() == n0 + 2
         _check_grads((qd.grad, kd.grad, vd.grad), q, kk, vv, do, causal, 1.0 / D, reference_rule=False)
+
+
+# ---- the reference's backward grid (test_scaled_dot_product_attention.py:938-1285), a slice of it ----------------------
+def _torch_attention_ref(q, k, v, do, scale, causal, keep, p, dtype):
+    """out and gradients of softmax(scale q k^T + bottom-right causal mask) (dropped with `keep`, rescaled) v, plain torch
+    ops on the device in `dtype` — float32 for the reference's `*_ref`, the inputs' dtype for its `*_lp_ref`."""
+    qq, kk, vv = (t.detach().to(dtype).requires_grad_() for t in (q, k, v))
+    Sq, Sk, D = q.shape[2], k.shape[2], q.shape[3]
+    s = torch.matmul(qq, kk.transpose(-1, -2)) * (scale if scale is not None else 1.0 / math.sqrt(D))
+    if causal:
+        i = torch.arange(Sq, device=q.device)[:, None]
+        j = torch.arange(Sk, device=q.device)[None, :]
+        hidden = j > i + (Sk - Sq)
+        s = s.masked_fill(hidden, float("-inf"))
+    a = torch.softmax(s, -1)
+    if causal and Sk < Sq:   # rows that see no key: 0, as the reference's oracle does (:142-146)
+        a = a.masked_fill(hidden.all(-1)[:, None], 0.0)
+    if keep is not None:
+        a = a * keep.to(dtype) / (1.0 - p)
+    out = torch.matmul(a, vv)
+    out.backward(do.to(dtype))
+    return out.detach(), qq.grad, kk.grad, vv.grad
+
+
+def _reference_grid_case(dtype, B, Sq, Sk, D, l1, causal, p):
+    H, scale = 4, (1.0 / D if l1 else None)
+    g = torch.Generator().manual_seed(B + Sq * 3 + Sk * 5 + D)
+    q, k, v, do = (torch.rand(B, H, s, D, generator=g).to(dtype).to(DEV) for s in (Sq, Sk, Sk, Sq))
+    qd, kd, vd = (t.clone().requires_grad_() for t in (q, k, v))
+    n0 = torch_mlu_amd.launch_count()
+    res = torch.ops.aten._scaled_dot_product_flash_attention(qd, kd, vd, dropout_p=p, is_causal=causal, scale=scale,
+                                                            return_debug_mask=True)
+    out, dbg = res[0], res[-1]
+    keep = (dbg > 0) if p > 0 else None
+    out.backward(do)
+    assert torch_mlu_amd.launch_count() == n0 + 2
+    ref = _torch_attention_ref(q, k, v, do, scale, causal, keep, p, torch.float32)
+    lp = _torch_attention_ref(q, k, v, do, scale, causal, keep, p, dtype)
+    for name, got, r, l, fudge in zip(("out", "dq", "dk", "dv"), (out, qd.grad, kd.grad, vd.grad), ref, lp,
+                                      (2.0, 4.0, 2.0, 2.0)):
+        # the rule's tolerances, computed on the device: atol = fudge * max(|ref - lp|, default), rtol likewise
+        dflt_atol, dflt_rtol = {"float16": (1e-3, 1e-3), "bfloat16": (1e-3, 1.6e-2)}[NAME[dtype]]
+        dev = (r - l.float()).abs()
+        atol = fudge * max(dev.max().item(), dflt_atol)
+        rel = dev / r.abs()
+        rel = torch.where(rel.isnan(), torch.full_like(rel, dflt_rtol), rel).max().item()
+        rtol = fudge * max(rel, dflt_rtol)
+        if rtol > 1e30:
+            rtol = dflt_rtol
+        assert torch.allclose(got.float(), r, atol=atol, rtol=rtol), (
+            name, (B, Sq, Sk, D, l1, causal, p), (got.float() - r).abs().max().item(), atol, rtol)
+
+
+@pytest.mark.parametrize("dtype", [HF, BF])
+@pytest.mark.parametrize("D", [128, 256])
+@pytest.mark.parametrize("p", [0.0, 0.22, 0.48])
+def test_reference_flash_backward_grid(dtype, D, p):
+    """The reference's whole backward grid: B in {4, 8}, Sq, Sk in {512, 1024, 2048}, head_dim 128 / 256, scale None or
+    1/D, causal or not, dropout 0 / 0.22 / 0.48, H = 4, inputs uniform in [0, 1); called as the reference does —
+    aten::_scaled_dot_product_flash_attention(..., return_debug_mask=True) and autograd — and judged by its rule: within
+    fudge x the error of the same math in the low precision (4 for dQ, 2 otherwise, `get_tolerances`, :166-204) against
+    float32 math fed with the returned keep-mask."""
+    for B in (4, 8):
+        for Sq in (512, 1024, 2048):
+            for Sk in (512, 1024, 2048):
+                for l1 in (False, True):
+                    for causal in (True, False):
+                        _reference_grid_case(dtype, B, Sq, Sk, D, l1, causal, p)
+        print(f"B={B} done", flush=True)
