@@ -552,3 +552,44 @@ def test_reference_long_sequence_mask():
         err = (got[:, h:h + 1].float() - r).abs().max().item()
         assert err <= 2 * EPS[HF] * max(r.abs().max().item(), 0.25), (name, err)
     assert all(torch.isfinite(t.grad).all().item() for t in (qd, kd, vd))
+
+
+@pytest.mark.parametrize("dtype", [HF, BF])
+def test_reference_fused_kernels_backward_packed_qkv(dtype):
+    """:728-935: one packed [B, S, 3 H D] leaf, chunked into q, k, v views (contiguous or not), flash and mem-efficient
+    backends forced in turn, causal or not; the gradient that arrives at the packed leaf against float64 math, within
+    the error of the same math in the low precision (`get_tolerances` with its default fudge)."""
+    B, S, H, D = 4, 512, 2, 128
+    g = torch.Generator().manual_seed(12)
+    qkv = torch.randn(B, S, 3 * H * D, generator=g).to(dtype)
+    up = torch.rand(B, H, S, D, generator=g)
+
+    def views(t, contiguous):
+        out = [x.view(B, -1, H, D).transpose(1, 2) for x in t.chunk(3, dim=-1)]
+        return [x.contiguous() for x in out] if contiguous else out
+
+    for contiguous in (True, False):
+        for causal in (True, False):
+            grads = {}
+            for name, flags in (("flash", dict(enable_flash=True, enable_math=False, enable_mem_efficient=False)),
+                                ("mem", dict(enable_flash=False, enable_math=False, enable_mem_efficient=True))):
+                leaf = qkv.to(DEV).requires_grad_()
+                q, k, v = views(leaf, contiguous)
+                n0 = torch_mlu_amd.launch_count()
+                with torch_mlu_amd.backends.sdp_kernel(**flags):
+                    out = F.scaled_dot_product_attention(q, k, v, None, 0.0, causal)
+                out.backward(up.to(dtype).to(DEV))
+                assert torch_mlu_amd.launch_count() == n0 + 2, name
+                grads[name] = leaf.grad.double().cpu()
+            ref_leaf = qkv.double().requires_grad_()
+            lp_leaf = qkv.clone().requires_grad_()
+            for leaf, u in ((ref_leaf, up.double()), (lp_leaf, up.to(dtype))):
+                q, k, v = views(leaf, contiguous)
+                s = torch.matmul(q, k.transpose(-1, -2)) / math.sqrt(D)
+                if causal:
+                    s = s.masked_fill(~torch.ones(S, S, dtype=torch.bool).tril(), float("-inf"))
+                torch.matmul(torch.softmax(s, -1), v).backward(u)
+            atol, rtol = oracle.get_tolerances(ref_leaf.grad.numpy(), lp_leaf.grad.double().numpy(), NAME[dtype])
+            for name, gr in grads.items():
+                assert torch.allclose(gr, ref_leaf.grad, atol=atol, rtol=rtol), (name, contiguous, causal,
+                                                                                 (gr - ref_leaf.grad).abs().max().item(), atol)
