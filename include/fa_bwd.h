@@ -85,8 +85,9 @@ typedef struct fa_bwd_params {
   const int64_t* philox_seed;
   const int64_t* philox_offset;
 
-  /* optional additive bias of the forward (same dtype as q; NULL = none), dense mode only:
-     element (b, h, row, col) at bias + b*bias_stride_b + h*bias_stride_h + row*bias_stride_q + col, h a query head.
+  /* optional additive bias of the forward (same dtype as q; NULL = none):
+     element (b, h, row, col) at bias + b*bias_stride_b + h*bias_stride_h + row*bias_stride_q + col, h a query head;
+     in packed mode b is the sequence and row, col count from the sequence's first row / key.
      Strides may be 0 (broadcast) and must be multiples of 4; the pointer must be 8-byte aligned (as in the forward). */
   const void* bias;
   int64_t bias_stride_b, bias_stride_h, bias_stride_q;

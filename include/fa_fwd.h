@@ -68,10 +68,10 @@ extern "C" {
  * packed row index and lse_stride_b is ignored (the reference's kernel-side buffer is [heads_q, total_q], :129).
  * Rows with no visible key (is_causal and Lk < Lq, Lk == 0, or a bias row that is -inf throughout) get out = 0 and
  * LSE = +inf.
- * bias (optional, dense mode only, same dtype as q): element (b,h,row,col) at bias + b*bias_stride_b + h*bias_stride_h
- * + row*bias_stride_q + col; columns contiguous; stride 0 broadcasts over batch or heads (or rows); the base pointer
- * and all three strides must keep 4-element groups 8-byte aligned (multiples of 4 elements).  A problem with a bias
- * always runs the tile kernel.
+ * bias (optional, same dtype as q): element (b,h,row,col) at bias + b*bias_stride_b + h*bias_stride_h
+ * + row*bias_stride_q + col (packed mode: b = the sequence, row and col counted from its first row / key); columns
+ * contiguous; stride 0 broadcasts over batch or heads (or rows); the base pointer and all three strides must keep
+ * 4-element groups 8-byte aligned (multiples of 4 elements).  A problem with a bias always runs the tile kernel.
  */
 typedef struct fa_fwd_params {
   const void* q;   /* device, 16-byte aligned */

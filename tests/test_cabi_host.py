@@ -185,7 +185,6 @@ def test_bwd_validate_accepts_good_params_and_sizes_delta_scratch():
     (dict(dbias=0xd000, dbias_stride_q=256), capi.FA_ERR_BAD_ARG),          # a bias gradient without a bias
     (dict(bias=0xc000, bias_stride_q=256, dbias=0xd000, dbias_stride_q=0), capi.FA_ERR_BAD_ARG),   # broadcast output
     (dict(bias=0xc000, bias_stride_q=256, dbias=0xd000, dbias_stride_q=256, dbias_stride_h=0), capi.FA_ERR_BAD_ARG),
-    (dict(bias=0xc000, bias_stride_q=256, cu_seqlens_q=0xa000, cu_seqlens_k=0xb000, total_q=200), capi.FA_ERR_UNSUPPORTED),
 ])
 def test_bwd_validate_rejects(over, rc):
     L = capi.lib()
@@ -219,7 +218,7 @@ def test_bias_and_mask_mode_validation_and_plan():
     for over, rc in ((dict(bias=0x7004), capi.FA_ERR_BAD_ARG),                 # 4-key groups must be 8-byte aligned
                      (dict(bias_stride_q=258), capi.FA_ERR_BAD_ARG),
                      (dict(bias_stride_h=-4), capi.FA_ERR_BAD_ARG),
-                     (dict(cu_seqlens_q=0x6000, cu_seqlens_k=0x6100), capi.FA_ERR_UNSUPPORTED),   # packed + bias
+                     (dict(cu_seqlens_q=0x6000, cu_seqlens_k=0x6100), capi.FA_OK),   # a bias is fine in packed mode too
                      (dict(kernel=capi.FA_KERNEL_SPLITKV, seqlen_q=1), capi.FA_ERR_UNSUPPORTED),
                      (dict(is_causal=3), capi.FA_ERR_BAD_ARG)):
         p = _good(**{**dict(bias=0x7000, bias_stride_b=0, bias_stride_h=128 * 256, bias_stride_q=256), **over})

@@ -276,8 +276,8 @@ def test_backward_op_errors():
         o.get("p", 0.0), seed, offset, o.get("cmt", 0), False)
     with pytest.raises(RuntimeError, match="dropout_p must be in"):
         args(p=1.5)
-    with pytest.raises(RuntimeError, match="cu_seqlens are not supported"):
-        args(cu=torch.zeros(2, dtype=torch.int32, device=DEV))
+    with pytest.raises(RuntimeError, match="cu_seqlens_q must have dtype int32"):
+        args(cu=torch.zeros(2, dtype=torch.int64, device=DEV))
     with pytest.raises(RuntimeError, match="custom_mask_type"):
         args(cmt=3)
     with pytest.raises(RuntimeError, match="compute_log_sumexp"):
@@ -593,3 +593,105 @@ def test_reference_fused_kernels_backward_packed_qkv(dtype):
             for name, gr in grads.items():
                 assert torch.allclose(gr, ref_leaf.grad, atol=atol, rtol=rtol), (name, contiguous, causal,
                                                                                  (gr - ref_leaf.grad).abs().max().item(), atol)
+
+
+@pytest.mark.parametrize("mask", ["none", "tl"])
+def test_packed_sequences_with_bias(mask):
+    """Bias in packed mode: indexed by sequence and by the row / key position inside the sequence; forward, backward and
+    the bias gradient (written inside each sequence only) against the dense oracle per sequence."""
+    lens_q, lens_k = [40, 130, 1, 64], [100, 70, 5, 64]
+    Hq, Hk, D, B = 4, 2, 64, 4
+    mq, mk = max(lens_q), max(lens_k)
+    cu_q = np.concatenate([[0], np.cumsum(lens_q)]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)
+    Tq, Tk = int(cu_q[-1]), int(cu_k[-1])
+    q, k, v, do = (seeded((Tq, Hq, D), 1800, BF), seeded((Tk, Hk, D), 1801, BF), seeded((Tk, Hk, D), 1802, BF),
+                   seeded((Tq, Hq, D), 1803, BF))
+    fb = _bias((B, Hq, mq, mk), BF, 1804, holes=0.1)
+    qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
+    bd = fb.to(DEV)[..., :mk]
+    cq, ck = torch.from_numpy(cu_q).to(DEV), torch.from_numpy(cu_k).to(DEV)
+    out, lse = capi.fa_forward_packed(qd, kd, vd, cq, ck, mq, mk, is_causal=MASKS[mask], bias=bd)
+    dq, dk, dv, db = capi.fa_backward_packed(dod, qd, kd, vd, out, lse, cq, ck, mq, mk, is_causal=MASKS[mask], bias=bd,
+                                             want_dbias=True)
+    for b in range(B):
+        qs, ks = slice(cu_q[b], cu_q[b + 1]), slice(cu_k[b], cu_k[b + 1])
+        args = [t.transpose(0, 1)[None] for t in (q[qs], k[ks], v[ks])]
+        bias_b = fb[b:b + 1, :, :lens_q[b], :lens_k[b]].double().numpy()
+        okw = dict(is_causal=mask != "none", causal_top_left=mask == "tl", attn_bias=bias_b)
+        ro, rl = oracle.sdpa_oracle(*args, **okw)
+        assert np.abs(out[qs].float().cpu().numpy() - ro[0].transpose(1, 0, 2)).max() <= 2e-2
+        fin = np.isfinite(rl[0])
+        assert np.abs(lse[:, qs].cpu().numpy()[fin] - rl[0][fin]).max() <= 2e-3
+        want = oracle.sdpa_backward_oracle(*args, do[qs].transpose(0, 1)[None], return_dbias=True, **okw)
+        for name, g, w, sl in zip(("dq", "dk", "dv"), (dq, dk, dv), want, (qs, ks, ks)):
+            _close(name, g[sl].transpose(0, 1)[None], w, BF)
+        _close("dbias", db[b:b + 1, :, :lens_q[b], :lens_k[b]], want[3], BF)
+        assert float(db[b, :, lens_q[b]:].abs().max()) == 0.0 if lens_q[b] < mq else True
+
+
+# ---- cu_seqlens on the mem-efficient ops (attention.cpp:431-466, :627-658; test_memory_efficient_attention, :1729-1960) -
+def test_reference_efficient_ops_with_uniform_cu_seqlens():
+    """As the reference's test calls them: [B, S, H, D] inputs, cu_seqlens = arange(0, (B+1) S, S), an [Sq, Sk] mask
+    expanded to [B, H, Sq, Sk]; forward and backward.  The result is that of the same call without cu_seqlens (the
+    packed and the dense launch run the same arithmetic: bit-identical) and agrees with the oracle."""
+    B, H, Sq, Sk, D = 4, 4, 512, 1024, 128
+    q, k, v, do = _inputs(B, H, H, Sq, Sk, D, HF, 1900)
+    mask = seeded((Sq, Sk), 1901, HF, std=1.0)
+    qs, ks, vs, dos = (t.to(DEV).transpose(1, 2) for t in (q, k, v, do))
+    me = mask.to(DEV).expand(B, H, Sq, Sk)
+    cu_q = torch.arange(0, (B + 1) * Sq, Sq, dtype=torch.int32, device=DEV)
+    cu_k = torch.arange(0, (B + 1) * Sk, Sk, dtype=torch.int32, device=DEV)
+    out, lse, seed, offset, mq, mk = aten._efficient_attention_forward(qs, ks, vs, me, cu_q, cu_k, None, None, 0.0, 0, True)
+    assert out.shape == (B, Sq, H, D) and lse.shape == (H, B * Sq) and (mq, mk) == (Sq, Sk)
+    gq, gk, gv, gb = aten._efficient_attention_backward(dos, qs, ks, vs, me, out, cu_q, cu_k, mq, mk, lse, 0.0, seed,
+                                                        offset, 0, True)
+    out_d, lse_d, seed_d, offset_d, _, _ = aten._efficient_attention_forward(qs, ks, vs, me, None, None, None, None, 0.0,
+                                                                             0, True)
+    gd = aten._efficient_attention_backward(dos, qs, ks, vs, me, out_d, None, None, Sq, Sk, lse_d, 0.0, seed_d, offset_d,
+                                            0, True)
+    assert torch.equal(out, out_d) and torch.equal(lse.view(H, B, Sq).transpose(0, 1), lse_d)
+    for a, b in zip((gq, gk, gv, gb), gd):
+        assert torch.equal(a, b)
+    want = oracle.sdpa_backward_oracle(q, k, v, do, attn_bias=mask.double().numpy(), return_dbias=True)
+    for name, g, w in zip(("dq", "dk", "dv"), (gq, gk, gv), want):
+        _close(name, g.transpose(1, 2), w, HF)
+    _close("dbias", gb, want[3], HF)
+
+
+def test_efficient_ops_with_ragged_cu_seqlens():
+    """Sequences of different lengths laid out back to back in the rows of the flattened [B * S] view, a bias indexed
+    by sequence and position inside it, causal from the top-left; rows outside every sequence stay zero."""
+    B, H, S, D = 3, 2, 128, 64
+    lens_q, lens_k = [50, 128, 90], [128, 77, 100]
+    cu_q = np.concatenate([[0], np.cumsum(lens_q)]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)
+    q, k, v, do = _inputs(B, H, H, S, S, D, BF, 1950)                    # [B, H, S, D]; flattened rows = (b, s)
+    fb = _bias((B, H, S, S), BF, 1951, holes=0.05)
+    qs, ks, vs, dos = (t.to(DEV).transpose(1, 2).contiguous() for t in (q, k, v, do))
+    bd = fb.to(DEV)[..., :S]
+    cq, ck = torch.from_numpy(cu_q).to(DEV), torch.from_numpy(cu_k).to(DEV)
+    out, lse, seed, offset, mq, mk = aten._efficient_attention_forward(qs, ks, vs, bd, cq, ck, None, None, 0.0, 1, True)
+    gq, gk, gv, gb = aten._efficient_attention_backward(dos, qs, ks, vs, bd, out, cq, ck, mq, mk, lse, 0.0, seed, offset,
+                                                        1, True)
+    flat = lambda t: t.transpose(1, 2).reshape(B * S, H, D)               # CPU [B,H,S,D] -> packed rows
+    qf, kf, vf, dof = (flat(t) for t in (q, k, v, do))
+    of, gqf, gkf, gvf = (t.reshape(B * S, H, D) for t in (out, gq, gk, gv))
+    for b in range(B):
+        rq, rk = slice(cu_q[b], cu_q[b + 1]), slice(cu_k[b], cu_k[b + 1])
+        args = [t.transpose(0, 1)[None] for t in (qf[rq], kf[rk], vf[rk])]
+        okw = dict(is_causal=True, causal_top_left=True, attn_bias=fb[b:b + 1, :, :lens_q[b], :lens_k[b]].double().numpy())
+        ro, _ = oracle.sdpa_oracle(*args, **okw)
+        assert np.abs(of[rq].float().cpu().numpy() - ro[0].transpose(1, 0, 2)).max() <= 2e-2
+        want = oracle.sdpa_backward_oracle(*args, dof[rq].transpose(0, 1)[None], return_dbias=True, **okw)
+        for name, g, w, sl in zip(("dq", "dk", "dv"), (gqf, gkf, gvf), want, (rq, rk, rk)):
+            _close(name, g[sl].transpose(0, 1)[None], w, BF)
+        _close("dbias", gb[b:b + 1, :, :lens_q[b], :lens_k[b]], want[3], BF)
+    tq, tk = int(cu_q[-1]), int(cu_k[-1])
+    assert float(of[tq:].abs().max()) == 0.0 and float(gqf[tq:].abs().max()) == 0.0 and float(gkf[tk:].abs().max()) == 0.0
+    with pytest.raises(RuntimeError, match="cu_seqlens_q must have dtype int32"):
+        aten._efficient_attention_forward(qs, ks, vs, None, cq.long(), ck, None, None, 0.0, 0, True)
+    with pytest.raises(RuntimeError, match=r"cu_seqlens_k must have shape \(batch_size \+ 1\)"):
+        aten._efficient_attention_forward(qs, ks, vs, None, cq, ck[:3], None, None, 0.0, 0, True)
+    with pytest.raises(RuntimeError, match="given together"):
+        aten._efficient_attention_forward(qs, ks, vs, None, cq, None, None, None, 0.0, 0, True)

@@ -260,16 +260,19 @@ def fa_forward_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seql
                       cu_seqlens_k: torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, *, is_causal: bool = False,
                       scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
                       dropout_p: float = 0.0, philox_seed: int = 0, philox_offset: int = 0,
-                      rng_out: Optional[torch.Tensor] = None, seqused_k: Optional[torch.Tensor] = None
-                      ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """q [Tq, Hq, D], k/v [Tk, Hk, D], cu_seqlens int32 [B+1] on the device -> out [Tq, Hq, D], lse [Hq, Tq]."""
+                      rng_out: Optional[torch.Tensor] = None, seqused_k: Optional[torch.Tensor] = None,
+                      bias: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """q [Tq, Hq, D], k/v [Tk, Hk, D], cu_seqlens int32 [B+1] on the device -> out [Tq, Hq, D], lse [Hq, Tq].
+    `bias`: [B, Hq, max_seqlen_q, max_seqlen_k] (or anything expanding to it), indexed by sequence and by the row / key
+    position inside the sequence."""
     Tq, Hq, D = q.shape
     out = torch.empty((Tq, Hq, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((Hq, Tq), dtype=torch.float32, device=q.device)
     p = make_params(q, k, v, out, lse, cu_seqlens_q=cu_seqlens_q, cu_seqlens_k=cu_seqlens_k,
                     max_seqlen_q=max_seqlen_q, max_seqlen_k=max_seqlen_k, scale=scale, is_causal=is_causal,
                     kernel=kernel, num_splits=num_splits, dropout_p=dropout_p, philox_seed=philox_seed,
-                    philox_offset=philox_offset, rng_out=rng_out, seqused_k=seqused_k)
+                    philox_offset=philox_offset, rng_out=rng_out, seqused_k=seqused_k,
+                    bias=None if bias is None else bias.expand(cu_seqlens_q.numel() - 1, Hq, max_seqlen_q, max_seqlen_k))
     launch(p, q.device)
     return out, lse
 
@@ -331,8 +334,10 @@ def fa_backward_dense(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: t
 
 def fa_backward_packed(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, max_seqlen_k: int, *,
                        is_causal: bool = False, scale: Optional[float] = None, dropout_p: float = 0.0,
-                       rng: Optional[torch.Tensor] = None):
-    """Packed: dout, q, out [Tq, Hq, D], k, v [Tk, Hk, D], lse [Hq, Tq] -> (dq, dk, dv) with the inputs' shapes."""
+                       rng: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None, want_dbias: bool = False):
+    """Packed: dout, q, out [Tq, Hq, D], k, v [Tk, Hk, D], lse [Hq, Tq] -> (dq, dk, dv) with the inputs' shapes (and
+    the gradient of the bias [B, Hq, max_seqlen_q, max_seqlen_k] with `want_dbias`; only the part inside each sequence
+    is written)."""
     Tq, Hq, D = q.shape
     dq, dk, dv = torch.empty_like(q, memory_format=torch.contiguous_format), torch.empty_like(
         k, memory_format=torch.contiguous_format), torch.empty_like(v, memory_format=torch.contiguous_format)
@@ -349,7 +354,20 @@ def fa_backward_packed(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_
     p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
     p.dtype, p.is_causal, p.reserved = _dtype_code(q.dtype), int(is_causal), 0
     _set_dropout(p, dropout_p, rng)
+    dbias = None
+    if bias is not None:
+        B = cu_seqlens_q.numel() - 1
+        bias = bias.expand(B, Hq, max_seqlen_q, max_seqlen_k)
+        p.bias = bias.data_ptr()
+        p.bias_stride_b, p.bias_stride_h, p.bias_stride_q = bias.stride(0), bias.stride(1), bias.stride(2)
+        if want_dbias:
+            dbias = torch.zeros((B, Hq, max_seqlen_q, (max_seqlen_k + 7) // 8 * 8), dtype=q.dtype,
+                                device=q.device)[..., :max_seqlen_k]
+            p.dbias = dbias.data_ptr()
+            p.dbias_stride_b, p.dbias_stride_h, p.dbias_stride_q = dbias.stride(0), dbias.stride(1), dbias.stride(2)
     _launch_bwd(p, q.device)
+    if want_dbias:
+        return dq, dk, dv, dbias
     return dq, dk, dv
 
 

@@ -29,6 +29,7 @@
 
 #include <atomic>
 #include <cmath>
+#include <limits>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -451,6 +452,20 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> scaled_dot_product_flash_attentio
 }
 
 namespace {
+// cu_seqlens of the mem-efficient ops: int32 [batch + 1] on the device (attention.cpp:433-443,455-465 and their messages)
+void check_efficient_cu_seqlens(const at::Tensor& cu_q, const at::Tensor& cu_k, int64_t batch) {
+  TORCH_CHECK(cu_q.scalar_type() == at::kInt, "cu_seqlens_q must have dtype int32");
+  TORCH_CHECK(cu_q.is_cuda(), "cu_seqlens_q must be on HIP device");
+  TORCH_CHECK(cu_q.dim() == 1 && cu_q.size(0) == batch + 1, "cu_seqlens_q must have shape (batch_size + 1)");
+  TORCH_CHECK(cu_k.scalar_type() == at::kInt, "cu_seqlens_k must have dtype int32");
+  TORCH_CHECK(cu_k.is_cuda(), "cu_seqlens_k must be on HIP device");
+  TORCH_CHECK(cu_k.dim() == 1 && cu_k.size(0) == batch + 1, "cu_seqlens_k must have shape (batch_size + 1)");
+  TORCH_CHECK(cu_q.is_contiguous() && cu_k.is_contiguous(), "cu_seqlens must be contiguous");
+}
+// A [B, S, H, D] tensor whose rows can be addressed by their index in the flattened [B * S] view (one copy if not)
+at::Tensor flattenable(const at::Tensor& t) {
+  return (t.size(0) <= 1 || t.stride(0) == t.size(1) * t.stride(1)) ? t : t.contiguous();
+}
 // The bias as a [B, H, Sq, Sk] view (stride 0 where broadcast) that meets the kernels' alignment rule: groups of 4
 // keys 8-byte aligned.  If the caller's does not, one copy of the un-broadcast bias with rows padded to a multiple of
 // 8 columns is made (the reference always copies: cnnl_contiguous, attention.cpp:660-663).
@@ -496,8 +511,10 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
               "Number of heads in key/value must divide number of heads in query");
   TORCH_CHECK(query.size(3) == key.size(3), "query and key must have the same head dimension");
   TORCH_CHECK(value.size(3) == query.size(3), "this build needs value.size(-1) == query.size(-1)");
-  TORCH_CHECK(!(cu_seqlens_q.has_value() && cu_seqlens_q->defined()) && !(cu_seqlens_k.has_value() && cu_seqlens_k->defined()),
-              "efficient attention forward: cu_seqlens are not supported by this build (use _flash_attention_forward)");
+  // cu_seqlens (attention.cpp:431-466): offsets of the sequences in the rows of the [B * S, H, D] view of the inputs
+  const bool packed = cu_seqlens_q.has_value() && cu_seqlens_q->defined();
+  TORCH_CHECK(packed == (cu_seqlens_k.has_value() && cu_seqlens_k->defined()), "cu_seqlens_q and cu_seqlens_k must be given together");
+  if (packed) check_efficient_cu_seqlens(*cu_seqlens_q, *cu_seqlens_k, query.size(0));
   TORCH_CHECK(!window_size.has_value() || *window_size <= 0, "efficient attention forward: sliding window is not supported");
   TORCH_CHECK(dropout_p >= 0.0 && dropout_p < 1.0, "efficient attention forward: dropout_p must be in [0, 1), got ", dropout_p);
   TORCH_CHECK(custom_mask_type >= 0 && custom_mask_type <= 2, "custom_mask_type must be 0, 1 or 2");
@@ -518,9 +535,15 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
 
   const c10::OptionalDeviceGuard guard(query.device());
   const float softmax_scale = resolve_scale(query, scale);
-  const at::Tensor q = aligned_or_copy(query), k = aligned_or_copy(key), v = aligned_or_copy(value);
-  at::Tensor output = at::empty({B, Sq, Hq, D}, q.options());
-  at::Tensor lse = at::empty({B, Hq, Sq}, q.options().dtype(at::kFloat));
+  at::Tensor q = aligned_or_copy(query), k = aligned_or_copy(key), v = aligned_or_copy(value);
+  if (packed) {  // rows are addressed by their index in the flattened [B * S] view
+    q = flattenable(q); k = flattenable(k); v = flattenable(v);
+  }
+  // packed: rows outside every sequence are never written; logsumexp is the kernel's raw [H, B * Sq] buffer, as the
+  // reference returns it (FlashAttention_internal.cpp:599-606,689)
+  at::Tensor output = packed ? at::zeros({B, Sq, Hq, D}, q.options()) : at::empty({B, Sq, Hq, D}, q.options());
+  at::Tensor lse = packed ? at::full({Hq, B * Sq}, std::numeric_limits<float>::infinity(), q.options().dtype(at::kFloat))
+                          : at::empty({B, Hq, Sq}, q.options().dtype(at::kFloat));
 
   at::Tensor bias_e;
   if (bias.has_value() && bias->defined()) bias_e = bias_for_kernels(*bias, dt, B, Hq, Sq, Sk);
@@ -532,7 +555,13 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   fill_strides(k, false, p.k_stride_b, p.k_stride_s, p.k_stride_h);
   fill_strides(v, false, p.v_stride_b, p.v_stride_s, p.v_stride_h);
   fill_strides(output, false, p.o_stride_b, p.o_stride_s, p.o_stride_h);
-  p.lse_stride_b = lse.stride(0); p.lse_stride_h = lse.stride(1); p.lse_stride_s = lse.stride(2);
+  if (packed) {
+    p.cu_seqlens_q = cu_seqlens_q->data_ptr<int32_t>();
+    p.cu_seqlens_k = cu_seqlens_k->data_ptr<int32_t>();
+    p.lse_stride_b = 0; p.lse_stride_h = lse.stride(0); p.lse_stride_s = lse.stride(1);
+  } else {
+    p.lse_stride_b = lse.stride(0); p.lse_stride_h = lse.stride(1); p.lse_stride_s = lse.stride(2);
+  }
   p.batch = static_cast<int32_t>(B);
   p.heads_q = static_cast<int32_t>(Hq);
   p.heads_k = static_cast<int32_t>(Hk);
@@ -571,7 +600,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
     TORCH_CHECK(rc == FA_OK, "fa_fwd_launch failed: ", fa_fwd_error_string(rc), " (rc=", rc, ")");
     g_launches.fetch_add(1, std::memory_order_relaxed);
   }
-  if (!compute_log_sumexp) lse = at::empty({B, Hq, 0}, q.options().dtype(at::kFloat));
+  if (!compute_log_sumexp) lse = packed ? at::empty({Hq, 0}, q.options().dtype(at::kFloat)) : at::empty({B, Hq, 0}, q.options().dtype(at::kFloat));
   return std::make_tuple(output, lse, seed_t, offset_t, c10::SymInt(Sq), c10::SymInt(Sk));
 }
 
@@ -620,8 +649,9 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> efficient_attention_b
   TORCH_CHECK(value.size(3) == grad_out_.size(3) && value.size(3) == query.size(3),
               "this build needs value.size(-1) == query.size(-1) == grad_out.size(-1)");
   TORCH_CHECK(out.sizes() == grad_out_.sizes(), "out must have the shape of grad_out");
-  TORCH_CHECK(!(cu_seqlens_q.has_value() && cu_seqlens_q->defined()) && !(cu_seqlens_k.has_value() && cu_seqlens_k->defined()),
-              "efficient attention backward: cu_seqlens are not supported by this build (use _flash_attention_backward)");
+  const bool packed = cu_seqlens_q.has_value() && cu_seqlens_q->defined();
+  TORCH_CHECK(packed == (cu_seqlens_k.has_value() && cu_seqlens_k->defined()), "cu_seqlens_q and cu_seqlens_k must be given together");
+  if (packed) check_efficient_cu_seqlens(*cu_seqlens_q, *cu_seqlens_k, query.size(0));
   TORCH_CHECK(!window_size.has_value() || *window_size <= 0, "efficient attention backward: sliding window is not supported");
   TORCH_CHECK(dropout_p >= 0.0 && dropout_p < 1.0, "efficient attention backward: dropout_p must be in [0, 1), got ", dropout_p);
   if (dropout_p > 0.0)
@@ -650,16 +680,29 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> efficient_attention_b
   TORCH_CHECK(D <= 256, "FlashAttention backward only supports head dimension at most 256");
   TORCH_CHECK(D % 8 == 0, "head dimension must be a multiple of 8");
   TORCH_CHECK(Sq <= INT32_MAX && Sk <= INT32_MAX && B <= INT32_MAX, "sequence length too large");
-  TORCH_CHECK(logsumexp.dim() == 3 && logsumexp.size(0) == B && logsumexp.size(1) == Hq && logsumexp.size(2) >= Sq,
-              "logsumexp must have shape (batch_size, num_heads, seqlen_q): call the forward with compute_log_sumexp");
+  if (packed) {
+    TORCH_CHECK(logsumexp.dim() == 2 && logsumexp.size(0) == Hq && logsumexp.size(1) == B * Sq,
+                "logsumexp must have shape (num_heads, batch_size * seqlen_q): call the forward with compute_log_sumexp");
+  } else {
+    TORCH_CHECK(logsumexp.dim() == 3 && logsumexp.size(0) == B && logsumexp.size(1) == Hq && logsumexp.size(2) >= Sq,
+                "logsumexp must have shape (batch_size, num_heads, seqlen_q): call the forward with compute_log_sumexp");
+  }
 
   const c10::OptionalDeviceGuard guard(query.device());
   const float softmax_scale = resolve_scale(query, scale);
   auto fix = [](const at::Tensor& t) { return t.stride(-1) == 1 ? aligned_or_copy(t) : t.contiguous(); };
-  const at::Tensor q = aligned_or_copy(query), k = aligned_or_copy(key), v = aligned_or_copy(value);
-  const at::Tensor dout = fix(grad_out_), o = fix(out);  // the reference makes both contiguous (attention.cpp:646-650)
+  at::Tensor q = aligned_or_copy(query), k = aligned_or_copy(key), v = aligned_or_copy(value);
+  at::Tensor dout = fix(grad_out_), o = fix(out);  // the reference makes both contiguous (attention.cpp:646-650)
+  if (packed) {
+    q = flattenable(q); k = flattenable(k); v = flattenable(v); dout = flattenable(dout); o = flattenable(o);
+  }
   at::Tensor dq, dk, dv;
-  if (shared_storage_dqdkdv) {  // one [B, S, 3, H, D] allocation, the three gradients as its slices
+  if (packed) {  // rows outside every sequence get no gradient
+    TORCH_CHECK(!shared_storage_dqdkdv, "shared_storage_dqdkdv is not supported together with cu_seqlens");
+    dq = at::zeros({B, Sq, Hq, D}, q.options());
+    dk = at::zeros({B, Sk, Hk, D}, q.options());
+    dv = at::zeros({B, Sk, Hk, D}, q.options());
+  } else if (shared_storage_dqdkdv) {  // one [B, S, 3, H, D] allocation, the three gradients as its slices
     TORCH_CHECK(Sq == Sk && Hq == Hk, "shared_storage_dqdkdv needs query and key of the same shape");
     at::Tensor chunk = at::empty({B, Sq, 3, Hq, D}, q.options());
     dq = chunk.select(2, 0); dk = chunk.select(2, 1); dv = chunk.select(2, 2);
@@ -672,8 +715,10 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> efficient_attention_b
   at::Tensor bias_e, dbias;
   if (has_bias) bias_e = bias_for_kernels(*bias, dt, B, Hq, Sq, Sk);
   const bool want_dbias = has_bias && bias_requires_grad;
-  if (want_dbias)  // rows padded to a multiple of 8 columns: every row start 16-byte aligned
-    dbias = at::empty({B, Hq, Sq, (Sk + 7) / 8 * 8}, q.options()).narrow(3, 0, Sk);
+  if (want_dbias)  // rows padded to a multiple of 8 columns: every row start 16-byte aligned; packed: only the part
+                   // inside each sequence is written
+    dbias = (packed ? at::zeros({B, Hq, Sq, (Sk + 7) / 8 * 8}, q.options())
+                    : at::empty({B, Hq, Sq, (Sk + 7) / 8 * 8}, q.options())).narrow(3, 0, Sk);
 
   fa_bwd_params p{};
   p.q = q.data_ptr(); p.k = k.data_ptr(); p.v = v.data_ptr(); p.out = o.data_ptr(); p.dout = dout.data_ptr();
@@ -687,7 +732,14 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> efficient_attention_b
   fill_strides(dq, false, p.dq_stride_b, p.dq_stride_s, p.dq_stride_h);
   fill_strides(dk, false, p.dk_stride_b, p.dk_stride_s, p.dk_stride_h);
   fill_strides(dv, false, p.dv_stride_b, p.dv_stride_s, p.dv_stride_h);
-  p.lse_stride_b = logsumexp.stride(0); p.lse_stride_h = logsumexp.stride(1); p.lse_stride_s = logsumexp.stride(2);
+  if (packed) {
+    p.cu_seqlens_q = cu_seqlens_q->data_ptr<int32_t>();
+    p.cu_seqlens_k = cu_seqlens_k->data_ptr<int32_t>();
+    p.total_q = B * Sq;
+    p.lse_stride_b = 0; p.lse_stride_h = logsumexp.stride(0); p.lse_stride_s = logsumexp.stride(1);
+  } else {
+    p.lse_stride_b = logsumexp.stride(0); p.lse_stride_h = logsumexp.stride(1); p.lse_stride_s = logsumexp.stride(2);
+  }
   p.batch = static_cast<int32_t>(B);
   p.heads_q = static_cast<int32_t>(Hq);
   p.heads_k = static_cast<int32_t>(Hk);

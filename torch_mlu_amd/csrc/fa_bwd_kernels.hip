@@ -893,7 +893,6 @@ int bwd_validate(const fa_bwd_params* p) {
     if (((uintptr_t)p->bias & 7) || p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_q < 0 ||
         ((p->bias_stride_b | p->bias_stride_h | p->bias_stride_q) & 3))
       return FA_ERR_BAD_ARG;
-    if (p->cu_seqlens_q) return FA_ERR_UNSUPPORTED;
   }
   if (p->dbias) {  // an output: aligned like the bias and not broadcast
     if (((uintptr_t)p->dbias & 7) || ((p->dbias_stride_b | p->dbias_stride_h | p->dbias_stride_q) & 3)) return FA_ERR_BAD_ARG;

@@ -834,7 +834,7 @@ int validate(const fa_fwd_params* p) {
     if (((uintptr_t)p->bias & 7) || p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_q < 0 ||
         ((p->bias_stride_b | p->bias_stride_h | p->bias_stride_q) & 3))
       return FA_ERR_BAD_ARG;
-    if (p->cu_seqlens_q || p->kernel == FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
+    if (p->kernel == FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
   }
   if (p->kernel == FA_KERNEL_SPLITKV) {
     if (p->seqlen_q != 1 || p->heads_q / p->heads_k > 16) return FA_ERR_UNSUPPORTED;
