@@ -30,12 +30,12 @@ PEAK_HBM_GBS = 8000.0
 # their commands are recorded under profiles/.  Counters cannot be read from inside a timed run, so these are the
 # recorded values (None: not profiled).
 TRAFFIC_BYTES = {
-    "cfg2": int((515.9 + 130.0) * 2 ** 20),
+    "cfg2": int((522.2 + 130.0) * 2 ** 20),
     "cfg5": int(2.0021 * 2 ** 30 + 4.25 * 2 ** 20),
-    "cfg2_bwd": int((1746.1 + 388.1) * 2 ** 20),  # the three launches of one backward together
-    "cfg2_mask": int(3.68 * 2 ** 30 + 223.6 * 2 ** 20),
-    "cfg2_drop": int((512.8 + 130.0) * 2 ** 20),
-    "cfg2_mask_bwd": int((3.44 + 4.43 + 2.40) * 2 ** 30 + (151.1 + 133.5 + 130.7) * 2 ** 20),  # three launches
+    "cfg2_bwd": int((1814.5 + 388.1) * 2 ** 20),  # the three launches of one backward together
+    "cfg2_mask": int(3.70 * 2 ** 30 + 223.3 * 2 ** 20),
+    "cfg2_drop": int((518.5 + 130.0) * 2 ** 20),
+    "cfg2_mask_bwd": int((3.23 + 4.42 + 2.42) * 2 ** 30 + (151.9 + 133.4 + 130.5) * 2 ** 20),  # three launches
 }
 
 
