@@ -48,14 +48,18 @@ def make_workload(name, dev):
     """-> dict(call=callable doing one step, flops, bytes_kv, desc, check=callable returning (out_err, lse_err))."""
     bf, hf = torch.bfloat16, torch.float16
     aten = torch.ops.aten
-    if name in ("cfg2", "cfg3"):
-        if name == "cfg2":
+    if name in ("cfg2", "cfg3", "cfg2_bshd"):
+        if name != "cfg3":
             B, Hq, Hk, S, D, seed = 4, 32, 32, 4096, 128, 1
         else:
             B, Hq, Hk, S, D, seed = 8, 32, 8, 2048, 128, 2
         q = seeded((B, Hq, S, D), seed, bf).to(dev)
         k = seeded((B, Hk, S, D), seed + 1, bf).to(dev)
         v = seeded((B, Hk, S, D), seed + 2, bf).to(dev)
+        if name == "cfg2_bshd":
+            # the same values seen through [B, H, S, D] views of [B, S, H, D] memory (what a projection layer hands
+            # over): the strides go down to the kernel, nothing is copied
+            q, k, v = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
 
         def call():
             return aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False)
@@ -65,7 +69,8 @@ def make_workload(name, dev):
             return _check_heads(q, k, v, out, lse, True, [(0, 0), (B - 1, Hq - 1)])
 
         return dict(call=call, check=check, flops=4 * B * Hq * S * S * D / 2, bytes_kv=2 * B * Hk * S * D * 2,
-                    desc=f"causal prefill bf16 B={B} Hq={Hq} Hkv={Hk} S={S} D={D}", dtype="bf16", bound="mfma",
+                    desc=f"causal prefill bf16 B={B} Hq={Hq} Hkv={Hk} S={S} D={D}"
+                         + (" on [B,S,H,D]-backed views" if name == "cfg2_bshd" else ""), dtype="bf16", bound="mfma",
                     kernel="fa_tile_kernel")
     if name == "cfg2_bwd":
         # the backward of the headline workload (same shape and inputs, plus a seeded dOut); FLOPs are the five matrix
@@ -300,7 +305,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "copy1g"])
+    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "copy1g"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -345,7 +350,7 @@ def main():
     main_r = run(args.config, args.steps, args.warmup)
     extras = []
     if not args.no_extras:
-        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd"):
+        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd"):
             if name != args.config:
                 extras.append(run(name, args.steps, args.warmup))
 

@@ -32,8 +32,10 @@ def _aligned_bias(shape, dtype, seed, std=2.0):
 @pytest.mark.parametrize("dtype", [BF, HF])
 @pytest.mark.parametrize("D", [64, 128, 256])
 def test_bias_shapes_through_c_abi(dtype, D):
+    # seqlen_k a multiple of 8 takes the variant that stages the bias through LDS, the others read it directly
     cases = [(2, 4, 2, 130, 130), (1, 2, 2, 64, 64), (2, 2, 1, 70, 333), (1, 4, 4, 257, 65), (3, 2, 2, 1, 500),
-             (1, 2, 2, 200, 3)]
+             (1, 2, 2, 200, 3), (2, 4, 2, 130, 136), (1, 2, 2, 300, 200), (2, 2, 1, 70, 328), (1, 4, 4, 257, 72),
+             (1, 2, 2, 40, 8)]
     for i, (B, Hq, Hk, Sq, Sk) in enumerate(cases):
         q, k, v = _qkv(B, Hq, Hk, Sq, Sk, D, dtype, seed=10 * i)
         for bshape in ((B, Hq, Sq, Sk), (1, Hq, Sq, Sk), (B, 1, Sq, Sk), (1, 1, 1, Sk)):
@@ -44,6 +46,24 @@ def test_bias_shapes_through_c_abi(dtype, D):
                                             causal_top_left=causal == capi.FA_MASK_CAUSAL_TOP_LEFT)
                 out_close(out.float().cpu().numpy(), ro, dtype)
                 lse_close(lse.cpu().numpy(), rl, tol=2e-3 if dtype == BF else LSE_TOL)
+
+
+def test_staged_and_direct_bias_reads_agree_bitwise():
+    """The same bias values at a 16-byte aligned address (fetched by DMA through LDS, one tile ahead) and at an address
+    that is only 8-byte aligned (read directly) go through the same arithmetic: identical bits out."""
+    for (B, Hq, Hk, Sq, Sk, D, causal) in ((2, 4, 2, 333, 456, 128, 0), (1, 2, 2, 200, 1000, 64, 2),
+                                           (1, 3, 3, 129, 192, 128, 1)):
+        q, k, v = (t.to(DEV) for t in _qkv(B, Hq, Hk, Sq, Sk, D, BF, seed=Sk))
+        vals = seeded((B, Hq, Sq, Sk), 5, BF, std=2.0).to(DEV)
+        store = torch.zeros(B, Hq, Sq, Sk + 8, dtype=BF, device=DEV)
+        aligned, shifted = store[..., :Sk], store[..., 4:Sk + 4]
+        assert aligned.data_ptr() % 16 == 0 and shifted.data_ptr() % 16 == 8
+        aligned.copy_(vals)
+        o1, l1 = capi.fa_forward_dense(q, k, v, bias=aligned, is_causal=causal)
+        store.zero_()
+        shifted.copy_(vals)
+        o2, l2 = capi.fa_forward_dense(q, k, v, bias=shifted, is_causal=causal)
+        assert torch.equal(o1, o2) and torch.equal(l1, l2)
 
 
 def test_top_left_causal_without_bias_and_splitkv_routing():

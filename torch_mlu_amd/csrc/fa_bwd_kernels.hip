@@ -114,7 +114,9 @@ struct TileIO {
 // BIAS: the additive bias of this lane's query row is read straight from global memory into the score layout (8 bytes
 // = 4 consecutive keys per load, as in the forward); dS of the tile, already packed for the dQ product, is also what
 // the gradient of the bias is, and is stored from here (tiles the causal mask skips are stored as zeros).
-template <typename T, int DP, bool DROP, bool BIAS>
+// BIAS = 2: the bias tile comes through LDS instead, fetched by DMA most of a tile ahead in 16-byte pieces (rows must be
+// 16-byte aligned and seqlen_k a multiple of 8): the direct loads are issued only 32 MFMAs before their use.
+template <typename T, int DP, bool DROP, int BIAS>
 __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const BArgs a) {
   using IO = TileIO<T, DP>;
   constexpr int CPR = IO::CPR, ROWB = IO::ROWB, TILE = IO::TILE, NI = IO::NI, RPI = IO::RPI, KS = IO::KS, MB = IO::MB;
@@ -291,6 +293,31 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
     brow = a.bias + (int64_t)b * a.bias_sb + (int64_t)h * a.bias_sh + r * a.bias_sq + 8 * g;
     if (a.dbias && row < Lq) dbrow = a.dbias + (int64_t)b * a.dbias_sb + (int64_t)h * a.dbias_sh + r * a.dbias_sq + 8 * g;
   }
+  // BIAS == 2: this wavefront's 32 rows x 64 keys of the bias tile (4 KiB) go through a private LDS area.  DMA
+  // instruction i brings rows 8 i .. 8 i + 7; lane l fetches 16 bytes (8 keys): row 8 i + l / 8, key chunk
+  // (l % 8) ^ (l / 8), so that row r keeps chunk ch at r * 128 + ((ch ^ (r & 7)) * 16).
+  const unsigned char* bbase = nullptr;  // wavefront-uniform: this block's first bias row
+  unsigned boff[BIAS == 2 ? 4 : 1];      // per-lane byte offsets of the four DMA instructions
+  const int bchunk = (lane & 7) ^ (lane >> 3);
+  const unsigned blds = lds0 - wave * 1024 + 4 * TILE + wave * 4096;
+  int baddr = 0;  // per-lane LDS read offset of key chunk 0; chunk ch is at baddr ^ (ch * 16)
+  if constexpr (BIAS == 2) {
+    bbase = a.bias + (int64_t)b * a.bias_sb + (int64_t)h * a.bias_sh + (int64_t)m0 * a.bias_sq;
+    const int rmax = Lq - 1 - m0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      boff[i] = (unsigned)min(32 * wave + 8 * i + (lane >> 3), rmax) * (unsigned)a.bias_sq + bchunk * 16;
+    baddr = 4 * TILE + wave * 4096 + c32 * 128 + (c32 & 7) * 16 + 8 * g;
+  }
+  // chunks that start at or beyond Lk (last, partial tile) are pointed at the tile's chunk 0: their scores are masked
+  auto issue_bias = [&](int j) {
+    const unsigned char* bt = bbase + (int64_t)j * (BN * 2);
+    const unsigned adj = (j * BN + bchunk * 8 >= Lk) ? bchunk * 16 : 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16s(bt, boff[i] - adj, blds + i * 1024);
+  };
+  if constexpr (BIAS == 2)
+    if (ntiles > 0) issue_bias(0);
   // chunk t of tile j holds dS of keys j BN + 32 (t >> 1) + 16 (t & 1) + 4 g + {0..3, 8..11} of this lane's row
   auto store_dbias = [&](int j, int t, u32x4 w) {
     if (!dbrow) return;
@@ -328,7 +355,7 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
     // one, masked below anyway), issued now and consumed after the S / dP MFMAs
     const bool full_tile = j * BN + BN <= Lk;
     u32x2 braw[BIAS ? 8 : 1];
-    if constexpr (BIAS) {
+    if constexpr (BIAS == 1) {
       if (full_tile) {
         const unsigned char* bt = brow + (int64_t)j * (BN * 2);
 #pragma unroll
@@ -389,6 +416,10 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
     s16x8 dsb[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
+      if constexpr (BIAS == 2) {  // the two 4-key groups of chunk t
+        braw[4 * (t >> 1) + 2 * (t & 1)] = *(const u32x2*)(smem + (baddr ^ ((4 * (t >> 1) + 2 * (t & 1)) * 16)));
+        braw[4 * (t >> 1) + 2 * (t & 1) + 1] = *(const u32x2*)(smem + (baddr ^ ((4 * (t >> 1) + 2 * (t & 1) + 1) * 16)));
+      }
       u32x4 w;
 #pragma unroll
       for (int e2 = 0; e2 < 4; ++e2) {
@@ -417,6 +448,11 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
       }
       dsb[t] = __builtin_bit_cast(s16x8, w);
       if constexpr (BIAS) store_dbias(j, t, w);
+    }
+    if constexpr (BIAS == 2) {
+      // the next tile's bias may overwrite this one now: every dS depends on the values that were read
+      asm volatile("" : : "v"(dsb[0]), "v"(dsb[1]), "v"(dsb[2]), "v"(dsb[3]) : "memory");
+      if (j + 1 < ntiles) issue_bias(j + 1);
     }
     // dQ^T += K^T dS^T; the transposed K fragments of chunk t + 1 are fetched while chunk t's MFMAs run
     {
@@ -937,7 +973,15 @@ int bwd_launch(const BArgs& a, hipStream_t st) {
   constexpr int lds_dq = 4 * 64 * DP * 2;
   constexpr int lds_dkv = 4 * 64 * DP * 2 + 4 * 256;
   constexpr bool split = DP > 64;  // head_dim 128: dK and dV as two launches
-  constexpr auto kq = fa_bwd_dq_kernel<T, DP, DROP, BIAS>;
+  constexpr auto kq = fa_bwd_dq_kernel<T, DP, DROP, BIAS ? 1 : 0>;
+  // the dQ kernel can fetch 16-byte pieces of bias rows by DMA when every row starts 16-byte aligned and no piece
+  // straddles the end of a row
+  constexpr bool can_stage = BIAS && !DROP && DP <= 128;
+  constexpr auto kq2 = fa_bwd_dq_kernel<T, DP, DROP, can_stage ? 2 : (BIAS ? 1 : 0)>;
+  constexpr int lds_dq2 = lds_dq + 4 * 4096;
+  const bool staged = can_stage && !a.cu_q && a.seqlen_k % 8 == 0 && (uintptr_t)a.bias % 16 == 0 && a.bias_sb % 16 == 0 &&
+                      a.bias_sh % 16 == 0 && a.bias_sq % 16 == 0;
+  if (staged && !ensure_dynamic_lds<kq2>(lds_dq2)) return FA_ERR_LAUNCH;
   constexpr auto kkv = fa_bwd_dkv_kernel<T, DP, split ? kDK : (kDK | kDV), DROP, BIAS>;
   constexpr auto kv2 = fa_bwd_dkv_kernel<T, DP, kDV, DROP, BIAS>;
   if (!ensure_dynamic_lds<kq>(lds_dq) || !ensure_dynamic_lds<kkv>(lds_dkv) || (split && !ensure_dynamic_lds<kv2>(lds_dkv)))
@@ -946,7 +990,8 @@ int bwd_launch(const BArgs& a, hipStream_t st) {
   const int64_t gk = (int64_t)a.batch * a.heads_k * a.n_kslot;
   if (gq > 0x7fffffffLL || gk > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
   if (gq > 0) {
-    hipLaunchKernelGGL(kq, dim3((unsigned)gq), dim3(256), lds_dq, st, a);
+    if (staged) hipLaunchKernelGGL(kq2, dim3((unsigned)gq), dim3(256), lds_dq2, st, a);
+    else hipLaunchKernelGGL(kq, dim3((unsigned)gq), dim3(256), lds_dq, st, a);
     if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
   }
   if (gk > 0) {

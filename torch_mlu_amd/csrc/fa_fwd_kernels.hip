@@ -93,13 +93,16 @@ __device__ __forceinline__ int swzV(int row) {
 // depend on which maximum was in use.
 constexpr float kLazyLog2 = 8.0f;
 
-// BIAS: an additive bias tile is read straight from global memory into the score layout (one lane = one query row,
-// groups of 4 consecutive keys = 8 bytes) and the softmax then runs on scores already in the log2 domain.
+// BIAS = 1: an additive bias tile is read straight from global memory into the score layout (one lane = one query
+// row, groups of 4 consecutive keys = 8 bytes) and the softmax then runs on scores already in the log2 domain.
+// BIAS = 2: the same, but the tile is fetched by DMA into LDS one tile ahead (16-byte pieces, so rows must be 16-byte
+// aligned and seqlen_k a multiple of 8) and read from there: the loads of mode 1 are issued only 16 MFMAs before
+// their use, which leaves most of an L2 miss exposed.
 // DROP: dropout on the probabilities.  The row sums (and LSE) are those of the undropped probabilities; dropped
 // entries are zeroed in the P operand of the PV product and 1 / (1 - p) is folded into the final normalisation.
 // DMASK (with DROP): also write the keep-mask out for tests; a variant of its own because the extra stores cost
 // registers (30 spilled at head_dim 128) that the plain dropout kernel does not have to pay.
-template <typename T, int DP, int MINB, bool BIAS, bool DROP = false, bool DMASK = false>
+template <typename T, int DP, int MINB, int BIAS, bool DROP = false, bool DMASK = false>
 __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   constexpr int CPR = DP / 8;          // 16-byte chunks per row
   constexpr int ROWB = DP * 2;         // bytes per LDS row
@@ -279,8 +282,33 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   unsigned char* drow = nullptr;  // this lane's row of the debug mask
   if constexpr (DROP && DMASK)
     if (a.dmask) drow = a.dmask + (((int64_t)b * a.heads_q + h) * a.seqlen_q + min(row, Lq - 1)) * (int64_t)a.seqlen_k * 2;
-  if constexpr (BIAS)
+  if constexpr (BIAS == 1)
     brow = a.bias + (int64_t)b * a.bias_sb + (int64_t)h * a.bias_sh + (int64_t)min(row, Lq - 1) * a.bias_sq + 8 * g;
+  // BIAS == 2: this wavefront's 32 rows x 64 keys of the bias tile (4 KiB) go through a private LDS area by DMA, one
+  // tile ahead.  DMA instruction i brings rows 8 i .. 8 i + 7; lane l fetches 16 bytes (8 keys): row 8 i + l / 8, key
+  // chunk (l % 8) ^ (l / 8), so that row r keeps chunk ch at r * 128 + ((ch ^ (r & 7)) * 16).
+  const unsigned char* bbase = nullptr;  // wavefront-uniform: this block's first bias row
+  unsigned boff[BIAS == 2 ? 4 : 1];      // per-lane byte offsets of the four DMA instructions
+  const int bchunk = (lane & 7) ^ (lane >> 3);
+  const unsigned blds = lds0 - wave * 1024 + 4 * TILE + wave * 4096;  // LDS byte address of this wavefront's area
+  int baddr = 0;  // per-lane LDS read offset of key chunk 0; chunk ch is at baddr ^ (ch * 16)
+  if constexpr (BIAS == 2) {
+    bbase = a.bias + (int64_t)b * a.bias_sb + (int64_t)h * a.bias_sh + (int64_t)m0 * a.bias_sq;
+    const int rmax = Lq - 1 - m0;  // >= 0
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      boff[i] = (unsigned)min(32 * wave + 8 * i + (lane >> 3), rmax) * (unsigned)a.bias_sq + bchunk * 16;
+    baddr = 4 * TILE + wave * 4096 + c32 * 128 + (c32 & 7) * 16 + 8 * g;
+  }
+  // chunks that start at or beyond Lk (last, partial tile) are pointed at the tile's chunk 0: their scores are masked
+  auto issue_bias = [&](int j) {
+    const unsigned char* bt = bbase + (int64_t)j * (BN * 2);
+    const unsigned adj = (j * BN + bchunk * 8 >= Lk) ? bchunk * 16 : 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16s(bt, boff[i] - adj, blds + i * 1024);
+  };
+  if constexpr (BIAS == 2)
+    if (ntiles > 0) issue_bias(0);
 
   auto tile = [&](int j, auto bufc) {
     constexpr int BUF = decltype(bufc)::value;
@@ -300,7 +328,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     // bias of a full tile: 8 loads of 4 keys each, issued now and consumed after the S MFMAs
     const bool full_tile = j * BN + BN <= Lk;
     u32x2 braw[BIAS ? 8 : 1];
-    if constexpr (BIAS) {
+    if constexpr (BIAS == 1) {
       if (full_tile) {
         const unsigned char* bt = brow + (int64_t)j * (BN * 2);
 #pragma unroll
@@ -340,11 +368,12 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     if constexpr (BIAS) {
       const float cs = a.scale_abs;
       typedef T T4 __attribute__((ext_vector_type(4)));
-      if (full_tile) {
+      if (BIAS == 2 || full_tile) {
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
           for (int q4 = 0; q4 < 4; ++q4) {
+            if constexpr (BIAS == 2) braw[4 * blk + q4] = *(const u32x2*)(smem + (baddr ^ ((4 * blk + q4) * 16)));
             const T4 bv = __builtin_bit_cast(T4, braw[4 * blk + q4]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -385,6 +414,11 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     for (int v = 1; v < 15; v += 2) mx = max3(mx, s1[v], s1[v + 1]);
     mx = fmaxf(mx, s1[15]);
     mx = pair_max32(mx);
+    if constexpr (BIAS == 2) {
+      // the next tile's bias may overwrite this one now: the maximum depends on every value that was read
+      asm volatile("" : : "v"(mx) : "memory");
+      if (more) issue_bias(j + 1);
+    }
     const bool grow = mx > m_run + lazy;  // first visible tile: m_run = -inf
     if (__builtin_amdgcn_ballot_w64(grow) != 0) {
       const float m_new = grow ? mx : m_run;
@@ -920,9 +954,9 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   return a;
 }
 
-template <typename T, int DP, int MINB, bool BIAS, bool DROP = false, bool DMASK = false>
+template <typename T, int DP, int MINB, int BIAS, bool DROP = false, bool DMASK = false>
 int launch_tile(KArgs a, hipStream_t st) {
-  constexpr int lds = 4 * 64 * DP * 2;
+  constexpr int lds = 4 * 64 * DP * 2 + (BIAS == 2 ? 4 * 4096 : 0);
   constexpr auto kfn = fa_tile_kernel<T, DP, MINB, BIAS, DROP, DMASK>;
   if (!ensure_dynamic_lds<kfn>(lds)) return FA_ERR_LAUNCH;
   const int nblk = (a.seqlen_q + 127) / 128;
@@ -980,9 +1014,15 @@ int dispatch(const KArgs& a, int kern, hipStream_t st) {
     return launch_tile<T, 256, 1, false, true>(a, st);
   }
   if (a.bias) {
-    if (dp == 64) return launch_tile<T, 64, 2, true>(a, st);
-    if (dp == 128) return launch_tile<T, 128, 2, true>(a, st);
-    return launch_tile<T, 256, 1, true>(a, st);
+    // 16-byte pieces of bias rows can be fetched by DMA one tile ahead when every row starts 16-byte aligned and no
+    // piece straddles the end of a row; otherwise the kernel reads 8-byte pieces directly
+    const bool staged = !a.cu_q && !a.seqused_k && a.seqlen_k % 8 == 0 && (uintptr_t)a.bias % 16 == 0 &&
+                        a.bias_sb % 16 == 0 && a.bias_sh % 16 == 0 && a.bias_sq % 16 == 0;
+    if (staged && dp == 64) return launch_tile<T, 64, 2, 2>(a, st);
+    if (staged && dp == 128) return launch_tile<T, 128, 2, 2>(a, st);
+    if (dp == 64) return launch_tile<T, 64, 2, 1>(a, st);
+    if (dp == 128) return launch_tile<T, 128, 2, 1>(a, st);
+    return launch_tile<T, 256, 1, 1>(a, st);
   }
   if (dp == 64) return launch_tile<T, 64, 2, false>(a, st);
   if (dp == 128) return launch_tile<T, 128, 2, false>(a, st);
