@@ -400,10 +400,10 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
     // P^T = exp2(S^T c - LSE), dS^T = P^T (dP^T - delta); masked positions contribute nothing
     // masked positions (beyond the sequence, above the causal diagonal) get a score whose exponential is 0; only the
     // diagonal and tail tiles run this
-    // (the bias variant, short of registers, selects per element in the loop below instead)
+    // (the variant that reads the bias directly, short of registers, selects per element in the loop below instead)
     const bool need_mask = (j * BN + BN > Lk) || (a.is_causal && j * BN + BN - 1 > wave_row_lo + off);
     const int lim = need_mask ? min(last_k, causal_row_lim) - j * BN - 4 * g : 0x7fffffff;  // element e visible iff e <= lim
-    if (!BIAS && need_mask) {
+    if (BIAS != 1 && need_mask) {
       const float gone = (c < 0.f) ? INFINITY : -INFINITY;           // times c: -inf (c is never 0)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
@@ -440,7 +440,7 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
             xl = lse2 - Mma<T>::to_float((unsigned short)((v & 1) ? (bw >> 16) : (bw & 0xffffu))) * kLog2e;
           }
           float p = fast_exp2(sv * c - xl);
-          if constexpr (BIAS) p = (32 * (t >> 1) + 8 * (v >> 2) + (v & 3) <= lim) ? p : 0.f;
+          if constexpr (BIAS == 1) p = (32 * (t >> 1) + 8 * (v >> 2) + (v & 3) <= lim) ? p : 0.f;
           if constexpr (DROP) dpv = (((word >> (8 * u)) & 0xffu) <= a.drop_thr) ? dpv * a.drop_rp : 0.f;
           ds[u] = p * (dpv - delta);
         }
@@ -801,6 +801,15 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
           }
         }
       }
+      // masked positions get a score whose exponential is 0; only diagonal and tail tiles run this
+      if (need_mask) {
+        const float gone = (c < 0.f) ? INFINITY : -INFINITY;  // times c: -inf (c is never 0)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int qc = 32 * qbk + 8 * (v >> 2) + (v & 3);  // ql - 4 g
+          if (!((unsigned)(qc - m_base) < m_span)) s[v] = gone;
+        }
+      }
       s16x8 pb[2], dsb[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
@@ -825,11 +834,6 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
           const float d0 = (DO_K && !DELTA_INIT) ? dl[v >> 2][v & 3] : 0.f;
           const float d1 = (DO_K && !DELTA_INIT) ? dl[v >> 2][(v & 3) + 1] : 0.f;
           float p0 = fast_exp2(s[v] * c - l0), p1 = fast_exp2(s[v + 1] * c - l1);
-          if (need_mask) {
-            const int qc = 32 * qbk + 8 * (v >> 2) + (v & 3);  // ql - 4 g
-            p0 = ((unsigned)(qc - m_base) < m_span) ? p0 : 0.f;
-            p1 = ((unsigned)(qc + 1 - m_base) < m_span) ? p1 : 0.f;
-          }
           float dp0 = DO_K ? dp[v] : 0.f, dp1 = DO_K ? dp[v + 1] : 0.f;
           float pv0 = p0, pv1 = p1;  // what multiplies dO in dV: P o M / (1 - p)
           if constexpr (DROP) {
