@@ -38,6 +38,10 @@
 #ifndef FA_RT
 #define FA_RT(DO_K, DO_V) ((DO_K) && (DO_V) ? 2 : 4)
 #endif
+// dV-only kernel: all 64 query rows of a tile in one pass (needs 16 more registers)
+#ifndef FA_WIDE
+#define FA_WIDE(DO_K, DO_V, DP, BIAS) (!(DO_K) && (DP) == 128 && !(BIAS))
+#endif
 namespace {
 
 using namespace fa;
@@ -740,6 +744,90 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
     const unsigned m_span = (unsigned)max(Lq - qlo - m_lo, 0);  // visible iff (unsigned)(ql - m_lo) < m_span
     const int m_base = m_lo - 4 * g;
 
+    // dV alone (head_dim > 64, no bias): the registers allow the scores of all 64 query rows at once, as in the forward
+    // kernel: two independent accumulator chains in the S product, one pass of exponentials, 16 dV MFMAs in a row.
+    // With 32 rows per pass a wavefront changes between matrix and vector work twice as often, and a SIMD's two
+    // wavefronts cover each other's changes less well.
+    constexpr bool WIDE = FA_WIDE(DO_K, DO_V, DP, BIAS);
+    if constexpr (WIDE) {
+      f32x16 s2[2];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) { s2[0][v] = 0.f; s2[1][v] = 0.f; }
+      f32x4 lv[2][4];
+      {
+        s16x8 qa[2][2];  // [slot][block]: fetched two k-steps ahead
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          qa[ks][0] = *(const s16x8*)(qt + kaddr[ks]);
+          qa[ks][1] = *(const s16x8*)(qt + kaddr[ks] + 32 * ROWB);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          s2[0] = Mma<T>::m32(qa[ks & 1][0], kf[ks], s2[0]);
+          s2[1] = Mma<T>::m32(qa[ks & 1][1], kf[ks], s2[1]);
+          if (ks + 2 < KS) {
+            qa[ks & 1][0] = *(const s16x8*)(qt + kaddr[ks + 2]);
+            qa[ks & 1][1] = *(const s16x8*)(qt + kaddr[ks + 2] + 32 * ROWB);
+          }
+          if (ks == KS / 2) {  // LSE of this lane's 32 rows, in time for the exponentials
+#pragma unroll
+            for (int qbk = 0; qbk < 2; ++qbk)
+#pragma unroll
+              for (int q4 = 0; q4 < 4; ++q4) lv[qbk][q4] = *(const f32x4*)(lse_t + 32 * qbk + 8 * q4 + 4 * g);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if (need_mask) {
+        const float gone = (c < 0.f) ? INFINITY : -INFINITY;  // times c: -inf (c is never 0)
+#pragma unroll
+        for (int qbk = 0; qbk < 2; ++qbk)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int qc = 32 * qbk + 8 * (v >> 2) + (v & 3);  // ql - 4 g
+            if (!((unsigned)(qc - m_base) < m_span)) s2[qbk][v] = gone;
+          }
+      }
+      // transposed dO fragments: step i = (chunk tt of 16 query rows, mb), fetched RT - 1 steps ahead
+      auto tfrag = [&](int i) {
+        const int ro = (16 * (i / MB)) * ROWB;
+        const s16x4 lo = lds_read_tr(dt + taddr[0][i % MB] + ro);
+        const s16x4 hi = lds_read_tr(dt + taddr[1][i % MB] + ro);
+        return s16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      };
+      constexpr int RT = 4;
+      s16x8 dav[RT];
+#pragma unroll
+      for (int i = 0; i < RT - 1; ++i) dav[i] = tfrag(i);
+      s16x8 pb[4];
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) {  // chunk tt: rows 16 tt .. 16 tt + 15 = block tt / 2, half tt % 2
+        u32x4 wp;
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          const int qbk = tt >> 1, v = 8 * (tt & 1) + 2 * e2;
+          const float l0 = lv[qbk][v >> 2][v & 3], l1 = lv[qbk][v >> 2][(v & 3) + 1];
+          float p0 = fast_exp2(s2[qbk][v] * c - l0), p1 = fast_exp2(s2[qbk][v + 1] * c - l1);
+          if constexpr (DROP) {
+            const uint32_t rp_const = 16 * qbk + 4 * (v >> 2) + ((v & 3) >> 1);
+            const uint32_t word = drop_mix(drop_tile ^ (rp_const << 16)) >> drop_sh;
+            p0 = ((word & 0xffu) <= a.drop_thr) ? p0 * a.drop_rp : 0.f;
+            p1 = (((word >> 16) & 0xffu) <= a.drop_thr) ? p1 * a.drop_rp : 0.f;
+          }
+          wp[e2] = Mma<T>::pack2(p0, p1);
+        }
+        pb[tt] = __builtin_bit_cast(s16x8, wp);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 4 * MB; ++i) {
+        if (i + RT - 1 < 4 * MB) dav[(i + RT - 1) % RT] = tfrag(i + RT - 1);
+        dv[i % MB] = Mma<T>::m32(dav[i % RT], pb[i / MB], dv[i % MB]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      continue;
+    }
 #pragma unroll
     for (int qbk = 0; qbk < 2; ++qbk) {  // two blocks of 32 query rows
       // LSE and delta of this lane's 16 rows (register v <-> row 32 qbk + 8 (v >> 2) + 4 g + (v & 3)), fetched ahead
