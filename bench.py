@@ -32,10 +32,10 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC_BYTES = {
     "cfg2": int((522.2 + 130.0) * 2 ** 20),
     "cfg5": int(2.0021 * 2 ** 30 + 4.25 * 2 ** 20),
-    "cfg2_bwd": int((1814.5 + 388.1) * 2 ** 20),  # the three launches of one backward together
-    "cfg2_mask": int(3.70 * 2 ** 30 + 223.3 * 2 ** 20),
-    "cfg2_drop": int((518.5 + 130.0) * 2 ** 20),
-    "cfg2_mask_bwd": int((3.23 + 4.42 + 2.42) * 2 ** 30 + (151.9 + 133.4 + 130.5) * 2 ** 20),  # three launches
+    "cfg2_bwd": int((1828.3 + 388.2) * 2 ** 20),  # the three launches of one backward together
+    "cfg2_mask": int(4.39 * 2 ** 30 + 255.0 * 2 ** 20),
+    "cfg2_drop": int((518.6 + 130.0) * 2 ** 20),
+    "cfg2_mask_bwd": int((4.71 + 4.44 + 4.21) * 2 ** 30 + (148.1 + 135.9 + 131.6) * 2 ** 20),  # three launches
 }
 
 

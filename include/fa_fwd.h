@@ -71,7 +71,9 @@ extern "C" {
  * bias (optional, same dtype as q): element (b,h,row,col) at bias + b*bias_stride_b + h*bias_stride_h
  * + row*bias_stride_q + col (packed mode: b = the sequence, row and col counted from its first row / key); columns
  * contiguous; stride 0 broadcasts over batch or heads (or rows); the base pointer and all three strides must keep
- * 4-element groups 8-byte aligned (multiples of 4 elements).  A problem with a bias always runs the tile kernel.
+ * 4-element groups 8-byte aligned (multiples of 4 elements).  A problem with a bias always runs the tile kernel; when
+ * the base pointer and the strides are multiples of 8 elements and seqlen_k is a multiple of 8 (dense mode), the kernel
+ * prefetches bias tiles through LDS, which is faster and gives the same bits.
  */
 typedef struct fa_fwd_params {
   const void* q;   /* device, 16-byte aligned */
