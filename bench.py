@@ -33,9 +33,9 @@ TRAFFIC_BYTES = {
     "cfg2": int((522.2 + 130.0) * 2 ** 20),
     "cfg5": int(2.0021 * 2 ** 30 + 4.25 * 2 ** 20),
     "cfg2_bwd": int((1828.3 + 388.2) * 2 ** 20),  # the three launches of one backward together
-    "cfg2_mask": int(4.39 * 2 ** 30 + 255.0 * 2 ** 20),
+    "cfg2_mask": int(2.17 * 2 ** 30 + 199.5 * 2 ** 20),
     "cfg2_drop": int((518.6 + 130.0) * 2 ** 20),
-    "cfg2_mask_bwd": int((4.71 + 4.44 + 4.21) * 2 ** 30 + (148.1 + 135.9 + 131.6) * 2 ** 20),  # three launches
+    "cfg2_mask_bwd": int((2.80 + 2.24 + 2.00) * 2 ** 30 + (148.1 + 128.6 + 128.0) * 2 ** 20),  # three launches
 }
 
 

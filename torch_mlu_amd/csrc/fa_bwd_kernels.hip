@@ -35,6 +35,9 @@
 #ifndef FA_RS
 #define FA_RS(DO_K, DO_V) ((DO_K) ? 2 : 4)
 #endif
+#ifndef FA_HGROUP
+#define FA_HGROUP 4
+#endif
 #ifndef FA_RT
 #define FA_RT(DO_K, DO_V) ((DO_K) && (DO_V) ? 2 : 4)
 #endif
@@ -77,6 +80,7 @@ struct BArgs {
   // causal problems with few workgroups per CU: heads of an XCD's range interleaved, heaviest block index first
   // (better balance); otherwise head after head (better L2 reuse)
   int32_t blockmajor_q, blockmajor_k;
+  int32_t hgroup_q, hgroup_k;  // a bias shared by all heads: (kv) heads whose workgroups are interleaved (1 = none)
   float scale;       // signed softmax scale
   float scale_log2;  // scale * log2(e), signed
   uint32_t drop_thr;  // dropout: an element was kept iff its byte <= drop_thr
@@ -152,8 +156,17 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
       bh = (lid & 7) * nh + idx % nh;
     } else {
       if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
-      pslot = lid % a.n_qslot;
-      bh = lid / a.n_qslot;
+      if (BIAS && a.hgroup_q > 1) {
+        // a bias broadcast over heads: the same query block of hgroup_q heads runs side by side, so that one fetch
+        // of a bias tile serves all of them from L2
+        const int span = a.hgroup_q * a.n_qslot;
+        const int r = lid % span;
+        pslot = r / a.hgroup_q;
+        bh = (lid / span) * a.hgroup_q + r % a.hgroup_q;
+      } else {
+        pslot = lid % a.n_qslot;
+        bh = lid / a.n_qslot;
+      }
     }
   }
   const int h = bh % a.heads_q, b = bh / a.heads_q;
@@ -556,8 +569,15 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
       bhk = (lid & 7) * nh + idx % nh;
     } else {
       if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
-      pslot = lid % a.n_kslot;
-      bhk = lid / a.n_kslot;
+      if (BIAS && a.hgroup_k > 1) {  // as in the dQ kernel: the same key block of hgroup_k kv heads side by side
+        const int span = a.hgroup_k * a.n_kslot;
+        const int r = lid % span;
+        pslot = r / a.hgroup_k;
+        bhk = (lid / span) * a.hgroup_k + r % a.hgroup_k;
+      } else {
+        pslot = lid % a.n_kslot;
+        bhk = lid / a.n_kslot;
+      }
     }
   }
   const int hk = bhk % a.heads_k, b = bhk / a.heads_k;
@@ -1161,6 +1181,13 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   a.n_kslot = (p->seqlen_k + 127) / 128;
   a.blockmajor_q = a.is_causal && (int64_t)p->batch * p->heads_q * a.n_qslot < 8 * 256;
   a.blockmajor_k = a.is_causal && (int64_t)p->batch * p->heads_k * a.n_kslot < 8 * 256;
+  a.hgroup_q = a.hgroup_k = 1;
+  if (p->bias && !p->cu_seqlens_q && p->bias_stride_h == 0) {
+    for (int gsz = FA_HGROUP; gsz > 1 && a.hgroup_q == 1; gsz >>= 1)
+      if (p->heads_q % gsz == 0) a.hgroup_q = gsz;
+    for (int gsz = FA_HGROUP; gsz > 1 && a.hgroup_k == 1; gsz >>= 1)
+      if (p->heads_k % gsz == 0) a.hgroup_k = gsz;
+  }
   a.scale = p->scale;
   a.scale_log2 = p->scale * kLog2e;
   if (a.scale_log2 == 0.f) a.scale_log2 = 1e-30f;  // scale 0: uniform probabilities, and -inf * c stays -inf

@@ -27,6 +27,9 @@
 #include "fa_device.h"
 #include "fa_fwd.h"
 
+#ifndef FA_HGROUP
+#define FA_HGROUP 4
+#endif
 namespace {
 
 using namespace fa;
@@ -49,6 +52,7 @@ struct KArgs {
   int32_t seqlen_q, seqlen_k, head_dim;
   int32_t n_mblk;     // tile kernels: workgroups per (sequence, head)
   int32_t pair;       // tile kernel: a workgroup owns query blocks p and n-1-p of its sequence
+  int32_t hgroup;     // tile kernel with a bias that is shared by all heads: heads whose workgroups are interleaved
   int32_t n_splits;   // split-KV kernel
   int32_t is_causal;
   int32_t neg_scale;  // scale < 0: Q is negated on load and |scale| is used, so that max() tracks the true row max
@@ -135,8 +139,17 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   } else {
     const int total = gridDim.x, per = total >> 3;
     if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
-    pslot = lid % a.n_mblk;  // a.n_mblk: workgroups per (sequence, head)
-    bh = lid / a.n_mblk;
+    if (BIAS && a.hgroup > 1) {
+      // a bias broadcast over heads: the same query block of hgroup heads runs side by side, so that one fetch of a
+      // bias tile serves all of them from L2 (at the price of fewer query blocks of a head sharing its K/V)
+      const int span = a.hgroup * a.n_mblk;
+      const int r = lid % span;
+      pslot = r / a.hgroup;
+      bh = (lid / span) * a.hgroup + r % a.hgroup;
+    } else {
+      pslot = lid % a.n_mblk;  // a.n_mblk: workgroups per (sequence, head)
+      bh = lid / a.n_mblk;
+    }
   }
   const int h = bh % a.heads_q, b = bh / a.heads_q;
   const int hk = h / a.group;
@@ -962,6 +975,13 @@ int launch_tile(KArgs a, hipStream_t st) {
   const int nblk = (a.seqlen_q + 127) / 128;
   a.pair = (DP != 256 && !a.cu_q && a.is_causal && nblk >= 2 && (int64_t)a.batch * a.heads_q * ((nblk + 1) / 2) >= 1024) ? 1 : 0;
   a.n_mblk = a.pair ? (nblk + 1) / 2 : nblk;
+  a.hgroup = 1;
+  if (BIAS && !a.cu_q && a.bias_sh == 0)
+    for (int gsz = FA_HGROUP; gsz > 1; gsz >>= 1)
+      if (a.heads_q % gsz == 0) {
+        a.hgroup = gsz;
+        break;
+      }
   const int64_t grid = (int64_t)a.batch * a.heads_q * a.n_mblk;
   if (grid <= 0) return FA_OK;
   if (grid > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
