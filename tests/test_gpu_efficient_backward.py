@@ -98,6 +98,26 @@ def test_broadcast_bias_shapes(bshape, mask):
         _close(name, g, w, BF)
 
 
+@pytest.mark.parametrize("heads", [(3, 3), (4, 4), (8, 2), (12, 4), (5, 1), (16, 16)])
+@pytest.mark.parametrize("mask", ["none", "tl"])
+def test_head_broadcast_bias_with_various_head_counts(heads, mask):
+    """A bias shared by all heads changes the order in which workgroups run (the same block of up to 4 heads side by
+    side, as many as divide the head count); seqlen_k a multiple of 8 also takes the variants that stage the bias
+    through LDS.  Several query and key blocks per head, so that the interleaving has something to reorder."""
+    Hq, Hk = heads
+    B, Sq, Sk, D = 2, 300, 328, 64
+    q, k, v, do = _inputs(B, Hq, Hk, Sq, Sk, D, BF, 650 + Hq)
+    fb = _bias((B, 1, Sq, Sk), BF, 660 + Hq, holes=0.1)
+    got, want = _run_capi(q, k, v, do, mask, None, fb)
+    for name, g, w in zip(("dq", "dk", "dv", "dbias"), got, want):
+        _close(name, g, w, BF)
+    out, lse = capi.fa_forward_dense(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=MASKS[mask], bias=fb.to(DEV)[..., :Sk])
+    ro, rl = oracle.sdpa_oracle(q, k, v, attn_bias=fb[..., :Sk].double().numpy(), is_causal=mask != "none",
+                                causal_top_left=mask == "tl")
+    assert np.abs(out.float().cpu().numpy() - ro).max() <= 2e-2
+    assert np.abs(lse.cpu().numpy() - rl).max() <= 2e-3
+
+
 @pytest.mark.parametrize("dtype", [BF, HF])
 @pytest.mark.parametrize("shape", [(1, 2, 2, 300, 100, 128), (2, 4, 1, 100, 300, 128), (1, 3, 3, 257, 257, 96),
                                    (2, 2, 2, 64, 512, 40), (1, 8, 2, 1, 333, 64)])
