@@ -352,3 +352,42 @@ def test_reference_flash_backward_grid(dtype, D, p):
                     for causal in (True, False):
                         _reference_grid_case(dtype, B, Sq, Sk, D, l1, causal, p)
         print(f"B={B} done", flush=True)
+
+
+def test_hip_graph_capture_of_forward_and_backward():
+    """A training step (forward + backward ops, flash and mem-efficient with a mask that takes a gradient) recorded into
+    a HIP graph: nothing in the launchers synchronises or reads device memory on the host, and no memset is recorded
+    (the kernels write every output element themselves).  Every replay must give the eager bits; the program's own
+    eager work and synchronisations run between replays."""
+    aten = torch.ops.aten
+    B, H, S, D = 2, 4, 320, 128
+    q, k, v, do = (seeded((B, H, S, D), 1300 + i, BF).to(DEV) for i in range(4))
+    mask = seeded((B, 1, S, S), 1310, BF, std=1.0).to(DEV).expand(B, H, S, S)
+
+    def step():
+        o, lse, cq, ck, mq, mk, ps, po, _ = aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False)
+        g1 = aten._scaled_dot_product_flash_attention_backward(do, q, k, v, o, lse, cq, ck, mq, mk, 0.0, True, ps, po)
+        o2, lse2, ps2, po2 = aten._scaled_dot_product_efficient_attention(q, k, v, mask, True)
+        g2 = aten._scaled_dot_product_efficient_attention_backward(do, q, k, v, mask, o2, lse2, ps2, po2, 0.0,
+                                                                   [True, True, True, True], False)
+        return [o, lse, *g1, o2, lse2, *g2]
+
+    eager = [t.clone() for t in step()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()  # warm the allocator and the kernels' one-time set-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for it in range(3):
+        for t in outs:
+            t.fill_(float("nan")) if t.is_floating_point() else t.zero_()
+        (q.float() @ k.float().transpose(-1, -2)).sum().item()  # eager work and a host read between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for i, (got, want) in enumerate(zip(outs, eager)):
+            assert torch.equal(got, want), (it, i)
