@@ -208,6 +208,38 @@ def test_bias_backward_at_a_prefill_shape():
         _close(name, g, w, BF)
 
 
+@pytest.mark.parametrize("mask", ["tl", "none"])
+def test_head_broadcast_mask_at_a_grid_that_pairs_and_interleaves(mask):
+    """Enough workgroups for the causal forward to pair heavy and light query blocks, a mask shared by all heads (the
+    same block of 4 heads side by side) and rows that qualify for staging through LDS, all at once; forward and the
+    three backward kernels against float32 math on the device, every head."""
+    B, H, S, D = 2, 32, 2048, 128
+    q, k, v, do = (seeded((B, H, S, D), 870 + i, BF).to(DEV) for i in range(4))
+    bias = seeded((B, 1, S, S), 875, BF, std=1.5).to(DEV)
+    hole = torch.rand(B, 1, S, S, generator=torch.Generator().manual_seed(876)) < 0.05
+    hole[..., 0] = False
+    bias = bias.masked_fill(hole.to(DEV), float("-inf"))
+    be = bias.expand(B, H, S, S)
+    out, lse = capi.fa_forward_dense(q, k, v, is_causal=MASKS[mask], bias=be)
+    dq, dk, dv = capi.fa_backward_dense(do, q, k, v, out, lse, is_causal=MASKS[mask], bias=be)[:3]
+    tri = torch.ones(S, S, dtype=torch.bool, device=DEV).tril() if mask == "tl" else None
+    worst = {}
+    for b in range(B):
+        qf, kf, vf, dof = (t[b].float().requires_grad_() for t in (q, k, v, do))
+        sc = qf @ kf.transpose(-1, -2) / math.sqrt(D) + bias[b].float()
+        if tri is not None:
+            sc = sc.masked_fill(~tri, float("-inf"))
+        ref = torch.softmax(sc, -1) @ vf
+        ref.backward(dof.detach())
+        for name, got, want in (("out", out[b], ref.detach()), ("lse", lse[b], torch.logsumexp(sc.detach(), -1)),
+                                ("dq", dq[b], qf.grad), ("dk", dk[b], kf.grad), ("dv", dv[b], vf.grad)):
+            err = (got.float() - want).abs().max().item()
+            bar = 1e-3 if name == "lse" else 2.0 * EPS[BF] * max(want.abs().max().item(), 0.25)
+            worst[name] = max(worst.get(name, 0.0), err / bar)
+        del qf, kf, vf, dof, sc, ref
+    assert all(r <= 1.0 for r in worst.values()), worst
+
+
 # ---- through the registered ATen ops and autograd -------------------------------------------------------------------
 aten = torch.ops.aten
 
