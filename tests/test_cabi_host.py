@@ -76,6 +76,8 @@ def test_validate_accepts_good_params():
     (dict(head_dim=100), capi.FA_ERR_UNSUPPORTED),      # not a multiple of 8
     (dict(heads_k=3), capi.FA_ERR_UNSUPPORTED),         # "must divide number of heads in query"
     (dict(kernel=capi.FA_KERNEL_SPLITKV), capi.FA_ERR_UNSUPPORTED),  # split-KV needs seqlen_q == 1
+    (dict(k_stride_s=1 << 24), capi.FA_ERR_UNSUPPORTED),  # 128 rows x 32 MiB overflow a 32-bit tile offset
+    (dict(v_stride_s=1 << 24), capi.FA_ERR_UNSUPPORTED),
 ])
 def test_validate_rejects(over, rc):
     p = _good(**over)

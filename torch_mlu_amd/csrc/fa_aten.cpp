@@ -106,12 +106,15 @@ void check_inputs(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
   }
 }
 
-// 16-byte vector access needs 8-element-aligned rows; anything else gets one copy (never hit by dense layouts).
+// 16-byte vector access needs 8-element-aligned rows, and the kernels address the rows of a tile with 32-bit byte
+// offsets, so the sequence stride ([.., S, H, D]: dimension -3) must stay below 32 MiB / 128 rows; anything else gets
+// one copy (never hit by dense layouts).
 at::Tensor aligned_or_copy(const at::Tensor& t) {
   bool ok = reinterpret_cast<uintptr_t>(t.data_ptr()) % 16 == 0;
   for (int64_t i = 0; i + 1 < t.dim(); ++i) ok = ok && (t.size(i) == 1 || (t.stride(i) % 8 == 0 && t.stride(i) >= 0));
+  if (t.dim() >= 3 && t.size(-3) > 1) ok = ok && t.stride(-3) * 2 <= (int64_t)(0xffffffffLL / 128);
   if (ok) return t;
-  TORCH_WARN_ONCE("flash attention: input rows are not 16-byte aligned; making one contiguous copy");
+  TORCH_WARN_ONCE("flash attention: input rows are not 16-byte aligned (or lie more than 32 MiB apart); making one contiguous copy");
   return t.contiguous();
 }
 

@@ -1022,6 +1022,8 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
 // ---------------------------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------------------------
+constexpr int64_t kMaxRowStrideBytes = 0xffffffffLL / 128;  // 128 rows x stride must fit an unsigned 32-bit offset
+
 int bwd_validate(const fa_bwd_params* p) {
   if (!p) return FA_ERR_BAD_ARG;
   if (!p->q || !p->k || !p->v || !p->out || !p->dout || !p->lse || !p->dq || !p->dk || !p->dv) return FA_ERR_BAD_ARG;
@@ -1067,8 +1069,9 @@ int bwd_validate(const fa_bwd_params* p) {
       if (s < 0 || (s & 7)) return FA_ERR_BAD_ARG;
   }
   if (p->lse_stride_h < 0 || p->lse_stride_s < 0) return FA_ERR_BAD_ARG;
-  if (p->k_stride_s * 2 > 0x7fffffffLL || p->v_stride_s * 2 > 0x7fffffffLL || p->q_stride_s * 2 > 0x7fffffffLL ||
-      p->do_stride_s * 2 > 0x7fffffffLL)
+  // per-lane byte offsets inside a tile (up to 128 rows) are 32-bit row x 32-bit stride
+  if (p->k_stride_s * 2 > kMaxRowStrideBytes || p->v_stride_s * 2 > kMaxRowStrideBytes ||
+      p->q_stride_s * 2 > kMaxRowStrideBytes || p->do_stride_s * 2 > kMaxRowStrideBytes)
     return FA_ERR_UNSUPPORTED;
   return FA_OK;
 }
@@ -1092,7 +1095,7 @@ int bwd_launch(const BArgs& a, hipStream_t st) {
   constexpr auto kq2 = fa_bwd_dq_kernel<T, DP, DROP, can_stage ? 2 : (BIAS ? 1 : 0)>;
   constexpr int lds_dq2 = lds_dq + 4 * 4096;
   const bool staged = can_stage && !a.cu_q && a.seqlen_k % 8 == 0 && (uintptr_t)a.bias % 16 == 0 && a.bias_sb % 16 == 0 &&
-                      a.bias_sh % 16 == 0 && a.bias_sq % 16 == 0;
+                      a.bias_sh % 16 == 0 && a.bias_sq % 16 == 0 && a.bias_sq <= kMaxRowStrideBytes;
   if (staged && !ensure_dynamic_lds<kq2>(lds_dq2)) return FA_ERR_LAUNCH;
   constexpr auto kkv = fa_bwd_dkv_kernel<T, DP, split ? kDK : (kDK | kDV), DROP, BIAS>;
   constexpr auto kv2 = fa_bwd_dkv_kernel<T, DP, kDV, DROP, BIAS>;

@@ -42,6 +42,10 @@ struct Mma<__bf16> {
     return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
   }
   static __device__ __forceinline__ float to_float(unsigned short bits) { return __builtin_bit_cast(float, (unsigned)bits << 16); }
+  // A pair of probabilities is summed in fp32 before it is rounded: bf16 keeps 8 bits, and a row sum of rounded
+  // values could be off by 2^-9 relative when one key dominates, which the logsumexp would show.
+  static constexpr bool kSumPacked = false;
+  static __device__ __forceinline__ float add_pair(unsigned, float acc) { return acc; }
   static constexpr unsigned short kOne = 0x3f80;     // 1.0
   static constexpr unsigned short kNegMax = 0xff7f;  // the most negative finite value; -inf is the next bit pattern
 };
@@ -58,6 +62,14 @@ struct Mma<_Float16> {
     return __builtin_bit_cast(unsigned, __builtin_convertvector(f, f16x2));
   }
   static __device__ __forceinline__ float to_float(unsigned short bits) { return (float)__builtin_bit_cast(_Float16, bits); }
+  // fp16 keeps 11 bits: the row sum is taken over the packed, rounded pair with one v_dot2c_f32_f16 (pair . (1, 1)
+  // + acc, fp32 accumulation) instead of two fp32 adds; the sum is then also exactly that of the values the PV
+  // product uses.  Worst-case relative error of a row sum 2^-12.
+  static constexpr bool kSumPacked = true;
+  static __device__ __forceinline__ float add_pair(unsigned w, float acc) {
+    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), ones, acc, false);
+  }
   static constexpr unsigned short kOne = 0x3c00;
   static constexpr unsigned short kNegMax = 0xfbff;
 };

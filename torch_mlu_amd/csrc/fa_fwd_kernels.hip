@@ -471,7 +471,9 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
         const int v = 8 * (t & 1) + 2 * e2;
         const float x0 = (t < 2) ? s0[v] : s1[v], x1 = (t < 2) ? s0[v + 1] : s1[v + 1];
         float p0 = fast_exp2(x0 * c - mc), p1 = fast_exp2(x1 * c - mc);
-        rs += p0 + p1;
+        // row sums are those of the undropped probabilities, so with dropout they are taken before the mask
+        constexpr bool sum_packed = Mma<T>::kSumPacked && !DROP;
+        if constexpr (!sum_packed) rs += p0 + p1;
         if constexpr (DROP) {
           // keys j BN + 32 (t >> 1) + 8 (v >> 2) + 4 g + (v & 3), + 1: one column pair, one patch word
           const uint32_t cp_const = 16 * (t >> 1) + 4 * (v >> 2) + ((v & 3) >> 1);
@@ -489,6 +491,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
           p1 = k1 ? p1 : 0.f;
         }
         w[e2] = Mma<T>::pack2(p0, p1);
+        if constexpr (sum_packed) rs = Mma<T>::add_pair(w[e2], rs);
       }
       const s16x8 pb = __builtin_bit_cast(s16x8, w);
 #pragma unroll
@@ -839,6 +842,7 @@ __global__ void __launch_bounds__(64) fa_merge_kernel(const KArgs a) {
 // Host side
 // ---------------------------------------------------------------------------------------------------------
 int padded_dim(int d) { return d <= 64 ? 64 : (d <= 128 ? 128 : 256); }
+constexpr int64_t kMaxRowStrideBytes = 0xffffffffLL / 128;  // 128 rows x stride must fit an unsigned 32-bit offset
 
 int validate(const fa_fwd_params* p) {
   if (!p) return FA_ERR_BAD_ARG;
@@ -867,8 +871,8 @@ int validate(const fa_fwd_params* p) {
     if (p->lse_stride_b < 0) return FA_ERR_BAD_ARG;
   }
   if (p->lse_stride_h < 0 || p->lse_stride_s < 0) return FA_ERR_BAD_ARG;
-  // the kernels form per-row byte offsets as 32-bit row x 32-bit stride
-  if (p->k_stride_s * 2 > 0x7fffffffLL || p->v_stride_s * 2 > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
+  // the kernels form per-lane byte offsets inside a tile (up to 128 rows) as 32-bit row x 32-bit stride
+  if (p->k_stride_s * 2 > kMaxRowStrideBytes || p->v_stride_s * 2 > kMaxRowStrideBytes) return FA_ERR_UNSUPPORTED;
   if (p->is_causal < FA_MASK_NONE || p->is_causal > FA_MASK_CAUSAL_TOP_LEFT) return FA_ERR_BAD_ARG;
   if (p->reserved2 != 0 || !(p->dropout_p >= 0.f && p->dropout_p < 1.f)) return FA_ERR_BAD_ARG;
   if (p->dropout_p > 0.f) {
@@ -1037,7 +1041,8 @@ int dispatch(const KArgs& a, int kern, hipStream_t st) {
     // 16-byte pieces of bias rows can be fetched by DMA one tile ahead when every row starts 16-byte aligned and no
     // piece straddles the end of a row; otherwise the kernel reads 8-byte pieces directly
     const bool staged = !a.cu_q && !a.seqused_k && a.seqlen_k % 8 == 0 && (uintptr_t)a.bias % 16 == 0 &&
-                        a.bias_sb % 16 == 0 && a.bias_sh % 16 == 0 && a.bias_sq % 16 == 0;
+                        a.bias_sb % 16 == 0 && a.bias_sh % 16 == 0 && a.bias_sq % 16 == 0 &&
+                        a.bias_sq <= kMaxRowStrideBytes;
     if (staged && dp == 64) return launch_tile<T, 64, 2, 2>(a, st);
     if (staged && dp == 128) return launch_tile<T, 128, 2, 2>(a, st);
     if (dp == 64) return launch_tile<T, 64, 2, 1>(a, st);
