@@ -118,6 +118,13 @@ def test_plan_decode_uses_splitkv_and_sizes_workspace():
     if need:
         assert capi.lib().fa_fwd_launch(ctypes.byref(p), None, 0, None) == capi.FA_ERR_BAD_ARG
         assert capi.lib().fa_fwd_launch(ctypes.byref(p), 0x7000, need - 1, None) == capi.FA_ERR_BAD_ARG
+    # a shape that is split: the workspace is needed, and a short or missing one is refused on the host
+    p2 = _good(batch=4, heads_q=32, heads_k=8, seqlen_q=1, seqlen_k=32768, is_causal=0)
+    assert _plan(p2) == (capi.FA_OK, capi.FA_KERNEL_SPLITKV, 8)
+    need2 = capi.lib().fa_fwd_workspace_bytes(ctypes.byref(p2))
+    assert need2 == 4 * 32 * 8 * (128 * 4 + 8)
+    assert capi.lib().fa_fwd_launch(ctypes.byref(p2), None, 0, None) == capi.FA_ERR_BAD_ARG
+    assert capi.lib().fa_fwd_launch(ctypes.byref(p2), 0x7000, need2 - 1, None) == capi.FA_ERR_BAD_ARG
     # explicit split count is honoured and capped by the number of 32-row blocks
     p.num_splits = 4
     assert _plan(p) == (capi.FA_OK, capi.FA_KERNEL_SPLITKV, 4)
@@ -129,6 +136,24 @@ def test_plan_decode_uses_splitkv_and_sizes_workspace():
     # wide GQA groups (> 16 query heads per kv head) fall back to the tile kernel
     p = _good(batch=1, heads_q=32, heads_k=1, seqlen_q=1, seqlen_k=4096)
     assert _plan(p)[1] == capi.FA_KERNEL_TILE
+
+
+@pytest.mark.parametrize("batch,heads_k,seqlen_k,want", [
+    (64, 8, 8192, 1),     # 512 (sequence, kv head) units: more than one per CU already
+    (16, 8, 8192, 2),     # 128 units -> 256 workgroups
+    (4, 8, 8192, 4),      # 32 units: 8 would fill the CUs, but 2048-row slices win while 128 workgroups remain
+    (4, 8, 131072, 8),
+    (1, 8, 8192, 16),
+    (1, 8, 32768, 16),
+    (1, 8, 131072, 32),
+    (1, 1, 131072, 64),   # the cap
+    (1, 8, 1024, 2),      # never below 512 rows per slice
+    (256, 8, 2048, 1),
+])
+def test_plan_split_count(batch, heads_k, seqlen_k, want):
+    """The automatic split count: one workgroup per CU at most, long slices preferred."""
+    p = _good(batch=batch, heads_q=4 * heads_k, heads_k=heads_k, seqlen_q=1, seqlen_k=seqlen_k, is_causal=0)
+    assert _plan(p) == (capi.FA_OK, capi.FA_KERNEL_SPLITKV, want)
 
 
 # ---- backward entry points ------------------------------------------------------------------------------------------
