@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0
 # recorded values (None: not profiled).
 TRAFFIC_BYTES = {
     "cfg2": int((522.2 + 130.0) * 2 ** 20),
-    "cfg5": int(2.0021 * 2 ** 30 + 4.25 * 2 ** 20),
+    "cfg5": int(2.0006 * 2 ** 30 + 0.52 * 2 ** 20),
     "cfg2_bwd": int((1828.3 + 388.2) * 2 ** 20),  # the three launches of one backward together
     "cfg2_mask": int(2.17 * 2 ** 30 + 199.5 * 2 ** 20),
     "cfg2_drop": int((518.6 + 130.0) * 2 ** 20),
