@@ -41,6 +41,8 @@ extern "C" {
  * head_dim elements contiguous; packed mode (cu_seqlens_q != NULL) ignores *_stride_b and addresses rows by their
  * packed index.  q, dq, out, dout have heads_q heads; k, v, dk, dv have heads_k heads.  lse is the forward's
  * logsumexp (natural log), read through the same three strides the forward wrote it with.
+ * The sequence strides of q, k, v and dout must stay below 32 MiB in bytes (a tile's rows are addressed with a
+ * 32-bit offset; FA_ERR_UNSUPPORTED otherwise).
  */
 typedef struct fa_bwd_params {
   const void* q;

@@ -64,6 +64,8 @@ extern "C" {
  *          tensors; *_stride_b is ignored; seqlen_q / seqlen_k are upper bounds (max_seqlen) used to size the grid.
  *          cu_seqlens are int32 device arrays of batch+1 non-decreasing entries starting at 0 (:81-84,125-127) and
  *          are only ever read on the device.
+ * The sequence strides (x_stride_s) of K and V must stay below 32 MiB in bytes: the kernels address the rows of a tile
+ * with a 32-bit offset (FA_ERR_UNSUPPORTED otherwise).
  * LSE element (b,h,s) is written at lse + b*lse_stride_b + h*lse_stride_h + s*lse_stride_s; in packed mode s is the
  * packed row index and lse_stride_b is ignored (the reference's kernel-side buffer is [heads_q, total_q], :129).
  * Rows with no visible key (is_causal and Lk < Lq, Lk == 0, or a bias row that is -inf throughout) get out = 0 and
