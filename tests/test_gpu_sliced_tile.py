@@ -1,0 +1,159 @@
+"""GPU parity tests of the sliced tile kernel: few query rows against a long K/V (speculative decoding, chunked prefill,
+a GQA group too wide for the split-KV kernel).  The launcher cuts each query block's key range into slices that run as
+separate workgroups and a merge kernel combines their partial (m, l, O) — the same rule as the split-KV decode path.
+
+Checked against float32 math on the device for every query row, against the unsliced kernel on the same inputs, and
+for the edge cases of the slicing itself: more slices than tiles, slices that a causal mask leaves empty, a ragged KV
+cache (`seqused_k`), head dims 64 / 128 / 256, and the registered ATen op.
+"""
+import ctypes
+import math
+
+import pytest
+import torch
+
+import torch_mlu_amd  # noqa: F401  (loads the extension; fails loudly if it is not built)
+from tests import _util
+from torch_mlu_amd import capi
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF, HF = torch.bfloat16, torch.float16
+
+
+def _randn(shape, seed, dtype, std=0.5):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    return (torch.randn(shape, generator=g, device=DEV, dtype=torch.float32) * std).to(dtype)
+
+
+@torch.no_grad()
+def _fp32(q, k, v, causal, scale=None, used=None):
+    """q [B,Hq,Sq,D], k/v [B,Hk,Sk,D] -> out fp32 [B,Hq,Sq,D], lse [B,Hq,Sq]; bottom-right causal; `used`: keys per
+    sequence that exist."""
+    B, Hq, Sq, D = q.shape
+    Hk, Sk = k.shape[1], k.shape[2]
+    scale = 1.0 / math.sqrt(D) if scale is None else scale
+    out = torch.empty(B, Hq, Sq, D, device=q.device)
+    lse = torch.empty(B, Hq, Sq, device=q.device)
+    for b in range(B):
+        Lk = Sk if used is None else int(used[b])
+        col = torch.arange(Lk, device=q.device)[None, :]
+        rowi = torch.arange(Sq, device=q.device)[:, None]
+        for h in range(Hq):
+            s = (q[b, h].float() @ k[b, h // (Hq // Hk), :Lk].float().T) * scale
+            if causal:
+                s = s.masked_fill(col > rowi + Lk - Sq, float("-inf"))
+            l = torch.logsumexp(s, -1)
+            out[b, h] = torch.exp(s - l[:, None]) @ v[b, h // (Hq // Hk), :Lk].float()
+            lse[b, h] = l
+    return out, lse
+
+
+def _close(out, lse, want_o, want_l, dtype):
+    _util.out_close(out.float().cpu().numpy(), want_o.cpu().numpy(), dtype)
+    _util.lse_close(lse.cpu().numpy(), want_l.cpu().numpy())
+
+
+def _plan(q, k, causal, num_splits=0, kernel=capi.FA_KERNEL_AUTO):
+    B, Hq, Sq, D = q.shape
+    out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    p = capi.make_params(q.transpose(1, 2), k.transpose(1, 2), k.transpose(1, 2), out, lse, is_causal=causal,
+                         kernel=kernel, num_splits=num_splits)
+    kern, ns = ctypes.c_int32(-1), ctypes.c_int32(-1)
+    assert capi.lib().fa_fwd_plan(ctypes.byref(p), ctypes.byref(kern), ctypes.byref(ns)) == capi.FA_OK
+    return kern.value, ns.value
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("Sq", [2, 4, 16, 128, 300])
+def test_few_query_rows_against_32k_keys(Sq, causal):
+    """B=1, Hq=8, Hkv=2, Skv=32768, D=128, bf16: the plan slices, and every row matches float32 math."""
+    B, Hq, Hk, Sk, D = 1, 8, 2, 32768, 128
+    q, k, v = _randn((B, Hq, Sq, D), 1, BF), _randn((B, Hk, Sk, D), 2, BF), _randn((B, Hk, Sk, D), 3, BF)
+    kern, ns = _plan(q, k, causal)
+    assert kern == capi.FA_KERNEL_TILE and ns > 1
+    out, lse = capi.fa_forward_dense(q, k, v, is_causal=causal)
+    _close(out, lse, *_fp32(q, k, v, causal), BF)
+    one, lse1 = capi.fa_forward_dense(q, k, v, is_causal=causal, num_splits=1)   # the unsliced kernel
+    assert (out.float() - one.float()).abs().max().item() <= 2.0 ** -7 * max(one.float().abs().max().item(), 0.25)
+    assert (lse - lse1).abs().max().item() <= 1e-4
+
+
+@pytest.mark.parametrize("dtype,D", [(HF, 64), (BF, 128), (HF, 256), (BF, 72)])
+def test_head_dims_and_explicit_slice_counts(dtype, D):
+    """Explicit slice counts, among them one that is no power of two and one above the number of tiles (clamped)."""
+    B, Hq, Hk, Sq, Sk = 2, 4, 2, 130, 1500   # 24 tiles of 64 keys, the last one partial
+    q, k, v = _randn((B, Hq, Sq, D), 11, dtype), _randn((B, Hk, Sk, D), 12, dtype), _randn((B, Hk, Sk, D), 13, dtype)
+    for causal in (False, True):
+        want = _fp32(q, k, v, causal)
+        for ns in (2, 3, 7, 24, 64):
+            assert _plan(q, k, causal, num_splits=ns)[1] == min(ns, 24)
+            out, lse = capi.fa_forward_dense(q, k, v, is_causal=causal, num_splits=ns)
+            _close(out, lse, *want, dtype)
+
+
+def test_slices_left_empty_by_the_causal_mask():
+    """Sq = 384 (three query blocks) against Skv = 640, bottom-right causal: the first block sees 384 keys only, so its
+    later slices hold no tile; with Skv < Sq the first rows see no key at all (out 0, logsumexp +inf)."""
+    B, Hq, Hk, D = 1, 4, 4, 128
+    for Sq, Sk in ((384, 640), (384, 200)):
+        q, k, v = _randn((B, Hq, Sq, D), 21, BF), _randn((B, Hk, Sk, D), 22, BF), _randn((B, Hk, Sk, D), 23, BF)
+        out, lse = capi.fa_forward_dense(q, k, v, is_causal=True, num_splits=4)
+        one, lse1 = capi.fa_forward_dense(q, k, v, is_causal=True, num_splits=1)
+        dead = torch.isinf(lse1)
+        assert torch.equal(torch.isinf(lse), dead)
+        assert (out.float()[dead] == 0).all()
+        live = ~dead
+        assert (out.float() - one.float()).abs().max().item() <= 2.0 ** -7 * max(one.float().abs().max().item(), 0.25)
+        assert (lse[live] - lse1[live]).abs().max().item() <= 1e-4
+        if Sk >= Sq:
+            _close(out, lse, *_fp32(q, k, v, True), BF)
+
+
+def test_wide_gqa_group_decode():
+    """Sq = 1 with 64 query heads on one kv head: too wide for the split-KV kernel, sliced tile kernel instead."""
+    B, Hq, Hk, Sk, D = 2, 64, 1, 16384, 128
+    q, k, v = _randn((B, Hq, 1, D), 31, BF), _randn((B, Hk, Sk, D), 32, BF), _randn((B, Hk, Sk, D), 33, BF)
+    kern, ns = _plan(q, k, False)
+    assert kern == capi.FA_KERNEL_TILE and ns > 1
+    out, lse = capi.fa_forward_dense(q, k, v)
+    _close(out, lse, *_fp32(q, k, v, False), BF)
+
+
+def test_ragged_kv_cache():
+    """`seqused_k`: slices are cut from each sequence's own used length (one of them shorter than a slice, one empty)."""
+    B, Hq, Hk, Sq, Sk, D = 4, 8, 2, 8, 16384, 128
+    q, k, v = _randn((B, Hq, Sq, D), 41, BF), _randn((B, Hk, Sk, D), 42, BF), _randn((B, Hk, Sk, D), 43, BF)
+    used = torch.tensor([16384, 5000, 70, 0], dtype=torch.int32, device=DEV)
+    for causal in (False, True):
+        out, lse = capi.fa_forward_dense(q, k, v, is_causal=causal, seqused_k=used)
+        assert _plan(q, k, causal)[1] > 1
+        want_o, want_l = _fp32(q[:3], k[:3], v[:3], causal, used=used[:3])
+        _close(out[:3], lse[:3], want_o, want_l, BF)
+        assert (out[3].float() == 0).all() and torch.isinf(lse[3]).all()
+
+
+def test_registered_op_chunked_prefill():
+    """aten::_flash_attention_forward on a 256-token chunk against a 16k cache (the op sizes the workspace itself),
+    and the same under a HIP graph: three replays equal the eager result bit for bit."""
+    B, Hq, Hk, Sq, Sk, D = 1, 16, 4, 256, 16384, 128
+    q, k, v = _randn((B, Sq, Hq, D), 51, BF), _randn((B, Sk, Hk, D), 52, BF), _randn((B, Sk, Hk, D), 53, BF)
+    call = lambda: torch.ops.aten._flash_attention_forward(q, k, v, None, None, Sq, Sk, 0.0, True, False)[:2]
+    out, lse = call()
+    want_o, want_l = _fp32(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), True)
+    _close(out.transpose(1, 2), lse, want_o, want_l, BF)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        call()
+    torch.cuda.current_stream().wait_stream(s)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_out, g_lse = call()
+    for _ in range(3):
+        g_out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_out, out) and torch.equal(g_lse, lse)

@@ -53,7 +53,7 @@ struct KArgs {
   int32_t n_mblk;     // tile kernels: workgroups per (sequence, head)
   int32_t pair;       // tile kernel: a workgroup owns query blocks p and n-1-p of its sequence
   int32_t hgroup;     // tile kernel with a bias that is shared by all heads: heads whose workgroups are interleaved
-  int32_t n_splits;   // split-KV kernel
+  int32_t n_splits;   // split-KV kernel; tile kernel: slices of the key range per query block (1 = none)
   int32_t is_causal;
   int32_t neg_scale;  // scale < 0: Q is negated on load and |scale| is used, so that max() tracks the true row max
   float scale_log2;   // |scale| * log2(e)
@@ -70,6 +70,7 @@ struct KArgs {
   unsigned char* dmask;  // debug mask [batch][heads_q][seqlen_q][seqlen_k] elements, or null
   float* ws_o;        // split-KV partials: [batch*heads_q*n_splits][head_dim] fp32, unnormalised
   float* ws_ml;       // [batch*heads_q*n_splits][2]: m (log2 domain), l
+                      // (sliced tile kernel: the same per query row, [batch*heads_q*seqlen_q*n_splits])
 };
 
 // ---------------------------------------------------------------------------------------------------------
@@ -132,6 +133,10 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   // shorter than that exit at once — longest-processing-time-first without knowing the lengths on the host.
   int lid = blockIdx.x;
   int pslot, bh;
+  // Sliced mode (dense, few query blocks against a long K/V: chunked prefill, speculative decoding): workgroup
+  // `split` of n_splits takes a contiguous range of a block's tiles and leaves unnormalised partials (m, l, O) in
+  // the workspace, which fa_merge_rows_kernel combines.
+  int split = 0;
   if (a.cu_q) {
     const int nbh = a.batch * a.heads_q;
     pslot = lid / nbh;
@@ -139,6 +144,10 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   } else {
     const int total = gridDim.x, per = total >> 3;
     if (lid < (per << 3)) lid = (lid & 7) * per + (lid >> 3);
+    if (a.n_splits > 1) {
+      split = lid % a.n_splits;
+      lid /= a.n_splits;
+    }
     if (BIAS && a.hgroup > 1) {
       // a bias broadcast over heads: the same query block of hgroup heads runs side by side, so that one fetch of a
       // bias tile serves all of them from L2 (at the price of fewer query blocks of a head sharing its K/V)
@@ -258,10 +267,16 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   int n_end = Lk;
   if (a.is_causal) n_end = min(Lk, m0 + BM + off);
   if (n_end < 0) n_end = 0;
-  const int ntiles = (n_end + BN - 1) / BN;
+  const int ntiles_all = (n_end + BN - 1) / BN;
+  int jt0 = 0, ntiles = ntiles_all;  // this workgroup's tiles: [jt0, ntiles)
+  if (a.n_splits > 1) {
+    const int per_split = (ntiles_all + a.n_splits - 1) / a.n_splits;
+    jt0 = split * per_split;
+    ntiles = min(ntiles_all, jt0 + per_split);
+  }
   const int row = m0 + 32 * wave + c32;  // this lane's query row (lanes l and l^32 share it)
   if (own) __syncthreads();  // the previous block's last LDS reads are done
-  if (ntiles > 0) issue_tile(0, 0);
+  if (ntiles > jt0) issue_tile(jt0, 0);
 
   // ---- Q fragments (B operand): lane (c32, g) holds Q[row][16 ks + 8 g .. +8] -----------------------------
   s16x8 qf[KS];
@@ -321,7 +336,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     for (int i = 0; i < 4; ++i) dma16s(bt, boff[i] - adj, blds + i * 1024);
   };
   if constexpr (BIAS == 2)
-    if (ntiles > 0) issue_bias(0);
+    if (ntiles > jt0) issue_bias(jt0);
 
   auto tile = [&](int j, auto bufc) {
     constexpr int BUF = decltype(bufc)::value;
@@ -500,8 +515,16 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     l_run += rs;
   };
 
-  {
-    int j = 0;
+  if (wave_row_lo >= Lq) {
+    // A wavefront without a query row (a block shorter than 128 rows: few-query calls against a long K/V) only
+    // moves its share of the tiles and keeps the barriers; one barrier per tile, as in tile().
+    for (int j = jt0; j < ntiles; ++j) {
+      WAIT_VMCNT(0);
+      __syncthreads();
+      if (j + 1 < ntiles) issue_tile(j + 1, (j + 1 - jt0) & 1);
+    }
+  } else {
+    int j = jt0;
     for (; j + 1 < ntiles; j += 2) {
       tile(j, IC<0>{});
       tile(j + 1, IC<1>{});
@@ -511,6 +534,24 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
 
   // ---- epilogue ----
   l_run = pair_sum32(l_run);
+  if (a.n_splits > 1) {  // sliced: unnormalised partials of this slice, one slot per (sequence, head, row, slice)
+    if (row < Lq) {
+      const int64_t slot = (((int64_t)b * a.heads_q + h) * a.seqlen_q + row) * a.n_splits + split;
+      float* dst = a.ws_o + slot * D;
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {
+          const int d = 32 * mb + 8 * v4 + 4 * g;
+          if (d < D) *(f32x4*)(dst + d) = f32x4{o[mb][4 * v4 + 0], o[mb][4 * v4 + 1], o[mb][4 * v4 + 2], o[mb][4 * v4 + 3]};
+        }
+      if (g == 0) {
+        a.ws_ml[slot * 2 + 0] = (m_run == -INFINITY) ? -INFINITY : m_run * c;
+        a.ws_ml[slot * 2 + 1] = l_run;
+      }
+    }
+    continue;
+  }
   const float inv = (l_run > 0.f) ? (DROP ? a.drop_rp : 1.f) / l_run : 0.f;
   if (row < Lq) {
     unsigned char* orow = a.out + ob + (int64_t)(q0 + row) * a.o_ss + (int64_t)h * a.o_sh;
@@ -838,6 +879,47 @@ __global__ void __launch_bounds__(64) fa_merge_kernel(const KArgs a) {
   if (lane == 0) a.lse[lb + (int64_t)h * a.lse_sh] = (lsum > 0.f) ? (M + __builtin_log2f(lsum)) * kLn2 : INFINITY;
 }
 
+// Merge the partials of the sliced tile kernel: one wavefront per (sequence, query head, query row), four rows per
+// workgroup; lane -> head_dim elements lane, lane+64, ...  Dense mode only.
+template <typename T>
+__global__ void __launch_bounds__(256) fa_merge_rows_kernel(const KArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // (b * heads_q + h) * seqlen_q + row
+  const int64_t rows = (int64_t)a.batch * a.heads_q * a.seqlen_q;
+  if (r >= rows) return;
+  const int row = (int)(r % a.seqlen_q);
+  const int bh = (int)(r / a.seqlen_q);
+  const int h = bh % a.heads_q, b = bh / a.heads_q;
+  const int D = a.head_dim, ns = a.n_splits;
+  const float* ml = a.ws_ml + r * ns * 2;
+  const float* po = a.ws_o + r * ns * D;
+  float M = -INFINITY;
+  for (int s = 0; s < ns; ++s) M = fmaxf(M, ml[2 * s]);
+  float lsum = 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};  // head_dim <= 256
+  for (int s = 0; s < ns; ++s) {
+    const float ms = ml[2 * s];
+    if (ms == -INFINITY) continue;  // a slice without a visible key for this row
+    const float sc = fast_exp2(ms - M);
+    lsum += ml[2 * s + 1] * sc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < D) acc[i] += po[(int64_t)s * D + d] * sc;
+    }
+  }
+  const float inv = (lsum > 0.f) ? 1.f / lsum : 0.f;
+  T* orow = (T*)(a.out + (int64_t)b * a.o_sb + (int64_t)row * a.o_ss + (int64_t)h * a.o_sh);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d < D) orow[d] = (T)(acc[i] * inv);
+  }
+  if (lane == 0)
+    a.lse[(int64_t)b * a.lse_sb + (int64_t)h * a.lse_sh + (int64_t)row * a.lse_ss] =
+        (lsum > 0.f) ? (M + __builtin_log2f(lsum)) * kLn2 : INFINITY;
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------------------------
@@ -920,18 +1002,38 @@ void plan(const fa_fwd_params* p, int* kernel, int* splits) {
     }
     const int nblk = (p->seqlen_k + 31) / 32;
     if (ns > nblk) ns = nblk > 0 ? nblk : 1;
+  } else if (!p->cu_seqlens_q && !p->bias && !(p->dropout_p > 0.f) && p->seqlen_q > 0) {
+    // Tile kernel, dense, plain: with few query blocks against a long K/V (chunked prefill, speculative decoding, a
+    // GQA group too wide for the split-KV kernel) the key range of each block is cut into slices so that the CUs
+    // have two workgroups each; a slice keeps at least 32 tiles (2048 keys).  Partials go through the workspace.
+    const int64_t wgs = (int64_t)p->batch * p->heads_q * ((p->seqlen_q + 127) / 128);
+    const int ntiles = (p->seqlen_k + 63) / 64;
+    ns = p->num_splits;
+    if (ns == 0) {
+      ns = 1;
+      while (ns * 2 <= FA_MAX_SPLITS && wgs * ns * 2 <= 512 && ntiles / (ns * 2) >= 32) ns *= 2;
+    }
+    if (ns > ntiles) ns = ntiles > 0 ? ntiles : 1;
+    // keep the partials (fp32, one slot per query row and slice) within 1 GiB
+    while (ns > 1 && (int64_t)p->batch * p->heads_q * p->seqlen_q * ns * (p->head_dim * 4 + 8) > (1LL << 30)) ns /= 2;
   }
   *kernel = kern;
   *splits = ns;
 }
 
+// partial slots: one per (sequence, query head, slice) for the split-KV kernel (a single query row), one per
+// (sequence, query head, query row, slice) for the sliced tile kernel
+size_t partial_slots(const fa_fwd_params* p, int kern, int ns) {
+  return (size_t)p->batch * p->heads_q * ns * (kern == FA_KERNEL_SPLITKV ? 1 : (size_t)p->seqlen_q);
+}
+
 size_t workspace_bytes(const fa_fwd_params* p, int kern, int ns) {
-  if (kern != FA_KERNEL_SPLITKV || ns <= 1) return 0;
-  const size_t slots = (size_t)p->batch * p->heads_q * ns;
+  if (ns <= 1) return 0;
+  const size_t slots = partial_slots(p, kern, ns);
   return slots * (size_t)p->head_dim * 4 + slots * 8;
 }
 
-KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
+KArgs make_args(const fa_fwd_params* p, int kern, int ns, void* ws) {
   KArgs a;
   a.q = (const unsigned char*)p->q;
   a.k = (const unsigned char*)p->k;
@@ -970,7 +1072,7 @@ KArgs make_args(const fa_fwd_params* p, int ns, void* ws) {
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
   if (ws && ns > 1) {
-    const size_t slots = (size_t)p->batch * p->heads_q * ns;
+    const size_t slots = partial_slots(p, kern, ns);
     a.ws_o = (float*)ws;
     a.ws_ml = (float*)((unsigned char*)ws + slots * (size_t)p->head_dim * 4);
   }
@@ -983,7 +1085,8 @@ int launch_tile(KArgs a, hipStream_t st) {
   constexpr auto kfn = fa_tile_kernel<T, DP, MINB, BIAS, DROP, DMASK>;
   if (!ensure_dynamic_lds<kfn>(lds)) return FA_ERR_LAUNCH;
   const int nblk = (a.seqlen_q + 127) / 128;
-  a.pair = (DP != 256 && !a.cu_q && a.is_causal && nblk >= 2 && (int64_t)a.batch * a.heads_q * ((nblk + 1) / 2) >= 1024) ? 1 : 0;
+  a.pair = (DP != 256 && !a.cu_q && a.n_splits == 1 && a.is_causal && nblk >= 2 &&
+            (int64_t)a.batch * a.heads_q * ((nblk + 1) / 2) >= 1024) ? 1 : 0;
   a.n_mblk = a.pair ? (nblk + 1) / 2 : nblk;
   a.hgroup = 1;
   if (BIAS && !a.cu_q && a.bias_sh == 0)
@@ -992,11 +1095,17 @@ int launch_tile(KArgs a, hipStream_t st) {
         a.hgroup = gsz;
         break;
       }
-  const int64_t grid = (int64_t)a.batch * a.heads_q * a.n_mblk;
+  const int64_t grid = (int64_t)a.batch * a.heads_q * a.n_mblk * a.n_splits;
   if (grid <= 0) return FA_OK;
   if (grid > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(256), lds, st, a);
-  return hipGetLastError() == hipSuccess ? FA_OK : FA_ERR_LAUNCH;
+  if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
+  if (a.n_splits > 1) {
+    const int64_t rows = (int64_t)a.batch * a.heads_q * a.seqlen_q;
+    hipLaunchKernelGGL(fa_merge_rows_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, a);
+    if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
+  }
+  return FA_OK;
 }
 
 template <typename T, int DP>
@@ -1103,7 +1212,7 @@ int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_byte
   const size_t need = workspace_bytes(p, kern, ns);
   if (need > 0 && (!workspace || workspace_bytes_given < need || ((uintptr_t)workspace & 15))) return FA_ERR_BAD_ARG;
   if (p->seqlen_q == 0) return FA_OK;  // nothing to write
-  const KArgs a = make_args(p, ns, workspace);
+  const KArgs a = make_args(p, kern, ns, workspace);
   hipStream_t st = (hipStream_t)stream;
   return p->dtype == FA_DTYPE_BF16 ? dispatch<__bf16>(a, kern, st) : dispatch<_Float16>(a, kern, st);
 }
