@@ -43,9 +43,10 @@ extern "C" {
                                          attention.cpp:368-370) */
 
 /* kernel selection */
-#define FA_KERNEL_AUTO 0     /* split-KV kernel when seqlen_q == 1 and heads_q/heads_k <= 16, else the tile kernel */
+#define FA_KERNEL_AUTO 0     /* split-KV kernel when seqlen_q * (heads_q/heads_k) <= 16 (decode, a few speculative
+                                tokens; packed mode: seqlen_q == 1), else the tile kernel */
 #define FA_KERNEL_TILE 1     /* MFMA tile (prefill) kernel */
-#define FA_KERNEL_SPLITKV 2  /* HBM-bound single-query split-KV kernel + merge */
+#define FA_KERNEL_SPLITKV 2  /* HBM-bound split-KV kernel (+ merge): query rows x group heads share one pass over K/V */
 
 /*
  * One attention-forward problem:  for every sequence b and query head h

@@ -72,10 +72,11 @@ def test_few_query_rows_against_32k_keys(Sq, causal):
     B, Hq, Hk, Sk, D = 1, 8, 2, 32768, 128
     q, k, v = _randn((B, Hq, Sq, D), 1, BF), _randn((B, Hk, Sk, D), 2, BF), _randn((B, Hk, Sk, D), 3, BF)
     kern, ns = _plan(q, k, causal)
-    assert kern == capi.FA_KERNEL_TILE and ns > 1
+    # up to 16 (query row, head of the group) pairs ride the split-KV kernel, more go to the sliced tile kernel
+    assert kern == (capi.FA_KERNEL_SPLITKV if Sq * (Hq // Hk) <= 16 else capi.FA_KERNEL_TILE) and ns > 1
     out, lse = capi.fa_forward_dense(q, k, v, is_causal=causal)
     _close(out, lse, *_fp32(q, k, v, causal), BF)
-    one, lse1 = capi.fa_forward_dense(q, k, v, is_causal=causal, num_splits=1)   # the unsliced kernel
+    one, lse1 = capi.fa_forward_dense(q, k, v, is_causal=causal, num_splits=1)   # the same kernel, unsliced
     assert (out.float() - one.float()).abs().max().item() <= 2.0 ** -7 * max(one.float().abs().max().item(), 0.25)
     assert (lse - lse1).abs().max().item() <= 1e-4
 
@@ -109,6 +110,46 @@ def test_slices_left_empty_by_the_causal_mask():
         assert (lse[live] - lse1[live]).abs().max().item() <= 1e-4
         if Sk >= Sq:
             _close(out, lse, *_fp32(q, k, v, True), BF)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("Sq,Hq,Hk", [(2, 8, 2), (3, 8, 2), (4, 8, 2), (16, 4, 4), (5, 6, 2), (2, 16, 2)])
+def test_speculative_tokens_ride_the_splitkv_kernel(Sq, Hq, Hk, causal):
+    """A few query rows x the heads of a GQA group (at most 16 pairs) share one pass over K/V: every row against
+    float32 math (the causal mask is bottom-right aligned, row r sees Skv - Sq + r + 1 keys), over key lengths around
+    block and slice edges, automatic and explicit slice counts, fp16 and bf16, the tile kernel on the same inputs."""
+    D = 128
+    for i, (B, Sk, dtype) in enumerate([(2, 300, HF), (3, 1025, BF), (1, 8192, BF), (2, 4097, HF)]):
+        q, k, v = (_randn((B, Hq, Sq, D), 60 + i, dtype), _randn((B, Hk, Sk, D), 70 + i, dtype),
+                   _randn((B, Hk, Sk, D), 80 + i, dtype))
+        assert _plan(q, k, causal)[0] == capi.FA_KERNEL_SPLITKV
+        want = _fp32(q, k, v, causal)
+        for ns in (0, 1, 3, 8):
+            out, lse = capi.fa_forward_dense(q, k, v, is_causal=causal, num_splits=ns)
+            _close(out, lse, *want, dtype)
+        til, lse_t = capi.fa_forward_dense(q, k, v, is_causal=causal, kernel=capi.FA_KERNEL_TILE, num_splits=1)
+        _close(til, lse_t, *want, dtype)
+
+
+def test_speculative_tokens_ragged_cache_and_short_keys():
+    """`seqused_k` per sequence, among them fewer keys than query rows (the first rows see nothing: out 0,
+    logsumexp +inf), one key, and none."""
+    B, Hq, Hk, Sq, Sk, D = 5, 8, 2, 4, 2048, 128
+    q, k, v = _randn((B, Hq, Sq, D), 91, BF), _randn((B, Hk, Sk, D), 92, BF), _randn((B, Hk, Sk, D), 93, BF)
+    used = torch.tensor([2048, 777, 3, 1, 0], dtype=torch.int32, device=DEV)
+    for ns in (0, 4):
+        out, lse = capi.fa_forward_dense(q, k, v, is_causal=True, seqused_k=used, num_splits=ns)
+        assert _plan(q, k, True)[0] == capi.FA_KERNEL_SPLITKV
+        _close(out[:2], lse[:2], *_fp32(q[:2], k[:2], v[:2], True, used=used[:2]), BF)
+        til, lse_t = capi.fa_forward_dense(q, k, v, is_causal=True, seqused_k=used, kernel=capi.FA_KERNEL_TILE, num_splits=1)
+        assert torch.equal(torch.isinf(lse), torch.isinf(lse_t))
+        assert torch.isinf(lse[2, :, 0]).all() and not torch.isinf(lse[2, :, 1:]).any()      # 3 keys, 4 rows
+        assert torch.isinf(lse[3, :, :3]).all() and not torch.isinf(lse[3, :, 3]).any()      # 1 key
+        assert torch.isinf(lse[4]).all() and (out[4].float() == 0).all()
+        fin = ~torch.isinf(lse_t)
+        assert (lse[fin] - lse_t[fin]).abs().max().item() <= 1e-3
+        assert (out.float() - til.float()).abs().max().item() <= 2e-2
+        assert (out.float()[torch.isinf(lse)] == 0).all()
 
 
 def test_wide_gqa_group_decode():

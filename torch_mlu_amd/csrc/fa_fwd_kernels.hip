@@ -621,7 +621,7 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
   int q0 = 0, k0 = 0, Lk = a.seqlen_k;  // dense: the query of sequence b is row 0 of batch b
   int64_t qb = (int64_t)b * a.q_sb, kb = (int64_t)b * a.k_sb, vb = (int64_t)b * a.v_sb, ob = (int64_t)b * a.o_sb;
   int64_t lb = (int64_t)b * a.lse_sb;
-  int Lq = 1;
+  int Lq = a.seqlen_q;  // dense: up to 16 / group query rows (a few speculative tokens); packed: one
   if (a.cu_q) {
     q0 = a.cu_q[b];
     Lq = a.cu_q[b + 1] - q0;
@@ -634,6 +634,12 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
   const int D = a.head_dim;
   const int group = a.group;
   const int h0 = hk * group;
+  // q slot L of the MFMA's N dimension <-> (query row L / group, head h0 + L % group); slots >= nslots are zero
+  const int nslots = group * max(Lq, 0);
+  const int slot_r = L / group, slot_g = L % group;
+  // keys this lane's slot may see: bottom-right causal lets row r see keys <= Lk - Lq + r
+  const int slot_lim = a.is_causal ? min(Lk - 1, Lk - Lq + slot_r) : Lk - 1;
+  const int mask_from = a.is_causal ? Lk - (Lq - 1) : Lk;  // first key that some slot does not see
 
   // slice of 32-row blocks owned by this workgroup, then by this wavefront (interleaved)
   const int nblk = (Lk + 31) >> 5;
@@ -673,16 +679,16 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
   int blk = blk_begin + wave;
   if (blk < blk_end && Lq > 0) issue_block(blk, 0);
 
-  // Q^T as B operand of 16x16x32: lane (q slot = L, G) holds Q[h0 + L][32 ks + 8 G .. +8]; slots >= group are zero
+  // Q^T as B operand of 16x16x32: lane (q slot = L, G) holds Q[row][head][32 ks + 8 G .. +8] of its slot
   s16x8 qf[KS];
   {
     const unsigned flip = a.neg_scale ? 0x80008000u : 0u;
-    const unsigned char* qrow = a.q + qb + (int64_t)q0 * a.q_ss + (int64_t)(h0 + L) * a.q_sh;
+    const unsigned char* qrow = a.q + qb + (int64_t)(q0 + slot_r) * a.q_ss + (int64_t)(h0 + slot_g) * a.q_sh;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int ch = 4 * ks + G;
       u32x4 x = {0, 0, 0, 0};
-      if (L < group && ch * 8 < D && Lq > 0) {
+      if (L < nslots && ch * 8 < D) {
         x = *(const u32x4*)(qrow + ch * 16);
         x ^= flip;
       }
@@ -726,8 +732,8 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
       sa = Mma<T>::m16(a0, qf[ks], sa);
       sb = Mma<T>::m16(a1, qf[ks], sb);
     }
-    if (blk * 32 + 32 > Lk) {
-      const int lim = last_k - blk * 32 - 4 * G;
+    if (blk * 32 + 32 > mask_from) {
+      const int lim = slot_lim - blk * 32 - 4 * G;
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         if (v > lim) sa[v] = -INFINITY;
@@ -738,9 +744,10 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
     mx = fmaxf(mx, fmaxf(fmaxf(sb[0], sb[1]), fmaxf(sb[2], sb[3])));
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = pair_max32(mx);
-    const float m_new = fmaxf(m_run, mx);  // a visited block always has at least one visible row: m_new is finite
-    const float alpha = fast_exp2((m_run - m_new) * c);
-    const float mc = m_new * c;
+    // a slot may have seen no key yet (causal rows against the last blocks of a slice): keep m = -inf, p = 0 then
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2((m_run - m_new) * c);
+    const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
     m_run = m_new;
     float rs = 0.f;
 #pragma unroll
@@ -790,7 +797,7 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
   if (Lq <= 0) return;
   // thread -> (q slot, 16 d-values)
   constexpr int TPQ = DP / 16;  // threads per q slot
-  for (int item = tid; item < group * TPQ; item += NW * 64) {
+  for (int item = tid; item < nslots * TPQ; item += NW * 64) {
     const int qs = item / TPQ, d0 = (item % TPQ) * 16;
     float M = -INFINITY;
 #pragma unroll
@@ -807,11 +814,12 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[i] += so[(w * 16 + qs) * DP + d0 + i] * sc;
     }
-    const int h = h0 + qs;
+    const int qr = qs / group;  // query row of this slot (0 in packed mode)
+    const int h = h0 + qs % group;
     if (a.n_splits == 1) {
       const float inv = (lsum > 0.f) ? 1.f / lsum : 0.f;
       if (d0 < D) {
-        unsigned char* orow = a.out + ob + (int64_t)q0 * a.o_ss + (int64_t)h * a.o_sh + d0 * 2;
+        unsigned char* orow = a.out + ob + (int64_t)(q0 + qr) * a.o_ss + (int64_t)h * a.o_sh + d0 * 2;
         u32x4 w0, w1;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -821,9 +829,13 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
         *(u32x4*)orow = w0;
         if (d0 + 8 < D) *(u32x4*)(orow + 16) = w1;
       }
-      if (d0 == 0) a.lse[lb + (int64_t)h * a.lse_sh] = (lsum > 0.f) ? (M + __builtin_log2f(lsum)) * kLn2 : INFINITY;
+      if (d0 == 0)
+        a.lse[lb + (int64_t)h * a.lse_sh + (int64_t)qr * a.lse_ss] = (lsum > 0.f) ? (M + __builtin_log2f(lsum)) * kLn2 : INFINITY;
     } else {
-      const int64_t slot = ((int64_t)b * a.heads_q + h) * a.n_splits + split;
+      // one slot per (sequence, head, query row, slice): what fa_merge_rows_kernel reads (packed: one row per sequence,
+      // which is fa_merge_kernel's layout)
+      const int rows_per = a.cu_q ? 1 : a.seqlen_q;
+      const int64_t slot = (((int64_t)b * a.heads_q + h) * rows_per + qr) * a.n_splits + split;
       if (d0 < D) {
         float* dst = a.ws_o + slot * D + d0;
 #pragma unroll
@@ -970,7 +982,9 @@ int validate(const fa_fwd_params* p) {
     if (p->kernel == FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
   }
   if (p->kernel == FA_KERNEL_SPLITKV) {
-    if (p->seqlen_q != 1 || p->heads_q / p->heads_k > 16) return FA_ERR_UNSUPPORTED;
+    // the query rows x the heads of a GQA group are the 16 columns of its MFMA; packed mode: one row per sequence
+    if (p->seqlen_q < 1 || (int64_t)p->seqlen_q * (p->heads_q / p->heads_k) > 16) return FA_ERR_UNSUPPORTED;
+    if (p->cu_seqlens_q && p->seqlen_q != 1) return FA_ERR_UNSUPPORTED;
     if (p->is_causal == FA_MASK_CAUSAL_TOP_LEFT) return FA_ERR_UNSUPPORTED;  // the single query row would see key 0 only
   }
   return FA_OK;
@@ -980,8 +994,8 @@ void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   int kern = p->kernel;
   const int group = p->heads_q / p->heads_k;
   if (kern == FA_KERNEL_AUTO)
-    kern = (p->seqlen_q == 1 && group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT &&
-            !(p->dropout_p > 0.f))
+    kern = (p->seqlen_q >= 1 && (int64_t)p->seqlen_q * group <= 16 && (p->seqlen_q == 1 || !p->cu_seqlens_q) &&
+            p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT && !(p->dropout_p > 0.f))
                ? FA_KERNEL_SPLITKV
                : FA_KERNEL_TILE;
   int ns = 1;
@@ -1021,10 +1035,11 @@ void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   *splits = ns;
 }
 
-// partial slots: one per (sequence, query head, slice) for the split-KV kernel (a single query row), one per
-// (sequence, query head, query row, slice) for the sliced tile kernel
+// partial slots: one per (sequence, query head, query row, slice) for both kernels (packed mode, split-KV kernel only:
+// one query row per sequence)
 size_t partial_slots(const fa_fwd_params* p, int kern, int ns) {
-  return (size_t)p->batch * p->heads_q * ns * (kern == FA_KERNEL_SPLITKV ? 1 : (size_t)p->seqlen_q);
+  (void)kern;
+  return (size_t)p->batch * p->heads_q * ns * (p->cu_seqlens_q ? 1 : (size_t)p->seqlen_q);
 }
 
 size_t workspace_bytes(const fa_fwd_params* p, int kern, int ns) {
@@ -1118,7 +1133,12 @@ int launch_splitkv(const KArgs& a, hipStream_t st) {
   hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(SplitCfg<DP>::NW * 64), lds, st, a);
   if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
   if (a.n_splits > 1) {
-    hipLaunchKernelGGL(fa_merge_kernel<T>, dim3((unsigned)(a.batch * a.heads_q)), dim3(64), 0, st, a);
+    if (a.cu_q) {
+      hipLaunchKernelGGL(fa_merge_kernel<T>, dim3((unsigned)(a.batch * a.heads_q)), dim3(64), 0, st, a);
+    } else {
+      const int64_t rows = (int64_t)a.batch * a.heads_q * a.seqlen_q;
+      hipLaunchKernelGGL(fa_merge_rows_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, a);
+    }
     if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
   }
   return FA_OK;
