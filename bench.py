@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the flash-attention forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop|cfg2_mask_bwd] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop|cfg2_mask_bwd|spec4|chunk256] [--no-extras] [--no-cpu-baseline]
 
 A "step" is one call of the registered op on one batch of seeded synthetic input that is already resident in HBM.
 The headline workload is BASELINE.json configs[1] (causal prefill, bf16 MHA, B=4 H=32 S=4096 D=128); the other
@@ -185,6 +185,36 @@ def make_workload(name, dev):
         return dict(call=call, check=check, flops=4 * B * Hq * Sk * D, bytes_kv=2 * B * Hk * Sk * D * 2,
                     desc=f"decode bf16 GQA B={B} Hq={Hq} Hkv={Hk} Sq=1 Skv={Sk} D={D}", dtype="bf16", bound="hbm",
                     kernel="fa_splitkv_kernel")
+    if name in ("spec4", "chunk256"):
+        # serving shapes beside the BASELINE configs (extras only): 4 speculative tokens per sequence against a 32k
+        # KV cache (rides the split-KV kernel, HBM-bound) and a 256-token prefill chunk of one sequence against a
+        # 32k cache (tile kernel, sliced over the key range); bottom-right causal, through the dense packed-op entry
+        if name == "spec4":
+            B, Hq, Hk, Sq, Sk, D = 8, 32, 8, 4, 32768, 128
+        else:
+            B, Hq, Hk, Sq, Sk, D = 1, 32, 8, 256, 32768, 128
+        q = seeded((B, Sq, Hq, D), 40, bf).to(dev)
+        nset = 3 if name == "spec4" else 1   # spec4: rotate K/V sets (3 x 1 GiB) past the Infinity Cache
+        k0, v0 = seeded((B, Sk, Hk, D), 41, bf).to(dev), seeded((B, Sk, Hk, D), 42, bf).to(dev)
+        kvs = [(k0, v0)] + [(torch.roll(k0, r, dims=0), torch.roll(v0, r, dims=0)) for r in range(1, nset)]
+        state = {"i": 0}
+
+        def call():
+            kk, vv = kvs[state["i"] % nset]
+            state["i"] += 1
+            return aten._flash_attention_forward(q, kk, vv, None, None, Sq, Sk, 0.0, True, False)
+
+        def check():
+            out, lse = aten._flash_attention_forward(q, k0, v0, None, None, Sq, Sk, 0.0, True, False)[:2]
+            return _check_heads(q.transpose(1, 2), k0.transpose(1, 2), v0.transpose(1, 2), out.transpose(1, 2), lse, True,
+                                [(0, 0), (B - 1, Hq - 1)])
+
+        visible = Sq * (Sk - Sq + 1) + Sq * (Sq - 1) // 2   # (row, key) pairs under the bottom-right causal mask
+        return dict(call=call, check=check, flops=4 * B * Hq * visible * D, bytes_kv=2 * B * Hk * Sk * D * 2,
+                    desc=(f"{Sq} speculative tokens" if name == "spec4" else f"{Sq}-token prefill chunk")
+                         + f" against a {Sk}-key cache, causal, bf16 GQA B={B} Hq={Hq} Hkv={Hk} D={D}",
+                    dtype="bf16", bound="hbm" if name == "spec4" else "mfma",
+                    kernel="fa_splitkv_kernel" if name == "spec4" else "fa_tile_kernel (sliced) + fa_merge_rows_kernel")
     if name == "copy1g":
         # calibration workload for the HBM traffic counters: a plain 1 GiB device-to-device copy
         src = torch.zeros(512 * 1024 * 1024, dtype=bf, device=dev)
@@ -305,7 +335,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "copy1g"])
+    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "spec4", "chunk256", "copy1g"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -350,11 +380,12 @@ def main():
     main_r = run(args.config, args.steps, args.warmup)
     extras = []
     if not args.no_extras:
-        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd"):
+        for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd",
+                     "spec4", "chunk256"):
             if name != args.config:
                 extras.append(run(name, args.steps, args.warmup))
 
-    is_decode = args.config in ("cfg5", "copy1g")
+    is_decode = args.config in ("cfg5", "spec4", "copy1g")
     line = {
         "metric": "fwd attn TFLOP/s + % MFMA peak (bf16 S=4096 D=128); decode HBM GB/s",
         "value": main_r.get("kv_gbs") if is_decode else main_r["tflops"],
@@ -369,7 +400,8 @@ def main():
         "dtype": main_r["dtype"],
         "data": "synthetic (seeded N(0, 0.5^2), generated on the CPU in fp32 and cast)",
         "config": {"workload": main_r["workload"], "name": args.config,
-                   "entry": {"cfg4": "aten::_flash_attention_forward",
+                   "entry": {"cfg4": "aten::_flash_attention_forward", "spec4": "aten::_flash_attention_forward",
+                             "chunk256": "aten::_flash_attention_forward",
                              "cfg2_bwd": "aten::_scaled_dot_product_flash_attention_backward",
                              "cfg2_mask": "aten::_scaled_dot_product_efficient_attention",
                              "cfg2_mask_bwd": "aten::_scaled_dot_product_efficient_attention_backward"}.get(
