@@ -905,18 +905,29 @@ __global__ void __launch_bounds__(256) fa_merge_rows_kernel(const KArgs a) {
   const int D = a.head_dim, ns = a.n_splits;
   const float* ml = a.ws_ml + r * ns * 2;
   const float* po = a.ws_o + r * ns * D;
-  float M = -INFINITY;
-  for (int s = 0; s < ns; ++s) M = fmaxf(M, ml[2 * s]);
-  float lsum = 0.f;
+  // lane s holds slice s's (m, l) (at most 64 slices); the maximum, the scale factors and the sum of l are formed
+  // across the wavefront, then the slices' rows are accumulated with independent loads
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < ns) {
+    const f32x2 v = *(const f32x2*)(ml + 2 * lane);
+    ms = v[0];
+    ls = v[1];
+  }
+  float M = ms;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+  const float scl = (ms == -INFINITY) ? 0.f : fast_exp2(ms - M);  // 0: a slice without a visible key for this row
+  float lsum = ls * scl;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) lsum += __shfl_xor(lsum, o);
   float acc[4] = {0.f, 0.f, 0.f, 0.f};  // head_dim <= 256
+#pragma unroll 4
   for (int s = 0; s < ns; ++s) {
-    const float ms = ml[2 * s];
-    if (ms == -INFINITY) continue;  // a slice without a visible key for this row
-    const float sc = fast_exp2(ms - M);
-    lsum += ml[2 * s + 1] * sc;
+    const float sc = __shfl(scl, s);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int d = lane + 64 * i;
+      // a slice that saw no key leaves zeros (the tile kernel) or finite partial sums; its factor is 0 either way
       if (d < D) acc[i] += po[(int64_t)s * D + d] * sc;
     }
   }
