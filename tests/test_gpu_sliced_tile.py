@@ -198,3 +198,48 @@ def test_registered_op_chunked_prefill():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(g_out, out) and torch.equal(g_lse, lse)
+
+
+@pytest.mark.parametrize("mask_mode", [0, capi.FA_MASK_CAUSAL_TOP_LEFT, True])
+@pytest.mark.parametrize("bias_shape", ["full", "per_batch", "row"])
+def test_sliced_with_additive_bias(bias_shape, mask_mode):
+    """The mem-efficient entry's additive bias (an `attn_mask` for a chunk against a long cache), sliced: full,
+    broadcast over heads, and one row for all queries; with -inf holes; all three mask modes; bias rows 16-byte aligned
+    (staged through LDS) and not."""
+    B, Hq, Hk, Sq, D = 1, 8, 2, 64, 128
+    for Sk in (16384, 16380):
+        q, k, v = _randn((B, Hq, Sq, D), 101, BF), _randn((B, Hk, Sk, D), 102, BF), _randn((B, Hk, Sk, D), 103, BF)
+        shape = {"full": (B, Hq, Sq, Sk), "per_batch": (B, 1, Sq, Sk), "row": (B, 1, 1, Sk)}[bias_shape]
+        bias = _randn(shape, 104, BF, std=1.0)
+        bias[..., 5000:5200] = float("-inf")
+        bias[..., 3::7] = float("-inf")
+        assert _plan_bias(q, k, bias, mask_mode) > 1
+        out, lse = capi.fa_forward_dense(q, k, v, is_causal=mask_mode, bias=bias)
+        one, lse1 = capi.fa_forward_dense(q, k, v, is_causal=mask_mode, bias=bias, num_splits=1)
+        # float32 math
+        be = bias.float().expand(B, Hq, Sq, Sk)
+        col = torch.arange(Sk, device=DEV)[None, :]
+        rowi = torch.arange(Sq, device=DEV)[:, None]
+        for h in range(Hq):
+            s_ = (q[0, h].float() @ k[0, h // 4].float().T) / math.sqrt(D) + be[0, h]
+            if mask_mode is True:
+                s_ = s_.masked_fill(col > rowi + Sk - Sq, float("-inf"))
+            elif mask_mode == capi.FA_MASK_CAUSAL_TOP_LEFT:
+                s_ = s_.masked_fill(col > rowi, float("-inf"))
+            l = torch.logsumexp(s_, -1)
+            o = torch.exp(s_ - l[:, None]) @ v[0, h // 4].float()
+            _close(out[0, h], lse[0, h], o, l, BF)
+        assert (out.float() - one.float()).abs().max().item() <= 2.0 ** -7 * max(one.float().abs().max().item(), 0.25)
+        assert (lse - lse1).abs().max().item() <= 1e-4
+
+
+def _plan_bias(q, k, bias, mask_mode):
+    B, Hq, Sq, D = q.shape
+    out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    p = capi.make_params(q.transpose(1, 2), k.transpose(1, 2), k.transpose(1, 2), out, lse, is_causal=mask_mode,
+                         bias=bias.expand(B, Hq, Sq, k.shape[2]))
+    kern, ns = ctypes.c_int32(-1), ctypes.c_int32(-1)
+    assert capi.lib().fa_fwd_plan(ctypes.byref(p), ctypes.byref(kern), ctypes.byref(ns)) == capi.FA_OK
+    assert kern.value == capi.FA_KERNEL_TILE
+    return ns.value

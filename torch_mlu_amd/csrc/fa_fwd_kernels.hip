@@ -1027,8 +1027,8 @@ void plan(const fa_fwd_params* p, int* kernel, int* splits) {
     }
     const int nblk = (p->seqlen_k + 31) / 32;
     if (ns > nblk) ns = nblk > 0 ? nblk : 1;
-  } else if (!p->cu_seqlens_q && !p->bias && !(p->dropout_p > 0.f) && p->seqlen_q > 0) {
-    // Tile kernel, dense, plain: with few query blocks against a long K/V (chunked prefill, speculative decoding, a
+  } else if (!p->cu_seqlens_q && !(p->dropout_p > 0.f) && p->seqlen_q > 0) {
+    // Tile kernel, dense, no dropout (an additive bias and either causal alignment are fine): with few query blocks against a long K/V (chunked prefill, speculative decoding, a
     // GQA group too wide for the split-KV kernel) the key range of each block is cut into slices so that the CUs
     // have two workgroups each; a slice keeps at least 32 tiles (2048 keys).  Partials go through the workspace.
     const int64_t wgs = (int64_t)p->batch * p->heads_q * ((p->seqlen_q + 127) / 128);
