@@ -243,3 +243,30 @@ def _plan_bias(q, k, bias, mask_mode):
     assert capi.lib().fa_fwd_plan(ctypes.byref(p), ctypes.byref(kern), ctypes.byref(ns)) == capi.FA_OK
     assert kern.value == capi.FA_KERNEL_TILE
     return ns.value
+
+
+def test_sdpa_chunk_with_attn_mask_and_gqa_speculative():
+    """Plain F.scaled_dot_product_attention: a 64-token chunk with a boolean attn_mask against a 16k cache (this build's
+    mem-efficient entry, sliced), and 4 speculative tokens with enable_gqa (this build's flash entry, split-KV kernel);
+    the launch counter proves that the registered HIP path ran."""
+    import torch.nn.functional as F
+    B, Hq, Hk, D, Sk = 1, 8, 2, 128, 16384
+    k, v = _randn((B, Hk, Sk, D), 112, BF), _randn((B, Hk, Sk, D), 113, BF)
+    # chunk + mask (MHA view of the same cache: attn_mask and enable_gqa do not combine in every backend)
+    q = _randn((B, Hk, 64, D), 111, BF)
+    g = torch.Generator(device=DEV).manual_seed(114)
+    mask = torch.rand((64, Sk), generator=g, device=DEV) > 0.3
+    mask[:, 0] = True
+    n0 = torch_mlu_amd.launch_count()
+    out = F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+    assert torch_mlu_amd.launch_count() == n0 + 1
+    s = (q.float() @ k.float().transpose(-1, -2)) / math.sqrt(D)
+    want = torch.softmax(s.masked_fill(~mask, float("-inf")), -1) @ v.float()
+    _util.out_close(out.float().cpu().numpy(), want.cpu().numpy(), BF)
+    # speculative tokens, GQA, no mask
+    q = _randn((B, Hq, 4, D), 115, BF)
+    n0 = torch_mlu_amd.launch_count()
+    out = F.scaled_dot_product_attention(q, k, v, enable_gqa=True)
+    assert torch_mlu_amd.launch_count() == n0 + 1
+    want, _ = _fp32(q, k, v, False)
+    _util.out_close(out.float().cpu().numpy(), want.cpu().numpy(), BF)
