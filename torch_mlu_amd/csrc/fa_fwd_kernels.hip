@@ -1030,13 +1030,15 @@ void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   } else if (!p->cu_seqlens_q && !(p->dropout_p > 0.f) && p->seqlen_q > 0) {
     // Tile kernel, dense, no dropout (an additive bias and either causal alignment are fine): with few query blocks against a long K/V (chunked prefill, speculative decoding, a
     // GQA group too wide for the split-KV kernel) the key range of each block is cut into slices so that the CUs
-    // have two workgroups each; a slice keeps at least 32 tiles (2048 keys).  Partials go through the workspace.
+    // have two workgroups each; a slice keeps at least 32 tiles (2048 keys), or 16 where the chunk is much shorter
+    // than the cache, so that a causal mask leaves every slice equally full.  Partials go through the workspace.
     const int64_t wgs = (int64_t)p->batch * p->heads_q * ((p->seqlen_q + 127) / 128);
     const int ntiles = (p->seqlen_k + 63) / 64;
+    const int min_tiles = ((int64_t)p->seqlen_q * 4 <= p->seqlen_k) ? 16 : 32;
     ns = p->num_splits;
     if (ns == 0) {
       ns = 1;
-      while (ns * 2 <= FA_MAX_SPLITS && wgs * ns * 2 <= 512 && ntiles / (ns * 2) >= 32) ns *= 2;
+      while (ns * 2 <= FA_MAX_SPLITS && wgs * ns * 2 <= 512 && ntiles / (ns * 2) >= min_tiles) ns *= 2;
     }
     if (ns > ntiles) ns = ntiles > 0 ? ntiles : 1;
     // keep the partials (fp32, one slot per query row and slice) within 1 GiB
