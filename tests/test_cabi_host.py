@@ -156,6 +156,28 @@ def test_plan_split_count(batch, heads_k, seqlen_k, want):
     assert _plan(p) == (capi.FA_OK, capi.FA_KERNEL_SPLITKV, want)
 
 
+@pytest.mark.parametrize("over,kern,ns", [
+    (dict(batch=4, heads_q=32, heads_k=32, seqlen_q=4096, seqlen_k=4096), "tile", 1),     # the headline prefill
+    (dict(batch=1, heads_q=32, heads_k=8, seqlen_q=128, seqlen_k=32768), "tile", 16),     # a chunk against a cache
+    (dict(batch=1, heads_q=32, heads_k=8, seqlen_q=512, seqlen_k=32768), "tile", 4),
+    (dict(batch=1, heads_q=8, heads_k=8, seqlen_q=4096, seqlen_k=4096), "tile", 2),       # small-batch prefill
+    (dict(batch=2, heads_q=8, heads_k=8, seqlen_q=2048, seqlen_k=2048), "tile", 1),       # slices would be too short
+    (dict(batch=1, heads_q=64, heads_k=1, seqlen_q=1, seqlen_k=32768), "tile", 8),        # group too wide for split-KV
+    (dict(batch=1, heads_q=32, heads_k=8, seqlen_q=128, seqlen_k=32768, dropout_p=0.1), "tile", 1),
+    (dict(batch=8, heads_q=32, heads_k=8, seqlen_q=4, seqlen_k=32768), "splitkv", 4),     # 4 rows x 4 heads = 16 columns
+    (dict(batch=8, heads_q=32, heads_k=8, seqlen_q=5, seqlen_k=32768), "tile", 2),        # 20 columns: tile kernel
+    (dict(batch=8, heads_q=8, heads_k=8, seqlen_q=16, seqlen_k=32768), "splitkv", 4),
+])
+def test_plan_slices_and_multi_row_decode(over, kern, ns):
+    """Automatic plans: the tile kernel sliced over the key range when a dense call has few query blocks and a long
+    K/V; up to 16 (query row, group head) pairs on the split-KV kernel."""
+    p = _good(**dict(dict(is_causal=1), **over))
+    want = capi.FA_KERNEL_TILE if kern == "tile" else capi.FA_KERNEL_SPLITKV
+    assert _plan(p) == (capi.FA_OK, want, ns)
+    slots = p.batch * p.heads_q * p.seqlen_q * ns
+    assert capi.lib().fa_fwd_workspace_bytes(ctypes.byref(p)) == (0 if ns == 1 else slots * (p.head_dim * 4 + 8))
+
+
 # ---- backward entry points ------------------------------------------------------------------------------------------
 def _good_bwd(**over):
     p = capi.FaBwdParams()
