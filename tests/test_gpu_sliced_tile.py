@@ -270,3 +270,17 @@ def test_sdpa_chunk_with_attn_mask_and_gqa_speculative():
     assert torch_mlu_amd.launch_count() == n0 + 1
     want, _ = _fp32(q, k, v, False)
     _util.out_close(out.float().cpu().numpy(), want.cpu().numpy(), BF)
+
+
+@pytest.mark.parametrize("dtype,D", [(HF, 64), (BF, 96), (HF, 256), (BF, 40)])
+def test_speculative_tokens_other_head_dims(dtype, D):
+    """Several query rows on the split-KV kernel at the other head-dim instances (64, 128 with padding, 256)."""
+    B, Hq, Hk, Sq = 2, 8, 2, 4
+    for causal in (False, True):
+        for Sk in (700, 5000):
+            q, k, v = _randn((B, Hq, Sq, D), 121, dtype), _randn((B, Hk, Sk, D), 122, dtype), _randn((B, Hk, Sk, D), 123, dtype)
+            assert _plan(q, k, causal)[0] == capi.FA_KERNEL_SPLITKV
+            want = _fp32(q, k, v, causal)
+            for ns in (0, 1, 5):
+                out, lse = capi.fa_forward_dense(q, k, v, is_causal=causal, num_splits=ns)
+                _close(out, lse, *want, dtype)
