@@ -44,7 +44,7 @@ extern "C" {
 
 /* kernel selection */
 #define FA_KERNEL_AUTO 0     /* split-KV kernel when seqlen_q * (heads_q/heads_k) <= 16 (decode, a few speculative
-                                tokens; packed mode: seqlen_q == 1), else the tile kernel */
+                                tokens; packed mode: seqlen_q is the longest sequence), else the tile kernel */
 #define FA_KERNEL_TILE 1     /* MFMA tile (prefill) kernel */
 #define FA_KERNEL_SPLITKV 2  /* HBM-bound split-KV kernel (+ merge): query rows x group heads share one pass over K/V */
 
@@ -104,8 +104,8 @@ typedef struct fa_fwd_params {
   int32_t dtype;     /* FA_DTYPE_* */
   int32_t is_causal; /* FA_MASK_* (0 / 1 keep their old meaning) */
   int32_t kernel;    /* FA_KERNEL_* */
-  int32_t num_splits; /* slices of the key range: 0 = choose, else 1..FA_MAX_SPLITS (split-KV kernel; tile kernel in
-                         dense mode without dropout, where each query block's tiles are cut into slices) */
+  int32_t num_splits; /* slices of the key range: 0 = choose, else 1..FA_MAX_SPLITS (split-KV kernel; tile kernel without
+                         dropout, where each query block's tiles are cut into slices) */
   int32_t reserved;  /* must be 0 */
 
   const void* bias;  /* device or NULL */
@@ -144,8 +144,8 @@ const char* fa_fwd_error_string(int rc);
 int fa_fwd_validate(const fa_fwd_params* p);
 
 /*
- * Bytes of device scratch fa_fwd_launch needs for `p`: partial (m, l, o) per slice — per (sequence, query head) for
- * the split-KV kernel, per (sequence, query head, query row) for the sliced tile kernel; 0 when nothing is sliced.  Mirrors cnnlGetFlashAttentionForwardWorkspaceSize_v2.  Returns 0 also when `p` is invalid.
+ * Bytes of device scratch fa_fwd_launch needs for `p`: partial (m, l, o) per slice — per (sequence, query head, query row) for both
+ * kernels (packed mode: seqlen_q rows per sequence); 0 when nothing is sliced.  Mirrors cnnlGetFlashAttentionForwardWorkspaceSize_v2.  Returns 0 also when `p` is invalid.
  */
 size_t fa_fwd_workspace_bytes(const fa_fwd_params* p);
 

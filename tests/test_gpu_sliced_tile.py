@@ -284,3 +284,51 @@ def test_speculative_tokens_other_head_dims(dtype, D):
             for ns in (0, 1, 5):
                 out, lse = capi.fa_forward_dense(q, k, v, is_causal=causal, num_splits=ns)
                 _close(out, lse, *want, dtype)
+
+
+def _packed(lens_q, lens_k, Hq, Hk, D, dtype, seed):
+    cu_q = torch.tensor([0] + list(torch.tensor(lens_q).cumsum(0)), dtype=torch.int32, device=DEV)
+    cu_k = torch.tensor([0] + list(torch.tensor(lens_k).cumsum(0)), dtype=torch.int32, device=DEV)
+    q = _randn((sum(lens_q), Hq, D), seed, dtype)
+    k = _randn((sum(lens_k), Hk, D), seed + 1, dtype)
+    v = _randn((sum(lens_k), Hk, D), seed + 2, dtype)
+    return q, k, v, cu_q, cu_k
+
+
+def _check_packed(out, lse, q, k, v, lens_q, lens_k, causal, dtype):
+    """every sequence against float32 math on its own rows"""
+    oq = ok = 0
+    for Lq, Lk in zip(lens_q, lens_k):
+        if Lq and Lk:
+            want_o, want_l = _fp32(q[oq:oq + Lq].transpose(0, 1)[None], k[ok:ok + Lk].transpose(0, 1)[None],
+                                   v[ok:ok + Lk].transpose(0, 1)[None], causal)
+            _close(out[oq:oq + Lq].transpose(0, 1)[None], lse[:, oq:oq + Lq][None], want_o, want_l, dtype)
+        oq += Lq
+        ok += Lk
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_packed_speculative_tokens(causal):
+    """Packed mode (`cu_seqlens`): sequences with 1-4 new tokens each against caches of different lengths ride the
+    split-KV kernel, sliced or not; an empty sequence in the middle."""
+    lens_q, lens_k = [4, 2, 0, 3, 1], [5000, 300, 0, 8192, 1025]
+    Hq, Hk, D = 8, 2, 128
+    q, k, v, cu_q, cu_k = _packed(lens_q, lens_k, Hq, Hk, D, BF, 131)
+    for ns in (0, 1, 6):
+        out, lse = capi.fa_forward_packed(q, k, v, cu_q, cu_k, max(lens_q), max(lens_k), is_causal=causal, num_splits=ns)
+        _check_packed(out, lse, q, k, v, lens_q, lens_k, causal, BF)
+    til, lse_t = capi.fa_forward_packed(q, k, v, cu_q, cu_k, max(lens_q), max(lens_k), is_causal=causal,
+                                        kernel=capi.FA_KERNEL_TILE, num_splits=1)
+    _check_packed(til, lse_t, q, k, v, lens_q, lens_k, causal, BF)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_packed_chunked_prefill(causal):
+    """Packed mode: chunks of different lengths (one longer than a query block, one empty) against long caches on the
+    sliced tile kernel, automatic and explicit slice counts."""
+    lens_q, lens_k = [200, 64, 0, 130], [16384, 9000, 0, 20000]
+    Hq, Hk, D = 8, 2, 128
+    q, k, v, cu_q, cu_k = _packed(lens_q, lens_k, Hq, Hk, D, HF, 141)
+    for ns in (0, 1, 5, 16):
+        out, lse = capi.fa_forward_packed(q, k, v, cu_q, cu_k, max(lens_q), max(lens_k), is_causal=causal, num_splits=ns)
+        _check_packed(out, lse, q, k, v, lens_q, lens_k, causal, HF)

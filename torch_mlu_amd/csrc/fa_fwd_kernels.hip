@@ -17,7 +17,7 @@
 //                        (sequence, kv head); every wavefront streams its own 32-row K/V blocks through a private
 //                        two-stage LDS ring by global->LDS DMA (no workgroup barriers in the loop), serves all
 //                        query heads of the GQA group from one pass over K/V with v_mfma_f32_16x16x32, and the
-//                        partial (m, l, o) triples are merged in LDS and, across slices, by fa_merge_kernel.
+//                        partial (m, l, o) triples are merged in LDS and, across slices, by fa_merge_rows_kernel.
 //
 // All arithmetic is bf16/fp16 inputs, fp32 accumulate and fp32 softmax in the exp2 domain
 // (the reference asks the vendor kernel for compute_dtype = FLOAT, HIGH_PRECISION: :147-148).
@@ -133,11 +133,15 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   // shorter than that exit at once — longest-processing-time-first without knowing the lengths on the host.
   int lid = blockIdx.x;
   int pslot, bh;
-  // Sliced mode (dense, few query blocks against a long K/V: chunked prefill, speculative decoding): workgroup
+  // Sliced mode (few query blocks against a long K/V: chunked prefill, speculative decoding): workgroup
   // `split` of n_splits takes a contiguous range of a block's tiles and leaves unnormalised partials (m, l, O) in
   // the workspace, which fa_merge_rows_kernel combines.
   int split = 0;
   if (a.cu_q) {
+    if (a.n_splits > 1) {
+      split = lid % a.n_splits;
+      lid /= a.n_splits;
+    }
     const int nbh = a.batch * a.heads_q;
     pslot = lid / nbh;
     bh = lid % nbh;
@@ -832,10 +836,9 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
       if (d0 == 0)
         a.lse[lb + (int64_t)h * a.lse_sh + (int64_t)qr * a.lse_ss] = (lsum > 0.f) ? (M + __builtin_log2f(lsum)) * kLn2 : INFINITY;
     } else {
-      // one slot per (sequence, head, query row, slice): what fa_merge_rows_kernel reads (packed: one row per sequence,
-      // which is fa_merge_kernel's layout)
-      const int rows_per = a.cu_q ? 1 : a.seqlen_q;
-      const int64_t slot = (((int64_t)b * a.heads_q + h) * rows_per + qr) * a.n_splits + split;
+      // one slot per (sequence, head, query row, slice): what fa_merge_rows_kernel reads (packed: seqlen_q is the
+      // longest sequence, shorter ones leave their last slots unused)
+      const int64_t slot = (((int64_t)b * a.heads_q + h) * a.seqlen_q + qr) * a.n_splits + split;
       if (d0 < D) {
         float* dst = a.ws_o + slot * D + d0;
 #pragma unroll
@@ -850,49 +853,9 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
   }
 }
 
-// Merge the per-slice partials: one wavefront per (sequence, query head); lane -> head_dim elements lane, lane+64, ...
-template <typename T>
-__global__ void __launch_bounds__(64) fa_merge_kernel(const KArgs a) {
-  const int bh = blockIdx.x;
-  const int h = bh % a.heads_q, b = bh / a.heads_q;
-  const int lane = threadIdx.x;
-  const int D = a.head_dim, ns = a.n_splits;
-  int q0 = 0;
-  int64_t ob = (int64_t)b * a.o_sb, lb = (int64_t)b * a.lse_sb;
-  if (a.cu_q) {
-    q0 = a.cu_q[b];
-    if (a.cu_q[b + 1] - q0 <= 0) return;
-    ob = 0;
-    lb = (int64_t)q0 * a.lse_ss;
-  }
-  const float* ml = a.ws_ml + (int64_t)bh * ns * 2;
-  const float* po = a.ws_o + (int64_t)bh * ns * D;
-  float M = -INFINITY;
-  for (int s = 0; s < ns; ++s) M = fmaxf(M, ml[2 * s]);
-  float lsum = 0.f;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};  // head_dim <= 256
-  for (int s = 0; s < ns; ++s) {
-    const float ms = ml[2 * s];
-    const float sc = (ms == -INFINITY) ? 0.f : fast_exp2(ms - M);
-    lsum += ml[2 * s + 1] * sc;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int d = lane + 64 * i;
-      if (d < D) acc[i] += po[(int64_t)s * D + d] * sc;
-    }
-  }
-  const float inv = (lsum > 0.f) ? 1.f / lsum : 0.f;
-  T* orow = (T*)(a.out + ob + (int64_t)q0 * a.o_ss + (int64_t)h * a.o_sh);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int d = lane + 64 * i;
-    if (d < D) orow[d] = (T)(acc[i] * inv);
-  }
-  if (lane == 0) a.lse[lb + (int64_t)h * a.lse_sh] = (lsum > 0.f) ? (M + __builtin_log2f(lsum)) * kLn2 : INFINITY;
-}
-
-// Merge the partials of the sliced tile kernel: one wavefront per (sequence, query head, query row), four rows per
-// workgroup; lane -> head_dim elements lane, lane+64, ...  Dense mode only.
+// Merge the per-slice partials of either kernel: one wavefront per (sequence, query head, query row), four rows per
+// workgroup; lane -> head_dim elements lane, lane+64, ...  Packed mode: seqlen_q is the longest sequence; rows beyond
+// a sequence's own length have no partials and are skipped.
 template <typename T>
 __global__ void __launch_bounds__(256) fa_merge_rows_kernel(const KArgs a) {
   const int lane = threadIdx.x & 63;
@@ -903,6 +866,14 @@ __global__ void __launch_bounds__(256) fa_merge_rows_kernel(const KArgs a) {
   const int bh = (int)(r / a.seqlen_q);
   const int h = bh % a.heads_q, b = bh / a.heads_q;
   const int D = a.head_dim, ns = a.n_splits;
+  int64_t orow_off = (int64_t)b * a.o_sb + (int64_t)row * a.o_ss;
+  int64_t lse_off = (int64_t)b * a.lse_sb + (int64_t)row * a.lse_ss;
+  if (a.cu_q) {
+    const int q0 = a.cu_q[b];
+    if (row >= a.cu_q[b + 1] - q0) return;
+    orow_off = (int64_t)(q0 + row) * a.o_ss;
+    lse_off = (int64_t)(q0 + row) * a.lse_ss;
+  }
   const float* ml = a.ws_ml + r * ns * 2;
   const float* po = a.ws_o + r * ns * D;
   // lane s holds slice s's (m, l) (at most 64 slices); the maximum, the scale factors and the sum of l are formed
@@ -932,15 +903,14 @@ __global__ void __launch_bounds__(256) fa_merge_rows_kernel(const KArgs a) {
     }
   }
   const float inv = (lsum > 0.f) ? 1.f / lsum : 0.f;
-  T* orow = (T*)(a.out + (int64_t)b * a.o_sb + (int64_t)row * a.o_ss + (int64_t)h * a.o_sh);
+  T* orow = (T*)(a.out + orow_off + (int64_t)h * a.o_sh);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int d = lane + 64 * i;
     if (d < D) orow[d] = (T)(acc[i] * inv);
   }
   if (lane == 0)
-    a.lse[(int64_t)b * a.lse_sb + (int64_t)h * a.lse_sh + (int64_t)row * a.lse_ss] =
-        (lsum > 0.f) ? (M + __builtin_log2f(lsum)) * kLn2 : INFINITY;
+    a.lse[lse_off + (int64_t)h * a.lse_sh] = (lsum > 0.f) ? (M + __builtin_log2f(lsum)) * kLn2 : INFINITY;
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -995,7 +965,6 @@ int validate(const fa_fwd_params* p) {
   if (p->kernel == FA_KERNEL_SPLITKV) {
     // the query rows x the heads of a GQA group are the 16 columns of its MFMA; packed mode: one row per sequence
     if (p->seqlen_q < 1 || (int64_t)p->seqlen_q * (p->heads_q / p->heads_k) > 16) return FA_ERR_UNSUPPORTED;
-    if (p->cu_seqlens_q && p->seqlen_q != 1) return FA_ERR_UNSUPPORTED;
     if (p->is_causal == FA_MASK_CAUSAL_TOP_LEFT) return FA_ERR_UNSUPPORTED;  // the single query row would see key 0 only
   }
   return FA_OK;
@@ -1005,8 +974,7 @@ void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   int kern = p->kernel;
   const int group = p->heads_q / p->heads_k;
   if (kern == FA_KERNEL_AUTO)
-    kern = (p->seqlen_q >= 1 && (int64_t)p->seqlen_q * group <= 16 && (p->seqlen_q == 1 || !p->cu_seqlens_q) &&
-            p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT && !(p->dropout_p > 0.f))
+    kern = (p->seqlen_q >= 1 && (int64_t)p->seqlen_q * group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT && !(p->dropout_p > 0.f))
                ? FA_KERNEL_SPLITKV
                : FA_KERNEL_TILE;
   int ns = 1;
@@ -1027,8 +995,8 @@ void plan(const fa_fwd_params* p, int* kernel, int* splits) {
     }
     const int nblk = (p->seqlen_k + 31) / 32;
     if (ns > nblk) ns = nblk > 0 ? nblk : 1;
-  } else if (!p->cu_seqlens_q && !(p->dropout_p > 0.f) && p->seqlen_q > 0) {
-    // Tile kernel, dense, no dropout (an additive bias and either causal alignment are fine): with few query blocks against a long K/V (chunked prefill, speculative decoding, a
+  } else if (!(p->dropout_p > 0.f) && p->seqlen_q > 0) {
+    // Tile kernel, no dropout (dense or packed, an additive bias and either causal alignment are fine): with few query blocks against a long K/V (chunked prefill, speculative decoding, a
     // GQA group too wide for the split-KV kernel) the key range of each block is cut into slices so that the CUs
     // have two workgroups each; a slice keeps at least 32 tiles (2048 keys), or 16 where the chunk is much shorter
     // than the cache, so that a causal mask leaves every slice equally full.  Partials go through the workspace.
@@ -1048,11 +1016,11 @@ void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   *splits = ns;
 }
 
-// partial slots: one per (sequence, query head, query row, slice) for both kernels (packed mode, split-KV kernel only:
-// one query row per sequence)
+// partial slots: one per (sequence, query head, query row, slice) for both kernels (packed mode: seqlen_q rows per
+// sequence, the longest one's)
 size_t partial_slots(const fa_fwd_params* p, int kern, int ns) {
   (void)kern;
-  return (size_t)p->batch * p->heads_q * ns * (p->cu_seqlens_q ? 1 : (size_t)p->seqlen_q);
+  return (size_t)p->batch * p->heads_q * ns * (size_t)p->seqlen_q;
 }
 
 size_t workspace_bytes(const fa_fwd_params* p, int kern, int ns) {
@@ -1146,12 +1114,8 @@ int launch_splitkv(const KArgs& a, hipStream_t st) {
   hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(SplitCfg<DP>::NW * 64), lds, st, a);
   if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
   if (a.n_splits > 1) {
-    if (a.cu_q) {
-      hipLaunchKernelGGL(fa_merge_kernel<T>, dim3((unsigned)(a.batch * a.heads_q)), dim3(64), 0, st, a);
-    } else {
-      const int64_t rows = (int64_t)a.batch * a.heads_q * a.seqlen_q;
-      hipLaunchKernelGGL(fa_merge_rows_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, a);
-    }
+    const int64_t rows = (int64_t)a.batch * a.heads_q * a.seqlen_q;
+    hipLaunchKernelGGL(fa_merge_rows_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, a);
     if (hipGetLastError() != hipSuccess) return FA_ERR_LAUNCH;
   }
   return FA_OK;
