@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FA_FWD_ABI_VERSION 4
+#define FA_FWD_ABI_VERSION 5
 
 /* element types accepted for q/k/v/out (FlashAttention_internal.cpp:73-80 allows exactly these two) */
 #define FA_DTYPE_FP16 0
@@ -45,8 +45,12 @@ extern "C" {
 /* kernel selection */
 #define FA_KERNEL_AUTO 0     /* split-KV kernel when seqlen_q * (heads_q/heads_k) <= 16 (decode, a few speculative
                                 tokens; packed mode: seqlen_q is the longest sequence), else the tile kernel */
-#define FA_KERNEL_TILE 1     /* MFMA tile (prefill) kernel */
+#define FA_KERNEL_TILE 1     /* MFMA tile (prefill) kernels; the launcher picks the rows per workgroup (fa_fwd_tile_rows) */
 #define FA_KERNEL_SPLITKV 2  /* HBM-bound split-KV kernel (+ merge): query rows x group heads share one pass over K/V */
+#define FA_KERNEL_TILE128 3  /* tile kernel with 128 query rows per workgroup, two workgroups per CU (every option) */
+#define FA_KERNEL_TILE256 4  /* tile kernel with 256 query rows per workgroup, one per CU, MFMA and softmax overlapped
+                                inside each wavefront: head_dim <= 128, no bias, no dropout, num_splits <= 1
+                                (FA_ERR_UNSUPPORTED otherwise) */
 
 /*
  * One attention-forward problem:  for every sequence b and query head h
@@ -162,6 +166,13 @@ int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_byte
  * negative code when `p` is invalid.  Host-only.
  */
 int fa_fwd_plan(const fa_fwd_params* p, int32_t* kernel, int32_t* num_splits);
+
+/*
+ * Query rows per workgroup of the tile kernel fa_fwd_launch would run for `p`: 128 or 256; 0 when `p` goes to the
+ * split-KV kernel; negative code when `p` is invalid or asks for FA_KERNEL_TILE256 with an option that kernel lacks.
+ * Host-only.  (No counterpart in the reference: its kernel choice is inside the vendor library.)
+ */
+int fa_fwd_tile_rows(const fa_fwd_params* p);
 
 #ifdef __cplusplus
 }

@@ -24,6 +24,9 @@ HIP_FLAGS = [
 ]
 
 
+KERNEL_SOURCES = ("fa_fwd_kernels.hip", "fa_fwd_tile256.hip", "fa_bwd_kernels.hip")
+
+
 def _run(cmd, **kw):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, **kw)
     out = "\n".join(l for l in r.stdout.splitlines() if "is not a recognized feature for this target" not in l)
@@ -32,15 +35,62 @@ def _run(cmd, **kw):
     return out
 
 
+def check_tile256_registers(asm_text: str) -> None:
+    """fa_fwd_tile256.hip assigns the accumulation registers a64 .. a255 by hand inside inline assembly.  The compiler
+    may use accumulation registers of its own (it takes them from a0 upwards); one at or above a64 outside the assembly
+    statements would silently corrupt the O accumulators or the Q fragments, so such a build is refused."""
+    import re
+
+    in_asm = False
+    for line in asm_text.splitlines():
+        t = line.strip()
+        if t.startswith(";;#ASMSTART"):
+            in_asm = True
+        elif t.startswith(";;#ASMEND"):
+            in_asm = False
+        elif not in_asm and t and not t.startswith((";", ".")):
+            code = t.split(";")[0]
+            for m in re.finditer(r"\ba(\d+)\b|\ba\[(\d+):(\d+)\]", code):
+                hi = int(m.group(1) if m.group(1) is not None else m.group(3))
+                if hi >= 64:
+                    raise RuntimeError("fa_fwd_tile256: the compiler allocated a hand-assigned accumulation register: " + t)
+        if "ScratchSize:" in t and "fa_tile256" not in t:
+            pass
+    for m in re.finditer(r"; ScratchSize: (\d+)", asm_text):
+        if int(m.group(1)) != 0:
+            raise RuntimeError("fa_fwd_tile256: vector registers spill to scratch memory")
+
+
 def build_kernels(verbose: bool = False) -> str:
-    """hipcc: csrc/fa_fwd_kernels.hip + csrc/fa_bwd_kernels.hip -> lib/libfa_fwd.so (the C ABI of include/fa_fwd.h and
-    include/fa_bwd.h)."""
+    """hipcc: csrc/fa_fwd_kernels.hip + csrc/fa_fwd_tile256.hip + csrc/fa_bwd_kernels.hip -> lib/libfa_fwd.so (the C ABI of
+    include/fa_fwd.h and include/fa_bwd.h)."""
     os.makedirs(LIBDIR, exist_ok=True)
     out = os.path.join(LIBDIR, "libfa_fwd.so")
     tmp = out + ".tmp"
-    srcs = [os.path.join(CSRC, f) for f in ("fa_fwd_kernels.hip", "fa_bwd_kernels.hip") if os.path.exists(os.path.join(CSRC, f))]
-    log = _run([HIPCC, *HIP_FLAGS, "-shared", f"-I{INCLUDE}", f"-I{CSRC}", *srcs, "-o", tmp])
+    srcs = [os.path.join(CSRC, f) for f in KERNEL_SOURCES]
+    objs = [os.path.join(LIBDIR, os.path.splitext(f)[0] + ".o") for f in KERNEL_SOURCES]
+    # one hipcc process per translation unit, side by side
+    procs = [(src, subprocess.Popen([HIPCC, *HIP_FLAGS, "-c", f"-I{INCLUDE}", f"-I{CSRC}", src, "-o", obj],
+                                    stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
+             for src, obj in zip(srcs, objs)]
+    # the same device code as text, for the register check of the 256-row kernel
+    asm_path = os.path.join(LIBDIR, "fa_fwd_tile256.s")
+    t256 = os.path.join(CSRC, "fa_fwd_tile256.hip")
+    _run([HIPCC, *HIP_FLAGS, "--offload-device-only", "-S", f"-I{INCLUDE}", f"-I{CSRC}", t256, "-o", asm_path])
+    with open(asm_path) as f:
+        check_tile256_registers(f.read())
+    os.remove(asm_path)
+    log = ""
+    for src, pr in procs:
+        o, _ = pr.communicate()
+        o = "\n".join(l for l in o.splitlines() if "is not a recognized feature for this target" not in l)
+        if pr.returncode != 0:
+            raise RuntimeError("build step failed: hipcc -c " + src + "\n" + o)
+        log += o
+    log += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp])
     os.replace(tmp, out)
+    for obj in objs:
+        os.remove(obj)
     if verbose and log.strip():
         print(log)
     return out

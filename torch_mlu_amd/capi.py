@@ -31,6 +31,8 @@ FA_MASK_NONE, FA_MASK_CAUSAL_BOTTOM_RIGHT, FA_MASK_CAUSAL_TOP_LEFT = 0, 1, 2
 FA_KERNEL_AUTO = 0
 FA_KERNEL_TILE = 1
 FA_KERNEL_SPLITKV = 2
+FA_KERNEL_TILE128 = 3
+FA_KERNEL_TILE256 = 4
 FA_MAX_SPLITS = 64
 
 # every symbol include/fa_fwd.h declares
@@ -41,6 +43,7 @@ EXPORTED_SYMBOLS = (
     "fa_fwd_workspace_bytes",
     "fa_fwd_launch",
     "fa_fwd_plan",
+    "fa_fwd_tile_rows",
     "fa_bwd_validate",
     "fa_bwd_workspace_bytes",
     "fa_bwd_launch",

@@ -22,7 +22,9 @@
 #include <ATen/hip/HIPContext.h>
 #include <ATen/hip/HIPGeneratorImpl.h>
 #include <c10/hip/HIPGraphsC10Utils.h>
+#include <ATen/hip/impl/HIPCachingAllocatorMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/core/InferenceMode.h>
 #include <c10/core/DeviceGuard.h>
 #include <c10/util/Logging.h>
 #include <torch/library.h>
@@ -264,25 +266,66 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> flash_att
 namespace {
 
 // Uniform prefix sums arange(0, (B+1) S, S) as the reference fabricates on every call (attention.cpp:109-119).
-// They are immutable, so one copy per (device, B, S) is kept; a miss costs one arange plus one stream sync so
-// that the cached tensor is safe on every stream afterwards.  While a HIP graph is being captured the cache is
-// bypassed (no sync, no allocation that outlives the capture).
+// They are immutable, so one copy per (device, B, S) is kept.  A miss enqueues one arange on the current stream and
+// records an event behind it; a later call on another stream makes that stream wait for the event (a device-side
+// dependency) — the host never waits.  The cached tensor is built outside inference mode and without a gradient
+// history, so that a first call under torch.inference_mode() cannot leave a tensor behind that autograd refuses to
+// save later.  While a HIP graph is being captured the cache is bypassed (no event, no allocation that outlives the
+// capture).  At most kCuSeqlensCacheEntries entries are kept; the least recently used one is dropped first.
+constexpr size_t kCuSeqlensCacheEntries = 256;
+
+struct CuSeqlensEntry {
+  at::Tensor t;
+  hipEvent_t ready = nullptr;   // recorded behind the arange on `stream`
+  hipStream_t stream = nullptr;
+  uint64_t last_use = 0;
+};
+
 at::Tensor uniform_cu_seqlens(int64_t batch, int64_t seqlen, const at::Tensor& like) {
   const auto opts = like.options().dtype(at::kInt);
   auto make = [&] { return at::arange(0, (batch + 1) * seqlen, seqlen > 0 ? seqlen : 1, opts); };
   if (seqlen == 0) return at::zeros({batch + 1}, opts);
   if (c10::hip::currentStreamCaptureStatusMayInitCtx() != c10::hip::CaptureStatus::None) return make();
   static std::mutex mu;
-  static std::map<std::tuple<int, int64_t, int64_t>, at::Tensor> cache;
-  const auto key = std::make_tuple(static_cast<int>(like.device().index()), batch, seqlen);
+  static std::map<std::tuple<int, int64_t, int64_t>, CuSeqlensEntry> cache;
+  static uint64_t tick = 0;
+  const int dev = static_cast<int>(like.device().index());
+  const auto cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(dev);
+  const auto key = std::make_tuple(dev, batch, seqlen);
   std::lock_guard<std::mutex> lock(mu);
   auto it = cache.find(key);
-  if (it != cache.end()) return it->second;
-  if (cache.size() >= 256) cache.clear();
-  at::Tensor t = make();
-  c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(like.device().index()).synchronize();
-  cache.emplace(key, t);
-  return t;
+  if (it == cache.end()) {
+    if (cache.size() >= kCuSeqlensCacheEntries) {
+      auto victim = cache.begin();
+      for (auto e = cache.begin(); e != cache.end(); ++e)
+        if (e->second.last_use < victim->second.last_use) victim = e;
+      // tensors handed out earlier keep the storage alive; the event is only needed by streams that have not used
+      // this entry yet, and no such use can start once the entry is gone
+      if (victim->second.ready) (void)hipEventDestroy(victim->second.ready);
+      cache.erase(victim);
+    }
+    CuSeqlensEntry e;
+    {
+      c10::InferenceMode no_inference(false);
+      at::AutoGradMode no_grad(false);
+      e.t = make();
+    }
+    e.stream = cur.stream();
+    if (hipEventCreateWithFlags(&e.ready, hipEventDisableTiming) != hipSuccess || hipEventRecord(e.ready, e.stream) != hipSuccess) {
+      (void)hipGetLastError();
+      if (e.ready) (void)hipEventDestroy(e.ready);
+      return e.t;  // not cached: the tensor is only known to be ready on this stream
+    }
+    it = cache.emplace(key, std::move(e)).first;
+  } else if (it->second.stream != cur.stream()) {
+    // device-side wait; free once the arange has completed
+    (void)hipStreamWaitEvent(cur.stream(), it->second.ready, 0);
+    // the storage was allocated on another stream: tell the caching allocator about this one, so that the block is
+    // not reused under a reader of this stream after the entry has been dropped
+    c10::hip::HIPCachingAllocatorMasqueradingAsCUDA::recordStreamMasqueradingAsCUDA(it->second.t.storage().data_ptr(), cur);
+  }
+  it->second.last_use = ++tick;
+  return it->second.t;
 }
 
 }  // namespace

@@ -120,6 +120,15 @@ struct IC {
   static constexpr int value = N;
 };
 
+// f(IC<B>{}), f(IC<B + 1>{}), ..., f(IC<E - 1>{}): a loop whose index is a compile-time constant in the body
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(IC<B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
 __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));

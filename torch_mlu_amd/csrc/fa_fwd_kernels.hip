@@ -26,6 +26,7 @@
 
 #include "fa_device.h"
 #include "fa_fwd.h"
+#include "fa_fwd_common.h"
 
 #ifndef FA_HGROUP
 #define FA_HGROUP 4
@@ -34,70 +35,9 @@ namespace {
 
 using namespace fa;
 
-// Kernel arguments: fa_fwd_params plus what the host derives once.
-struct KArgs {
-  const unsigned char* q;
-  const unsigned char* k;
-  const unsigned char* v;
-  unsigned char* out;
-  float* lse;
-  const int32_t* cu_q;
-  const int32_t* cu_k;
-  int64_t q_sb, q_ss, q_sh;  // byte strides
-  int64_t k_sb, k_ss, k_sh;
-  int64_t v_sb, v_ss, v_sh;
-  int64_t o_sb, o_ss, o_sh;
-  int64_t lse_sb, lse_sh, lse_ss;  // element strides
-  int32_t batch, heads_q, heads_k, group;
-  int32_t seqlen_q, seqlen_k, head_dim;
-  int32_t n_mblk;     // tile kernels: workgroups per (sequence, head)
-  int32_t pair;       // tile kernel: a workgroup owns query blocks p and n-1-p of its sequence
-  int32_t hgroup;     // tile kernel with a bias that is shared by all heads: heads whose workgroups are interleaved
-  int32_t n_splits;   // split-KV kernel; tile kernel: slices of the key range per query block (1 = none)
-  int32_t is_causal;
-  int32_t neg_scale;  // scale < 0: Q is negated on load and |scale| is used, so that max() tracks the true row max
-  float scale_log2;   // |scale| * log2(e)
-  float scale_abs;    // |scale| (bias path)
-  int32_t causal_tl;  // causal mask aligned to the top-left corner (col <= row) instead of the bottom-right one
-  const int32_t* seqused_k;   // optional: keys of sequence b beyond seqused_k[b] do not exist
-  const unsigned char* bias;  // optional additive bias, dense mode: [b][h][row][col] through byte strides
-  int64_t bias_sb, bias_sh, bias_sq;
-  uint32_t drop_thr;  // dropout: an element is kept iff its byte <= drop_thr
-  float drop_rp;      // 1 / (1 - p)
-  uint64_t seed, offset;
-  int64_t* rng_seed_out;
-  int64_t* rng_offset_out;
-  unsigned char* dmask;  // debug mask [batch][heads_q][seqlen_q][seqlen_k] elements, or null
-  float* ws_o;        // split-KV partials: [batch*heads_q*n_splits][head_dim] fp32, unnormalised
-  float* ws_ml;       // [batch*heads_q*n_splits][2]: m (log2 domain), l
-                      // (sliced tile kernel: the same per query row, [batch*heads_q*seqlen_q*n_splits])
-};
-
 // ---------------------------------------------------------------------------------------------------------
 // Tile kernel
 // ---------------------------------------------------------------------------------------------------------
-// LDS layouts (rows of DP elements = CPR chunks of 16 bytes; a tile is 64 rows):
-//   K tile: physical chunk = logical chunk ^ swzK(row) so that the 16 lanes of a ds_read_b128 (16 different rows,
-//           same logical chunk) hit 16 different 16-byte bank groups.
-//   V tile: physical chunk = logical chunk ^ swzV(row) so that the 4 rows x 64 bytes a half-wave reads with
-//           ds_read_b64_tr_b16 cover all 64 banks once.
-template <int DP>
-__device__ __forceinline__ int swzK(int row) {
-  if constexpr (DP == 64) return (row >> 1) & 7;
-  return row & 15;
-}
-template <int DP>
-__device__ __forceinline__ int swzV(int row) {
-  if constexpr (DP == 64) return ((row >> 1) & 1) << 2;
-  return (row & 3) << 2;
-}
-
-// A new row maximum only forces a rescale of the accumulators when it exceeds the one in use by more than this
-// many powers of two; until then probabilities are formed against the older maximum and may reach 2^kLazyLog2,
-// which fp32 sums and fp16/bf16 P operands hold without loss.  The final out = O / l and LSE = m c + log2 l do not
-// depend on which maximum was in use.
-constexpr float kLazyLog2 = 8.0f;
-
 // BIAS = 1: an additive bias tile is read straight from global memory into the score layout (one lane = one query
 // row, groups of 4 consecutive keys = 8 bytes) and the softmax then runs on scores already in the log2 domain.
 // BIAS = 2: the same, but the tile is fetched by DMA into LDS one tile ahead (16-byte pieces, so rows must be 16-byte
@@ -929,7 +869,7 @@ int validate(const fa_fwd_params* p) {
   if (p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_UNSUPPORTED;
   if (p->head_dim > 256 || (p->head_dim & 7)) return FA_ERR_UNSUPPORTED;
   if (p->heads_q % p->heads_k) return FA_ERR_UNSUPPORTED;
-  if (p->kernel < FA_KERNEL_AUTO || p->kernel > FA_KERNEL_SPLITKV) return FA_ERR_BAD_ARG;
+  if (p->kernel < FA_KERNEL_AUTO || p->kernel > FA_KERNEL_TILE256) return FA_ERR_BAD_ARG;
   if (p->num_splits < 0 || p->num_splits > FA_MAX_SPLITS) return FA_ERR_BAD_ARG;
   // 16-byte vector access on every row: base pointers and row strides must be multiples of 8 elements
   const uintptr_t al = (uintptr_t)p->q | (uintptr_t)p->k | (uintptr_t)p->v | (uintptr_t)p->out;
@@ -973,6 +913,7 @@ int validate(const fa_fwd_params* p) {
 void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   int kern = p->kernel;
   const int group = p->heads_q / p->heads_k;
+  if (kern == FA_KERNEL_TILE128 || kern == FA_KERNEL_TILE256) kern = FA_KERNEL_TILE;  // the family; tile_rows() picks
   if (kern == FA_KERNEL_AUTO)
     kern = (p->seqlen_q >= 1 && (int64_t)p->seqlen_q * group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT && !(p->dropout_p > 0.f))
                ? FA_KERNEL_SPLITKV
@@ -1007,6 +948,7 @@ void plan(const fa_fwd_params* p, int* kernel, int* splits) {
     if (ns == 0) {
       ns = 1;
       while (ns * 2 <= FA_MAX_SPLITS && wgs * ns * 2 <= 512 && ntiles / (ns * 2) >= min_tiles) ns *= 2;
+      if (p->kernel == FA_KERNEL_TILE256) ns = 1;  // the 256-row kernel is never sliced
     }
     if (ns > ntiles) ns = ntiles > 0 ? ntiles : 1;
     // keep the partials (fp32, one slot per query row and slice) within 1 GiB
@@ -1027,6 +969,18 @@ size_t workspace_bytes(const fa_fwd_params* p, int kern, int ns) {
   if (ns <= 1) return 0;
   const size_t slots = partial_slots(p, kern, ns);
   return slots * (size_t)p->head_dim * 4 + slots * 8;
+}
+
+// Rows per workgroup of the tile kernel that runs `p` (plan() chose the tile family with ns slices): the 256-row
+// kernel takes what it can (head_dim <= 128, no bias, no dropout, not sliced) once there are enough query blocks to
+// give every CU two of its workgroups, one after the other; smaller problems spread better in 128-row workgroups, two
+// per CU.
+int tile_rows(const fa_fwd_params* p, int ns) {
+  const bool can256 = p->head_dim <= 128 && !p->bias && !(p->dropout_p > 0.f) && ns == 1;
+  if (p->kernel == FA_KERNEL_TILE128) return 128;
+  if (p->kernel == FA_KERNEL_TILE256) return can256 ? 256 : 0;
+  if (!can256) return 128;
+  return 128;  // the 256-row kernel only on request while it is being tuned
 }
 
 KArgs make_args(const fa_fwd_params* p, int kern, int ns, void* ws) {
@@ -1194,6 +1148,16 @@ int fa_fwd_plan(const fa_fwd_params* p, int32_t* kernel, int32_t* num_splits) {
   return FA_OK;
 }
 
+int fa_fwd_tile_rows(const fa_fwd_params* p) {
+  const int rc = validate(p);
+  if (rc != FA_OK) return rc;
+  int k, s;
+  plan(p, &k, &s);
+  if (k != FA_KERNEL_TILE) return 0;
+  const int rows = tile_rows(p, s);
+  return rows ? rows : FA_ERR_UNSUPPORTED;
+}
+
 size_t fa_fwd_workspace_bytes(const fa_fwd_params* p) {
   if (validate(p) != FA_OK) return 0;
   int k, s;
@@ -1211,6 +1175,11 @@ int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_byte
   if (p->seqlen_q == 0) return FA_OK;  // nothing to write
   const KArgs a = make_args(p, kern, ns, workspace);
   hipStream_t st = (hipStream_t)stream;
+  if (kern == FA_KERNEL_TILE) {
+    const int rows = tile_rows(p, ns);
+    if (rows == 0) return FA_ERR_UNSUPPORTED;
+    if (rows == 256) return launch_tile256(a, p->dtype, st);
+  }
   return p->dtype == FA_DTYPE_BF16 ? dispatch<__bf16>(a, kern, st) : dispatch<_Float16>(a, kern, st);
 }
 
