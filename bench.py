@@ -300,34 +300,77 @@ def time_steps(call, steps, warmup, spin_up_s=0.4):
     return wall_ms / steps, float(np.mean(per)), float(np.median(per)), float(np.min(per))
 
 
-def cpu_baseline(budget_s=12.0):
-    """PyTorch's own CPU SDPA (aten::_scaled_dot_product_flash_attention_for_cpu, reached through the oracle package)
-    on a bounded sample of the headline workload: cfg2's shape with fewer (batch, head) pairs."""
-    import oracle
-
-    S, D = 4096, 128
-    threads = torch.get_num_threads()
-    heads = 4
-    q, k, v = (seeded((1, heads, S, D), 1 + i, torch.bfloat16) for i in range(3))
-    t = time.perf_counter()
-    oracle.cpu_sdpa_flash(q, k, v, is_causal=True)
-    first = time.perf_counter() - t
-    # scale the sample towards the time budget (at most the full 128 (batch, head) pairs of cfg2)
-    heads = int(max(4, min(128, 4 * (budget_s / 2) / max(first, 1e-3))))
-    q, k, v = (seeded((1, heads, S, D), 1 + i, torch.bfloat16) for i in range(3))
-    oracle.cpu_sdpa_flash(q, k, v, is_causal=True)  # warm-up
+def _timed_runs(fn, budget_s):
+    fn()  # warm-up
     runs = []
     t_all = time.perf_counter()
     while len(runs) < 2 or (time.perf_counter() - t_all < budget_s and len(runs) < 200):
         t = time.perf_counter()
-        oracle.cpu_sdpa_flash(q, k, v, is_causal=True)
+        fn()
         runs.append(time.perf_counter() - t)
-    sec = float(np.mean(runs))
-    flops = 4 * heads * S * S * D / 2
-    return {"value": flops / sec / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"PyTorch CPU SDPA (flash_attention_for_cpu), cfg2 shape, {heads} of 128 (batch, head) pairs, "
-                      f"bf16 causal S=4096 D=128, mean of {len(runs)} runs over {sum(runs):.1f} s ({sec:.2f} s each, "
-                      f"best {min(runs):.2f} s); os.cpu_count()={os.cpu_count()}"}
+    return runs
+
+
+def cpu_baseline(name="cfg2", budget_s=12.0):
+    """PyTorch's own CPU SDPA (reached through the oracle package) on the host cores, on a bounded sample of workload
+    `name`: cfg2 -> aten::_scaled_dot_product_flash_attention_for_cpu on fewer (batch, head) pairs; cfg3 / cfg5 ->
+    F.scaled_dot_product_attention(enable_gqa=True) on fewer sequences; cfg4 -> a loop over its 16 sequences."""
+    import oracle
+
+    bf, hf = torch.bfloat16, torch.float16
+    threads = torch.get_num_threads()
+    tail = f"; os.cpu_count()={os.cpu_count()}"
+    if name == "cfg2":
+        S, D = 4096, 128
+        heads = 4
+        q, k, v = (seeded((1, heads, S, D), 1 + i, bf) for i in range(3))
+        t = time.perf_counter()
+        oracle.cpu_sdpa_flash(q, k, v, is_causal=True)
+        first = time.perf_counter() - t
+        # scale the sample towards the time budget (at most the full 128 (batch, head) pairs of cfg2)
+        heads = int(max(4, min(128, 4 * (budget_s / 2) / max(first, 1e-3))))
+        q, k, v = (seeded((1, heads, S, D), 1 + i, bf) for i in range(3))
+        runs = _timed_runs(lambda: oracle.cpu_sdpa_flash(q, k, v, is_causal=True), budget_s)
+        sec = float(np.mean(runs))
+        return {"value": 4 * heads * S * S * D / 2 / sec / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": f"PyTorch CPU SDPA (flash_attention_for_cpu), cfg2 shape, {heads} of 128 (batch, head) pairs, "
+                          f"bf16 causal S=4096 D=128, mean of {len(runs)} runs over {sum(runs):.1f} s ({sec:.2f} s each, "
+                          f"best {min(runs):.2f} s)" + tail}
+    if name == "cfg3":
+        nb, Hq, Hk, S, D = 2, 32, 8, 2048, 128
+        q, k, v = seeded((nb, Hq, S, D), 2, bf), seeded((nb, Hk, S, D), 3, bf), seeded((nb, Hk, S, D), 4, bf)
+        runs = _timed_runs(lambda: oracle.cpu_sdpa(q, k, v, is_causal=True, enable_gqa=True), budget_s)
+        sec = float(np.mean(runs))
+        return {"value": 4 * nb * Hq * S * S * D / 2 / sec / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": f"PyTorch CPU F.scaled_dot_product_attention(enable_gqa=True), cfg3 shape, {nb} of 8 sequences, "
+                          f"bf16 causal Hq=32 Hkv=8 S=2048 D=128, mean of {len(runs)} runs over {sum(runs):.1f} s" + tail}
+    if name == "cfg4":
+        g = torch.Generator().manual_seed(3)
+        lens = torch.randint(256, 2049, (16,), generator=g).tolist()
+        H, D = 16, 128
+        seqs = [tuple(seeded((1, H, L, D), 30 + 3 * i + j, hf) for j in range(3)) for i, L in enumerate(lens)]
+
+        def loop():
+            for q, k, v in seqs:
+                oracle.cpu_sdpa(q, k, v, is_causal=True)
+
+        runs = _timed_runs(loop, budget_s)
+        sec = float(np.mean(runs))
+        return {"value": 4096.0 * sum(L * L for L in lens) / sec / 1e12, "unit": "TFLOP/s", "cores": threads,
+                "kind": "port",
+                "sample": f"PyTorch CPU F.scaled_dot_product_attention in a loop over cfg4's 16 sequences (all of them, "
+                          f"lengths as drawn), fp16 causal H=16 D=128, mean of {len(runs)} passes over {sum(runs):.1f} s"
+                          + tail}
+    if name == "cfg5":
+        nb, Hq, Hk, Sk, D = 8, 32, 8, 8192, 128
+        q, k, v = seeded((nb, Hq, 1, D), 4, bf), seeded((nb, Hk, Sk, D), 5, bf), seeded((nb, Hk, Sk, D), 6, bf)
+        runs = _timed_runs(lambda: oracle.cpu_sdpa(q, k, v, enable_gqa=True), budget_s)
+        sec = float(np.mean(runs))
+        return {"value": 2 * nb * Hk * Sk * D * 2 / sec / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": f"PyTorch CPU F.scaled_dot_product_attention(enable_gqa=True), cfg5 shape, {nb} of 64 sequences, "
+                          f"bf16 Hq=32 Hkv=8 Sq=1 Skv=8192 D=128 (bytes = K + V), mean of {len(runs)} runs over "
+                          f"{sum(runs):.1f} s" + tail}
+    return None
 
 
 def main():
@@ -420,7 +463,11 @@ def main():
             line["decode"] = {"value": dec[0]["kv_gbs"], "unit": "GB/s", "ms_per_step": dec[0]["ms_per_step"],
                               "roofline": dec[0]["roofline"]}
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline()
+        # the CPU legs run after every GPU measurement: the headline's own, then one per other BASELINE config
+        line["cpu_baseline"] = cpu_baseline(args.config if args.config in ("cfg2", "cfg3", "cfg4", "cfg5") else "cfg2")
+        for e in extras:
+            if e["config"] in ("cfg2", "cfg3", "cfg4", "cfg5"):
+                e["cpu_baseline"] = cpu_baseline(e["config"], budget_s=6.0)
     print(json.dumps(line))
 
 

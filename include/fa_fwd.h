@@ -49,8 +49,10 @@ extern "C" {
 #define FA_KERNEL_SPLITKV 2  /* HBM-bound split-KV kernel (+ merge): query rows x group heads share one pass over K/V */
 #define FA_KERNEL_TILE128 3  /* tile kernel with 128 query rows per workgroup, two workgroups per CU (every option) */
 #define FA_KERNEL_TILE256 4  /* tile kernel with 256 query rows per workgroup, one per CU, MFMA and softmax overlapped
-                                inside each wavefront: head_dim <= 128, no bias, no dropout, num_splits <= 1
+                                inside each wavefront (8 wavefronts of 32 rows, two per SIMD): head_dim <= 128, no
+                                bias, no dropout, num_splits <= 1, query / output row stride < 16 MiB
                                 (FA_ERR_UNSUPPORTED otherwise) */
+#define FA_KERNEL_TILE256W 5 /* the same with 4 wavefronts of 64 rows, one per SIMD */
 
 /*
  * One attention-forward problem:  for every sequence b and query head h
@@ -68,7 +70,8 @@ extern "C" {
  *   packed (cu_seqlens_q != NULL): sequence b owns rows [cu[b], cu[b+1]) of the packed [total, heads, head_dim]
  *          tensors; *_stride_b is ignored; seqlen_q / seqlen_k are upper bounds (max_seqlen) used to size the grid.
  *          cu_seqlens are int32 device arrays of batch+1 non-decreasing entries starting at 0 (:81-84,125-127) and
- *          are only ever read on the device.
+ *          are only ever read on the device.  A sequence longer than seqlen_q / seqlen_k says is not an error the
+ *          launcher can see: its rows beyond seqlen_q are left unwritten (never written elsewhere).
  * The sequence strides (x_stride_s) of K and V must stay below 32 MiB in bytes: the kernels address the rows of a tile
  * with a 32-bit offset (FA_ERR_UNSUPPORTED otherwise).
  * LSE element (b,h,s) is written at lse + b*lse_stride_b + h*lse_stride_h + s*lse_stride_s; in packed mode s is the
@@ -117,7 +120,10 @@ typedef struct fa_fwd_params {
 
   /* dropout on the softmax probabilities (tile kernel only; 0 = off).  The mask is a pure function of
      (philox_seed, philox_offset, sequence, query head, row, col), so the backward regenerates it from the two numbers. */
-  float dropout_p;         /* 0 <= p < 1 */
+  float dropout_p;         /* 0 <= p < 1.  An element is kept iff one byte of a hash word is <= floor((1 - p) 255), i.e.
+                              with probability (floor((1 - p) 255) + 1) / 256, and kept elements are scaled by
+                              1 / (1 - p) exactly as the reference's oracle scales them: the expectation of the output
+                              is off by at most 1 / (256 (1 - p)) relative (p = 0.1: 0.18 %) */
   int32_t reserved2;       /* must be 0 */
   uint64_t philox_seed;
   uint64_t philox_offset;
@@ -125,7 +131,8 @@ typedef struct fa_fwd_params {
   int64_t* rng_offset_out; /* device int64 or NULL */
   void* dropout_mask;      /* device or NULL: debug output, dense [batch][heads_q][seqlen_q][seqlen_k] elements of
                               `dtype`, +1 kept / -1 dropped, positions outside a sequence or masked left untouched
-                              (dense mode only) */
+                              (packed mode: seqlen_q / seqlen_k are the maxima, rows and keys count from each
+                              sequence's start, as FlashAttention_internal.cpp:141-146 shapes it) */
   /* optional (NULL = all of them): device int32[batch]; only the first min(seqused_k[b], its length) keys of sequence b
      exist — a KV cache that is allocated to seqlen_k rows but filled to a per-sequence length (the `seqused_k` of
      aten::_flash_attention_forward, the `seqlen_k` of aten::_efficient_attention_forward).  The causal mask aligns to

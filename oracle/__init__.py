@@ -6,6 +6,7 @@ cpu_baseline leg of bench.py use it, and only as the checker.
 from .attention_oracle import (  # noqa: F401
     attention_ref,
     construct_local_mask,
+    cpu_sdpa,
     cpu_sdpa_flash,
     default_atol,
     default_rtol,

@@ -284,3 +284,11 @@ def cpu_sdpa_flash(q, k, v, is_causal: bool = False, scale: Optional[float] = No
     out, lse = torch.ops.aten._scaled_dot_product_flash_attention_for_cpu(q, k, v, 0.0, is_causal, attn_mask=None,
                                                                          scale=scale)
     return out, lse
+
+
+def cpu_sdpa(q, k, v, is_causal: bool = False, enable_gqa: bool = False):
+    """PyTorch's CPU `F.scaled_dot_product_attention` on torch tensors [B, H, S, D] (K/V with fewer heads when
+    `enable_gqa`): the routine bench.py times on the host cores beside each GPU config."""
+    import torch
+
+    return torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=is_causal, enable_gqa=enable_gqa)

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_version_and_error_strings():
     L = capi.lib()
-    assert L.fa_fwd_version() == 4
+    assert L.fa_fwd_version() == capi.FA_FWD_ABI_VERSION == 5
     assert capi.error_string(0) == "ok"
     for rc in (-1, -2, -3, -99):
         assert capi.error_string(rc)
@@ -282,3 +282,91 @@ def test_bias_and_mask_mode_validation_and_plan():
     assert L.fa_fwd_plan(ctypes.byref(tl), ctypes.byref(kern), ctypes.byref(ns)) == 0 and kern.value == capi.FA_KERNEL_TILE
     tl.kernel = capi.FA_KERNEL_SPLITKV
     assert L.fa_fwd_validate(ctypes.byref(tl)) == capi.FA_ERR_UNSUPPORTED
+
+
+def _c_layout(header: str, struct: str, fields):
+    """sizeof and every offsetof of `struct`, as a C compiler lays it out from the header itself."""
+    import subprocess
+    import tempfile
+
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    src = "#include <stddef.h>\n#include <stdio.h>\n#include \"%s\"\nint main(void) {\n" % header
+    src += '  printf("%%zu\\n", sizeof(%s));\n' % struct
+    for f in fields:
+        src += '  printf("%s %%zu\\n", offsetof(%s, %s));\n' % (f, struct, f)
+    src += "  return 0;\n}\n"
+    with tempfile.TemporaryDirectory() as d:
+        c, exe = os.path.join(d, "layout.c"), os.path.join(d, "layout")
+        with open(c, "w") as fh:
+            fh.write(src)
+        subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", f"-I{inc}", c, "-o", exe], check=True)
+        out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split("\n")
+    return int(out[0]), {l.split()[0]: int(l.split()[1]) for l in out[1:] if l}
+
+
+@pytest.mark.parametrize("header,struct,mirror", [("fa_fwd.h", "fa_fwd_params", capi.FaFwdParams),
+                                                  ("fa_bwd.h", "fa_bwd_params", capi.FaBwdParams)])
+def test_ctypes_mirrors_match_the_headers(header, struct, mirror):
+    """The ctypes structures are kept in step with include/*.h by hand: a field added to a header without its mirror (or
+    the other way round, or in another order) must fail here, not read past the end of a short struct on the GPU."""
+    import re
+
+    names = [f[0] for f in mirror._fields_]
+    size, offs = _c_layout(header, struct, names)
+    assert ctypes.sizeof(mirror) == size
+    for n in names:
+        assert getattr(mirror, n).offset == offs[n], n
+    # and the header declares no field the mirror lacks
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", header)
+    text = open(inc).read()
+    body = text[text.index("typedef struct " + struct):text.index("} " + struct + ";")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    declared = []
+    for stmt in body.split("{", 1)[1].split(";"):
+        stmt = stmt.strip()
+        if not stmt:
+            continue
+        for part in stmt.split(","):
+            declared.append(re.findall(r"[A-Za-z_][A-Za-z_0-9]*", part)[-1])
+    assert declared == names
+
+
+def test_tile_rows_choice():
+    """fa_fwd_tile_rows: 128 or 256 rows per workgroup for the tile kernels, 0 for the split-KV kernel; an explicit
+    256-row request with an option those kernels lack is refused."""
+    L = capi.lib()
+    L.fa_fwd_tile_rows.restype = ctypes.c_int
+    L.fa_fwd_tile_rows.argtypes = [ctypes.POINTER(capi.FaFwdParams)]
+    p = _good()
+    assert L.fa_fwd_tile_rows(ctypes.byref(p)) in (128, 256)
+    for kern, rows in ((capi.FA_KERNEL_TILE128, 128), (capi.FA_KERNEL_TILE256, 256), (capi.FA_KERNEL_TILE256W, 256)):
+        p = _good(kernel=kern)
+        assert L.fa_fwd_tile_rows(ctypes.byref(p)) == rows
+        assert _plan(p)[:2] == (capi.FA_OK, capi.FA_KERNEL_TILE)
+    p = _good(kernel=capi.FA_KERNEL_TILE256, head_dim=256)
+    assert L.fa_fwd_tile_rows(ctypes.byref(p)) == capi.FA_ERR_UNSUPPORTED
+    p = _good(kernel=capi.FA_KERNEL_TILE256, dropout_p=0.5)
+    assert L.fa_fwd_tile_rows(ctypes.byref(p)) == capi.FA_ERR_UNSUPPORTED
+    p = _good(seqlen_q=1, seqlen_k=4096, heads_q=8, heads_k=8)
+    assert L.fa_fwd_tile_rows(ctypes.byref(p)) == 0
+
+
+def test_host_glue_is_clean_under_asan_and_ubsan():
+    """The host-only half of the launchers (validation, kernel choice, workspace sizes for both directions) built with
+    the address and undefined-behaviour sanitizers and pushed through ~2.5 million ordinary, extreme (INT32_MAX sizes,
+    INT64 strides) and malformed parameter blocks: any overflow or out-of-bounds access aborts the driver."""
+    import shutil
+    import subprocess
+    import tempfile
+
+    if shutil.which("g++") is None:
+        pytest.skip("no host C++ compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with tempfile.TemporaryDirectory() as d:
+        exe = os.path.join(d, "host_sanitize")
+        subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-static-libasan", "-fno-sanitize-recover=all", "-Wall",
+                        "-Werror", "-I" + os.path.join(root, "include"), "-I" + os.path.join(root, "torch_mlu_amd", "csrc"),
+                        os.path.join(root, "tests", "host_sanitize.cpp"), "-o", exe], check=True)
+        res = subprocess.run([exe], capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert re.match(r"\d+ blocks", res.stdout)

@@ -122,3 +122,22 @@ def test_config5_decode_bf16_gqa():
     assert (o_tile.float() - out[:4].float()).abs().max().item() <= 4e-3
     assert (l_tile - lse[:4]).abs().max().item() <= 1e-4
     print(f"cfg5 max|dout|={err:.3e} max|dlse|={lerr:.3e}")
+
+
+@pytest.mark.parametrize("dtype", [HF, BF])
+def test_config1_shape_through_the_hip_kernels(dtype):
+    """BASELINE config 1 is the reference's CPU-runnable fp32 case (B=2, H=8, Sq=Skv=512, D=64, non-causal, scale 1/8,
+    N(0, 1) inputs; pinned on the CPU in tests/test_oracle.py).  The HIP kernels take fp16 / bf16 only, so its shape
+    and input distribution go through them in both and are judged against the oracle on the same rounded inputs; the
+    unit-variance inputs make the scores five times larger than those of configs 2-5."""
+    q, k, v = (seeded((2, 8, 512, 64), s, dtype, std=1.0) for s in (0, 1, 2))
+    ro, rl = oracle.sdpa_oracle(q, k, v, scale=0.125)
+    n0 = torch_mlu_amd.launch_count()
+    r = torch.ops.aten._scaled_dot_product_flash_attention(q.to(DEV), k.to(DEV), v.to(DEV), 0.0, False, False, scale=0.125)
+    assert torch_mlu_amd.launch_count() == n0 + 1
+    out_close(r[0].float().cpu().numpy(), ro, dtype)
+    lse_close(r[1].cpu().numpy(), rl)
+    for kern in (capi.FA_KERNEL_TILE128, capi.FA_KERNEL_TILE256, capi.FA_KERNEL_TILE256W):
+        o, l = capi.fa_forward_dense(q.to(DEV), k.to(DEV), v.to(DEV), scale=0.125, kernel=kern)
+        out_close(o.float().cpu().numpy(), ro, dtype)
+        lse_close(l.cpu().numpy(), rl)

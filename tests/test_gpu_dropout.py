@@ -130,13 +130,19 @@ def test_packed_forward_and_backward_with_dropout():
     c = torch.from_numpy(cu).to(DEV)
     torch.manual_seed(7)
     out, lse, seed, offset, dbg = aten._flash_attention_forward(qd, kd, vd, c, c, max(lens), max(lens), p, True, True)
-    assert dbg.numel() == 0                                  # no debug mask in packed mode
+    # the debug mask of the packed call: [B, H, max_q, max_k] as the reference shapes it
+    # (FlashAttention_internal.cpp:141-146); +1 kept / -1 dropped inside each sequence's causal part, 0 elsewhere
+    assert tuple(dbg.shape) == (len(lens), Hq, max(lens), max(lens))
+    dbg_h = dbg.float().cpu().numpy()
     dq, dk, dv = aten._flash_attention_backward(dod, qd, kd, vd, out, lse, c, c, max(lens), max(lens), p, True, seed,
                                                 offset)
     sd, of = seed.item(), offset.item()
     for b, L in enumerate(lens):
         s = slice(int(cu[b]), int(cu[b + 1]))
         keep = np.stack([oracle.dropout_keep_mask(sd, of, b * Hq + h, L, L, p) for h in range(Hq)])[None]
+        vis = _visible(L, L, True)
+        assert (dbg_h[b, :, :L, :L] == np.where(vis, np.where(keep[0], 1.0, -1.0), 0.0)).all()
+        assert (dbg_h[b, :, L:, :] == 0).all() and (dbg_h[b, :, :, L:] == 0).all()
         args = [t[s].transpose(0, 1)[None] for t in (q, k, v)]
         ro, _ = oracle.sdpa_oracle(*args, is_causal=True, dropout_p=p, dropout_mask=keep)
         out_close(out[s].transpose(0, 1)[None].float().cpu().numpy(), ro, BF, tol=3e-2)

@@ -186,6 +186,67 @@ def test_dense_op_return_tuple_and_layout_contract():
     assert torch.equal(q, q2) and torch.equal(k, k2) and torch.equal(v, v2)
 
 
+def test_dense_op_cum_seq_after_inference_mode_and_across_streams():
+    """The dense op hands back cum_seq tensors from a per-(batch, length) cache.  A pair first built inside
+    torch.inference_mode() must be usable by a later training step of the same shape (autograd may save it: an inference
+    tensor there raises), and a second stream that asks for a freshly built pair must see its contents."""
+    B, H, D = 2, 4, 64
+    Sq = Sk = 88  # a length no other test in this file uses, so the cache entry is made here
+    q, k, v = (t.to(DEV) for t in _dense_inputs(B, H, H, Sq, Sk, D, HF, 720))
+    with torch.inference_mode():
+        r0 = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False)
+    assert r0[2].tolist() == [0, Sq, 2 * Sq] and r0[3].tolist() == [0, Sk, 2 * Sk]
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+    n0 = torch_mlu_amd.launch_count()
+    out = torch_mlu_amd.sdpa(qg, kg, vg, is_causal=True)
+    assert torch_mlu_amd.launch_count() == n0 + 1
+    out.float().square().sum().backward()
+    ref = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=True)
+    out_close(out.detach().float().cpu().numpy(), ref.cpu().numpy(), HF)
+    assert qg.grad is not None and torch.isfinite(qg.grad).all()
+    r1 = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False)
+    assert not r1[2].is_inference() and r1[2].tolist() == [0, Sq, 2 * Sq]
+    # a new pair requested on a side stream and read there
+    side = torch.cuda.Stream()
+    Sq2 = 104
+    q2 = q[:, :, :1].expand(B, H, Sq2, D).contiguous()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        r2 = torch.ops.aten._scaled_dot_product_flash_attention(q2, k, v, 0.0, False, False)
+        doubled = r2[2] * 2
+    side.synchronize()
+    assert doubled.tolist() == [0, 2 * Sq2, 4 * Sq2]
+    # and the same pair asked for from the default stream afterwards
+    r3 = torch.ops.aten._scaled_dot_product_flash_attention(q2, k, v, 0.0, False, False)
+    assert (r3[2] + 1).tolist() == [1, Sq2 + 1, 2 * Sq2 + 1]
+
+
+def test_dense_op_many_lengths_never_blocks_the_host():
+    """Several hundred distinct (batch, length) pairs, more than the cum_seq cache holds: every pair is right (evicted
+    entries are rebuilt), and the host is never made to wait for the device: with a long kernel queued first, issuing
+    the whole series returns while that kernel still runs."""
+    B, H, D = 1, 1, 64
+    k = torch.randn(B, H, 64, D, device=DEV, dtype=HF)
+    big = torch.randn(8192, 8192, device=DEV)
+    torch.cuda.synchronize()
+    done = torch.cuda.Event()
+    for _ in range(20):
+        big = (big @ big).clamp_(-1, 1)    # tens of milliseconds of queued device work
+    done.record()
+    results = []
+    for S in range(8, 8 + 8 * 300, 8):     # 300 new lengths > the cache's 256 entries
+        q = k[:, :, :1].expand(B, H, S, D)
+        r = torch.ops.aten._scaled_dot_product_flash_attention(q.contiguous(), k, k, 0.0, False, False)
+        results.append((S, r[2]))
+    still_running = not done.query()
+    torch.cuda.synchronize()
+    assert still_running, "issuing the series waited for the device"
+    for S, cq in results:
+        assert cq.tolist() == [0, S]
+    r = torch.ops.aten._scaled_dot_product_flash_attention(k[:, :, :8].contiguous(), k, k, 0.0, False, False)
+    assert r[2].tolist() == [0, 8]         # evicted long ago, rebuilt
+
+
 def test_sdpa_drop_in_default_scale_gqa_and_autocast():
     q, k, v = _dense_inputs(2, 8, 2, 96, 96, 128, BF, 710)
     qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)

@@ -236,14 +236,24 @@ def test_split_merge_identity():
     assert np.allclose(M + np.log(w.sum(axis=0)), lse, atol=1e-12)
 
 
-def test_tolerance_rule_restatement():
-    t = np.array([1.0, 2.0, 0.0])
-    c = np.array([1.001, 2.0, 0.0])
-    atol, rtol = oracle.get_tolerances(t, c, "bfloat16")
-    assert math.isclose(atol, 2 * 1e-3 * 1.0, rel_tol=1e-6) or atol >= 2e-3
-    assert math.isclose(rtol, 2 * 1.6e-2)
-    atol, rtol = oracle.get_tolerances(t, t + 0.5, "float16", fudge_factor=None)
-    assert math.isclose(atol, 0.5)
+@pytest.mark.parametrize("true,computed,dtype,fudge,want", [
+    # worked by hand from test_scaled_dot_product_attention.py:166-204 (atol = fudge * max(max|t - c|, default_atol),
+    # rtol = fudge * max(max|(t - c) / t| with 0/0 -> default_rtol, default_rtol), rtol > 1e30 -> default_rtol):
+    # |dev| = (0.000999.., 0, 0) < 1e-3 -> atol 2 * 1e-3; rel = (0.000999.., 0, 0/0 -> 1.6e-2) -> rtol 2 * 1.6e-2
+    ([1.0, 2.0, 0.0], [1.001, 2.0, 0.0], "bfloat16", 2.0, (2e-3, 3.2e-2)),
+    # no fudge factor (None = 1): |dev| = (0.5, 0) -> atol 0.5; rel = (0.125, 0) -> rtol 0.125
+    ([4.0, -2.0], [4.5, -2.0], "float16", None, (0.5, 0.125)),
+    # a true value of 0 with a non-zero computed one: rel = inf -> 2 inf > 1e30 -> rtol falls back to the default
+    ([0.0], [0.25], "float16", 2.0, (0.5, 1e-3)),
+    # fudge 4 (the reference's query_fudge_factor, :1079): |dev| = (0.5, 1) -> atol 4; rel = (0.05, 0.05) -> rtol 0.2
+    ([10.0, 20.0], [10.5, 19.0], "bfloat16", 4.0, (4.0, 0.2)),
+    # identical tensors: the defaults times the fudge factor
+    ([1.0], [1.0], "float32", 2.0, (2e-5, 2.6e-6)),
+])
+def test_tolerance_rule_restatement(true, computed, dtype, fudge, want):
+    atol, rtol = oracle.get_tolerances(np.array(true), np.array(computed), dtype, fudge_factor=fudge)
+    assert math.isclose(atol, want[0], rel_tol=1e-9)
+    assert math.isclose(rtol, want[1], rel_tol=1e-9)
 
 
 # ---- additive bias and top-left causal (mem-efficient entry points) ----------------------------------------------

@@ -36,26 +36,32 @@ def _run(cmd, **kw):
 
 
 def check_tile256_registers(asm_text: str) -> None:
-    """fa_fwd_tile256.hip assigns the accumulation registers a64 .. a255 by hand inside inline assembly.  The compiler
-    may use accumulation registers of its own (it takes them from a0 upwards); one at or above a64 outside the assembly
-    statements would silently corrupt the O accumulators or the Q fragments, so such a build is refused."""
+    """fa_fwd_tile256.hip assigns accumulation registers by hand inside inline assembly: a64 .. a255 in the kernels with
+    two 32-row halves per wavefront (last template argument 2), a32 .. a127 in those with one.  The compiler may use
+    accumulation registers of its own (it takes them from a0 upwards); one inside the hand-assigned range outside the
+    assembly statements would silently corrupt the O accumulators or the Q fragments, and vector registers that
+    spill to scratch memory would ruin the kernel's speed, so such a build is refused."""
     import re
 
     in_asm = False
+    first_own = None  # first hand-assigned register of the kernel being read
     for line in asm_text.splitlines():
         t = line.strip()
+        m = re.match(r"^_ZN2fa.*fa_tile256_kernel\w*Li(\d+)EEEvNS_5KArgsE:", line)
+        if m:
+            first_own = 64 if m.group(1) == "2" else 32
+        elif line.startswith(".Lfunc_end"):
+            first_own = None
         if t.startswith(";;#ASMSTART"):
             in_asm = True
         elif t.startswith(";;#ASMEND"):
             in_asm = False
-        elif not in_asm and t and not t.startswith((";", ".")):
+        elif first_own is not None and not in_asm and t and not t.startswith((";", ".")):
             code = t.split(";")[0]
             for m in re.finditer(r"\ba(\d+)\b|\ba\[(\d+):(\d+)\]", code):
                 hi = int(m.group(1) if m.group(1) is not None else m.group(3))
-                if hi >= 64:
+                if hi >= first_own:
                     raise RuntimeError("fa_fwd_tile256: the compiler allocated a hand-assigned accumulation register: " + t)
-        if "ScratchSize:" in t and "fa_tile256" not in t:
-            pass
     for m in re.finditer(r"; ScratchSize: (\d+)", asm_text):
         if int(m.group(1)) != 0:
             raise RuntimeError("fa_fwd_tile256: vector registers spill to scratch memory")

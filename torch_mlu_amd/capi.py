@@ -21,6 +21,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libfa_fwd.so")
 
+FA_FWD_ABI_VERSION = 5
 FA_DTYPE_FP16 = 0
 FA_DTYPE_BF16 = 1
 FA_OK = 0
@@ -33,6 +34,7 @@ FA_KERNEL_TILE = 1
 FA_KERNEL_SPLITKV = 2
 FA_KERNEL_TILE128 = 3
 FA_KERNEL_TILE256 = 4
+FA_KERNEL_TILE256W = 5
 FA_MAX_SPLITS = 64
 
 # every symbol include/fa_fwd.h declares

@@ -240,7 +240,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> flash_att
     p.dropout_p = static_cast<float>(dropout_p);
     p.rng_seed_out = seed_t.data_ptr<int64_t>();
     p.rng_offset_out = offset_t.data_ptr<int64_t>();
-    if (return_debug_mask && !packed) {
+    if (return_debug_mask) {
       // [B, H, max_q, max_k], > 0 where kept (the reference: zeros filled by the kernel, :141-146; its tests use
       // `mask > 0`, test_scaled_dot_product_attention.py:1049-1050)
       debug_attn_mask = at::zeros({batch, heads, seqlen_q, seqlen_k}, q.options());

@@ -23,6 +23,7 @@
 
 #include "fa_bwd.h"
 #include "fa_device.h"
+#include "fa_host.h"
 
 // ring depths of the two operand prefetch loops of the dK/dV kernel, by what the instantiation computes
 // ring depths of the two operand prefetch loops of the dQ kernel
@@ -1022,66 +1023,10 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
 // ---------------------------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------------------------
-constexpr int64_t kMaxRowStrideBytes = 0xffffffffLL / 128;  // 128 rows x stride must fit an unsigned 32-bit offset
-
-int bwd_validate(const fa_bwd_params* p) {
-  if (!p) return FA_ERR_BAD_ARG;
-  if (!p->q || !p->k || !p->v || !p->out || !p->dout || !p->lse || !p->dq || !p->dk || !p->dv) return FA_ERR_BAD_ARG;
-  if ((p->cu_seqlens_q == nullptr) != (p->cu_seqlens_k == nullptr)) return FA_ERR_BAD_ARG;
-  if (p->batch <= 0 || p->heads_q <= 0 || p->heads_k <= 0) return FA_ERR_BAD_ARG;
-  if (p->seqlen_q < 0 || p->seqlen_k < 0 || p->head_dim <= 0) return FA_ERR_BAD_ARG;
-  if (p->reserved != 0 || p->reserved2 != 0) return FA_ERR_BAD_ARG;
-  if (!(p->dropout_p >= 0.f && p->dropout_p < 1.f)) return FA_ERR_BAD_ARG;
-  if (p->dropout_p > 0.f && (!p->philox_seed || !p->philox_offset ||
-                             (((uintptr_t)p->philox_seed | (uintptr_t)p->philox_offset) & 7)))
-    return FA_ERR_BAD_ARG;
-  if (p->cu_seqlens_q && p->total_q < 0) return FA_ERR_BAD_ARG;
-  if (p->is_causal != FA_MASK_NONE && p->is_causal != FA_MASK_CAUSAL_BOTTOM_RIGHT && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT)
-    return FA_ERR_BAD_ARG;
-  if (p->dbias && !p->bias) return FA_ERR_BAD_ARG;
-  if (p->bias) {
-    if (((uintptr_t)p->bias & 7) || p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_q < 0 ||
-        ((p->bias_stride_b | p->bias_stride_h | p->bias_stride_q) & 3))
-      return FA_ERR_BAD_ARG;
-  }
-  if (p->dbias) {  // an output: aligned like the bias and not broadcast
-    if (((uintptr_t)p->dbias & 7) || ((p->dbias_stride_b | p->dbias_stride_h | p->dbias_stride_q) & 3)) return FA_ERR_BAD_ARG;
-    if (p->dbias_stride_q < p->seqlen_k || (p->seqlen_q > 1 && p->dbias_stride_q <= 0) ||
-        (p->heads_q > 1 && p->dbias_stride_h <= 0) || (p->batch > 1 && p->dbias_stride_b <= 0))
-      return FA_ERR_BAD_ARG;
-  }
-  if (p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_UNSUPPORTED;
-  if (p->head_dim > 256 || (p->head_dim & 7)) return FA_ERR_UNSUPPORTED;
-  if (p->heads_q % p->heads_k) return FA_ERR_UNSUPPORTED;
-  const uintptr_t al = (uintptr_t)p->q | (uintptr_t)p->k | (uintptr_t)p->v | (uintptr_t)p->out | (uintptr_t)p->dout |
-                       (uintptr_t)p->dq | (uintptr_t)p->dk | (uintptr_t)p->dv;
-  if (al & 15) return FA_ERR_BAD_ARG;
-  if ((uintptr_t)p->lse & 3) return FA_ERR_BAD_ARG;
-  const int64_t st[] = {p->q_stride_s,  p->q_stride_h,  p->k_stride_s,  p->k_stride_h,  p->v_stride_s,  p->v_stride_h,
-                        p->o_stride_s,  p->o_stride_h,  p->do_stride_s, p->do_stride_h, p->dq_stride_s, p->dq_stride_h,
-                        p->dk_stride_s, p->dk_stride_h, p->dv_stride_s, p->dv_stride_h};
-  for (int64_t s : st)
-    if (s < 0 || (s & 7)) return FA_ERR_BAD_ARG;
-  if (!p->cu_seqlens_q) {
-    const int64_t sb[] = {p->q_stride_b,  p->k_stride_b,  p->v_stride_b,  p->o_stride_b,
-                          p->do_stride_b, p->dq_stride_b, p->dk_stride_b, p->dv_stride_b};
-    for (int64_t s : sb)
-      if (s < 0 || (s & 7)) return FA_ERR_BAD_ARG;
-  }
-  if (p->lse_stride_h < 0 || p->lse_stride_s < 0) return FA_ERR_BAD_ARG;
-  // per-lane byte offsets inside a tile (up to 128 rows) are 32-bit row x 32-bit stride
-  if (p->k_stride_s * 2 > kMaxRowStrideBytes || p->v_stride_s * 2 > kMaxRowStrideBytes ||
-      p->q_stride_s * 2 > kMaxRowStrideBytes || p->do_stride_s * 2 > kMaxRowStrideBytes)
-    return FA_ERR_UNSUPPORTED;
-  return FA_OK;
-}
-
-// two fp32 planes per (row, head): -delta and LSE log2(e)
-size_t bwd_ws_plane(const fa_bwd_params* p) {
-  const size_t rows = p->cu_seqlens_q ? (size_t)p->total_q : (size_t)p->batch * p->seqlen_q;
-  return (rows * p->heads_q * 4 + 15) & ~(size_t)15;
-}
-size_t bwd_ws_bytes(const fa_bwd_params* p) { return 2 * bwd_ws_plane(p); }
+constexpr int64_t kMaxRowStrideBytes = fa::host::kMaxRowStrideBytes;
+using fa::host::bwd_validate;
+using fa::host::bwd_ws_bytes;
+using fa::host::bwd_ws_plane;
 
 template <typename T, int DP, bool DROP, bool BIAS>
 int bwd_launch(const BArgs& a, hipStream_t st) {

@@ -71,10 +71,11 @@ __device__ __forceinline__ int swzV(int row) {
 constexpr float kLazyLog2 = 8.0f;
 
 
-// The 256-row tile kernel (fa_fwd_tile256.hip): one workgroup owns 256 query rows, each wavefront 64 of them.
+// The 256-row tile kernels (fa_fwd_tile256.hip): one workgroup owns 256 query rows; `halves` = 32-row halves per
+// wavefront: 1 (8 wavefronts, two per SIMD) or 2 (4 wavefronts, one per SIMD).
 // Eligible problems: head_dim padded to 64 or 128, no bias, no dropout, not sliced.  Returns an FA_* code.
 bool tile256_eligible(const KArgs& a);
-int launch_tile256(const KArgs& a, int dtype, hipStream_t st);
+int launch_tile256(const KArgs& a, int dtype, int halves, hipStream_t st);
 
 }  // namespace fa
 

@@ -230,24 +230,11 @@ SDPBackend select_sdp_backend(const sdp_params& p, std::optional<double> scale) 
   // order (sdp_utils.cpp:9-12)
   if (use_flash_attention(p, /*debug=*/false)) return SDPBackend::flash_attention;
   if (use_mem_efficient_attention(p, /*debug=*/false)) return SDPBackend::efficient_attention;
-  // Not eligible here: PyTorch's own selector decides among what is left.  Its flash and mem-efficient choices would
-  // land on this build's registered ops again, so both are masked out while it looks.
-  if (ctx.userEnabledMathSDP() || ctx.userEnabledCuDNNSDP()) {
-    struct Restore {
-      at::Context& c;
-      bool flash, mem;
-      ~Restore() {
-        c.setSDPUseFlash(flash);
-        c.setSDPUseMemEfficient(mem);
-      }
-    } restore{ctx, ctx.userEnabledFlashSDP(), ctx.userEnabledMemEfficientSDP()};
-    ctx.setSDPUseFlash(false);
-    ctx.setSDPUseMemEfficient(false);
-    const at::AutoDispatchBelowAutograd below;  // skip this file's own registration of the op, reach PyTorch's
-    const int64_t choice = at::_fused_sdp_choice(p.query, p.key, p.value, p.attn_mask, p.dropout, p.is_causal, scale,
-                                                 p.enable_gqa);
-    return static_cast<SDPBackend>(choice);
-  }
+  // Not eligible here.  Of PyTorch's own backends only the math one is left for HIP tensors: its flash and
+  // mem-efficient choices would land on this build's registered ops again, and the cuDNN backend does not exist in a
+  // ROCm build.  The choice is made here, from the flags as they are: nothing process-wide is changed while another
+  // host thread may be selecting a backend too.
+  if (ctx.userEnabledMathSDP()) return SDPBackend::math;
   // Only fused kernels are enabled and they cannot take these inputs: say why, as the reference does
   // (sdp_utils.cpp:135-146).
   TORCH_WARN("Memory efficient kernel not used because:");
