@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FA_FWD_ABI_VERSION 5
+#define FA_FWD_ABI_VERSION 6
 
 /* element types accepted for q/k/v/out (FlashAttention_internal.cpp:73-80 allows exactly these two) */
 #define FA_DTYPE_FP16 0
@@ -35,6 +35,7 @@ extern "C" {
 #define FA_ERR_BAD_ARG (-1)     /* null pointer, non-positive size, misaligned pointer/stride, short workspace */
 #define FA_ERR_UNSUPPORTED (-2) /* shape or dtype outside the supported envelope */
 #define FA_ERR_LAUNCH (-3)      /* the HIP runtime refused the launch (hipGetLastError != hipSuccess) */
+#define FA_ERR_WORKSPACE (-4)   /* fa_fwd_launch_static only: the plan needs more than FA_STATIC_WORKSPACE_BYTES */
 
 /* is_causal values */
 #define FA_MASK_NONE 0
@@ -167,6 +168,21 @@ size_t fa_fwd_workspace_bytes(const fa_fwd_params* p);
  * synchronises, never throws.  Returns FA_OK or a negative code (nothing is enqueued on error).
  */
 int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * fa_fwd_launch for callers that cannot allocate device memory or pass a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels and results
+ * as fa_fwd_launch; the per-slice partials go to a fixed array of FA_STATIC_WORKSPACE_BYTES bytes of device memory
+ * that is part of the library's code object, so each device the library runs on holds that much until the process
+ * ends.  Calls no allocating routine.  The first call on a device that needs scratch looks the array's device address
+ * up (make that call outside graph capture).  Returns FA_ERR_WORKSPACE, with nothing enqueued, when
+ * fa_fwd_workspace_bytes(p) exceeds FA_STATIC_WORKSPACE_BYTES.  All calls on one device share the one array: two
+ * launches that both need scratch must not overlap on that device (issue them on one stream, or order the streams
+ * with events); calls whose fa_fwd_workspace_bytes(p) is 0 never touch it.  Nothing in the array needs clearing
+ * between calls: every slot a launch reads it has written first.
+ */
+#define FA_STATIC_WORKSPACE_BYTES (64u << 20)
+int fa_fwd_launch_static(const fa_fwd_params* p, void* stream);
 
 /*
  * Which kernel fa_fwd_launch would run for `p` (FA_KERNEL_TILE / FA_KERNEL_SPLITKV) and with how many splits;

@@ -21,13 +21,15 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libfa_fwd.so")
 
-FA_FWD_ABI_VERSION = 5
+FA_FWD_ABI_VERSION = 6
 FA_DTYPE_FP16 = 0
 FA_DTYPE_BF16 = 1
 FA_OK = 0
 FA_ERR_BAD_ARG = -1
 FA_ERR_UNSUPPORTED = -2
 FA_ERR_LAUNCH = -3
+FA_ERR_WORKSPACE = -4
+FA_STATIC_WORKSPACE_BYTES = 64 << 20
 FA_MASK_NONE, FA_MASK_CAUSAL_BOTTOM_RIGHT, FA_MASK_CAUSAL_TOP_LEFT = 0, 1, 2
 FA_KERNEL_AUTO = 0
 FA_KERNEL_TILE = 1
@@ -44,6 +46,7 @@ EXPORTED_SYMBOLS = (
     "fa_fwd_validate",
     "fa_fwd_workspace_bytes",
     "fa_fwd_launch",
+    "fa_fwd_launch_static",
     "fa_fwd_plan",
     "fa_fwd_tile_rows",
     "fa_bwd_validate",
@@ -133,6 +136,8 @@ def lib() -> ctypes.CDLL:
         L.fa_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FaFwdParams)]
         L.fa_fwd_launch.restype = ctypes.c_int
         L.fa_fwd_launch.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        L.fa_fwd_launch_static.restype = ctypes.c_int
+        L.fa_fwd_launch_static.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.c_void_p]
         L.fa_fwd_plan.restype = ctypes.c_int
         L.fa_fwd_plan.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.POINTER(ctypes.c_int32),
                                   ctypes.POINTER(ctypes.c_int32)]

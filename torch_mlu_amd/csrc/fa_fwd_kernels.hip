@@ -24,6 +24,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "fa_device.h"
 #include "fa_fwd.h"
 #include "fa_fwd_common.h"
@@ -1012,6 +1014,7 @@ const char* fa_fwd_error_string(int rc) {
     case FA_ERR_BAD_ARG: return "bad argument (null pointer, non-positive size, misaligned pointer or stride, short workspace)";
     case FA_ERR_UNSUPPORTED: return "unsupported shape or dtype";
     case FA_ERR_LAUNCH: return "HIP launch failure";
+    case FA_ERR_WORKSPACE: return "the plan needs more scratch than fa_fwd_launch_static holds (FA_STATIC_WORKSPACE_BYTES); use fa_fwd_launch with a workspace";
     default: return "unknown error";
   }
 }
@@ -1043,6 +1046,49 @@ size_t fa_fwd_workspace_bytes(const fa_fwd_params* p) {
   int k, s;
   plan(p, &k, &s);
   return workspace_bytes(p, k, s);
+}
+
+}  // extern "C"
+
+// Scratch of fa_fwd_launch_static: the per-slice partials of the split-KV and sliced tile kernels, in device memory
+// that belongs to the code object (present on every device the library is loaded on, for the life of the process).
+// The name below is a host-side handle only; the device address is looked up once per device.
+static __device__ __align__(256) unsigned char scratch[FA_STATIC_WORKSPACE_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device; nullptr when the runtime cannot give one.
+void* static_scratch() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr) return ptr;
+  if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // every thread gets the same answer, so a race is harmless
+  return ptr;
+}
+}  // namespace
+
+extern "C" {
+
+int fa_fwd_launch_static(const fa_fwd_params* p, void* stream) {
+  const int rc = validate(p);
+  if (rc != FA_OK) return rc;
+  int kern, ns;
+  plan(p, &kern, &ns);
+  const size_t need = workspace_bytes(p, kern, ns);
+  if (need > (size_t)FA_STATIC_WORKSPACE_BYTES) return FA_ERR_WORKSPACE;
+  void* ws = nullptr;
+  if (need > 0) {
+    ws = static_scratch();
+    if (!ws) return FA_ERR_LAUNCH;
+  }
+  return fa_fwd_launch(p, ws, need > 0 ? (size_t)FA_STATIC_WORKSPACE_BYTES : 0, stream);
 }
 
 int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_bytes_given, void* stream) {
