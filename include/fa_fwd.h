@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FA_FWD_ABI_VERSION 6
+#define FA_FWD_ABI_VERSION 7
 
 /* element types accepted for q/k/v/out (FlashAttention_internal.cpp:73-80 allows exactly these two) */
 #define FA_DTYPE_FP16 0
@@ -139,6 +139,13 @@ typedef struct fa_fwd_params {
      aten::_flash_attention_forward, the `seqlen_k` of aten::_efficient_attention_forward).  The causal mask aligns to
      the used length.  Forward only: the backward has no such argument. */
   const int32_t* seqused_k;
+  /* optional (NULL = philox_seed / philox_offset above are the numbers): device int64 each.  When given, the kernel
+     reads the seed from *philox_seed_ptr and adds *philox_offset_ptr to philox_offset when it RUNS, so a launch
+     recorded into a HIP graph draws a new mask on every replay from a generator state the host advances between
+     replays (the capture-aware generator of the reference, framework/generator/generator_impl.cpp:264-292).
+     rng_seed_out / rng_offset_out receive the resolved numbers. */
+  const int64_t* philox_seed_ptr;
+  const int64_t* philox_offset_ptr;
 } fa_fwd_params;
 
 #define FA_MAX_SPLITS 64

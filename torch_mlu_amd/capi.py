@@ -21,7 +21,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libfa_fwd.so")
 
-FA_FWD_ABI_VERSION = 6
+FA_FWD_ABI_VERSION = 7
 FA_DTYPE_FP16 = 0
 FA_DTYPE_BF16 = 1
 FA_OK = 0
@@ -93,6 +93,8 @@ class FaFwdParams(ctypes.Structure):
         ("rng_offset_out", ctypes.c_void_p),
         ("dropout_mask", ctypes.c_void_p),
         ("seqused_k", ctypes.c_void_p),
+        ("philox_seed_ptr", ctypes.c_void_p),
+        ("philox_offset_ptr", ctypes.c_void_p),
     ]
 
 
@@ -175,7 +177,8 @@ def make_params(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Te
                 is_causal=False, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
                 bias: Optional[torch.Tensor] = None, dropout_p: float = 0.0, philox_seed: int = 0,
                 philox_offset: int = 0, rng_out: Optional[torch.Tensor] = None,
-                dropout_mask: Optional[torch.Tensor] = None, seqused_k: Optional[torch.Tensor] = None) -> FaFwdParams:
+                dropout_mask: Optional[torch.Tensor] = None, seqused_k: Optional[torch.Tensor] = None,
+                philox_state: Optional[torch.Tensor] = None) -> FaFwdParams:
     """Fill a params struct.  `is_causal`: False / True (bottom-right aligned) or one of the FA_MASK_* codes; `bias`:
     a [B, Hq, Sq, Sk] view (dense mode; stride 0 where broadcast) of the inputs' dtype.
 
@@ -227,6 +230,9 @@ def make_params(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Te
     p.rng_offset_out = rng_out[1:].data_ptr() if rng_out is not None else None
     p.dropout_mask = dropout_mask.data_ptr() if dropout_mask is not None else None
     p.seqused_k = seqused_k.data_ptr() if seqused_k is not None else None
+    # int64[2] on the device: (seed, offset base) read by the kernel when it runs; philox_offset is added to the base
+    p.philox_seed_ptr = philox_state[0:].data_ptr() if philox_state is not None else None
+    p.philox_offset_ptr = philox_state[1:].data_ptr() if philox_state is not None else None
     return p
 
 
@@ -245,8 +251,8 @@ def fa_forward_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, is_ca
                      scale: Optional[float] = None, kernel: int = FA_KERNEL_AUTO, num_splits: int = 0,
                      bias: Optional[torch.Tensor] = None, dropout_p: float = 0.0, philox_seed: int = 0,
                      philox_offset: int = 0, rng_out: Optional[torch.Tensor] = None,
-                     dropout_mask: Optional[torch.Tensor] = None, seqused_k: Optional[torch.Tensor] = None
-                     ) -> Tuple[torch.Tensor, torch.Tensor]:
+                     dropout_mask: Optional[torch.Tensor] = None, seqused_k: Optional[torch.Tensor] = None,
+                     philox_state: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """q [B, Hq, Sq, D], k/v [B, Hk, Sk, D] (any strides, contiguous last dim) -> out [B, Hq, Sq, D] (stored
     [B, Sq, Hq, D] like the reference's dense wrapper, attention.cpp:146-148), lse [B, Hq, Sq] fp32.
     `bias`: anything that expands to [B, Hq, Sq, Sk]; `is_causal` may also be FA_MASK_CAUSAL_TOP_LEFT.
@@ -261,7 +267,7 @@ def fa_forward_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, is_ca
     p = make_params(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), out, lse, scale=scale,
                     is_causal=is_causal, kernel=kernel, num_splits=num_splits, bias=bias, dropout_p=dropout_p,
                     philox_seed=philox_seed, philox_offset=philox_offset, rng_out=rng_out, dropout_mask=dropout_mask,
-                    seqused_k=seqused_k)
+                    seqused_k=seqused_k, philox_state=philox_state)
     launch(p, q.device)
     return out.transpose(1, 2), lse
 

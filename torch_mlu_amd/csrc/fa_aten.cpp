@@ -148,15 +148,24 @@ static at::Tensor checked_seqused_k(const at::Tensor& t, int64_t batch, const at
   return t.contiguous();
 }
 
-static void take_philox_state(int64_t seqlen_q, int64_t seqlen_k, uint64_t& seed, uint64_t& offset) {
-  TORCH_CHECK(c10::hip::currentStreamCaptureStatusMayInitCtx() == c10::hip::CaptureStatus::None,
-              "attention forward: dropout under graph capture is not supported by this build");
+// The generator's Philox state, advanced under its mutex (FlashAttention_internal.cpp:198-210).  Outside graph
+// capture the two numbers are known here; during capture the generator hands out device pointers that it refills
+// before every replay (the reference's generator does the same, framework/generator/generator_impl.cpp:264-292), and
+// the kernel reads them when it runs: seed = *seed_ptr, offset = *offset_ptr + the intra-graph offset.
+static void take_philox_state(int64_t seqlen_q, int64_t seqlen_k, fa_fwd_params& p) {
   auto* gen = at::get_generator_or_default<at::CUDAGeneratorImpl>(std::nullopt, at::cuda::detail::getDefaultCUDAGenerator());
   std::lock_guard<std::mutex> lock(gen->mutex_);
   const uint64_t increment = 4 * static_cast<uint64_t>((seqlen_q * seqlen_k + 1023) / 1024 + 1);
   const at::PhiloxCudaState st = gen->philox_cuda_state(increment);
-  seed = st.seed_.val;
-  offset = st.offset_.val;
+  if (st.captured_) {
+    p.philox_seed = 0;
+    p.philox_offset = st.offset_intragraph_;
+    p.philox_seed_ptr = st.seed_.ptr;
+    p.philox_offset_ptr = st.offset_.ptr;
+  } else {
+    p.philox_seed = st.seed_.val;
+    p.philox_offset = st.offset_.val;
+  }
 }
 
 // ---- _flash_attention_forward ---------------------------------------------------------------------------------
@@ -236,7 +245,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> flash_att
   at::Tensor offset_t = at::empty({}, q.options().dtype(at::kLong));
   at::Tensor debug_attn_mask = at::empty({0}, q.options());
   if (dropout_p > 0.0) {
-    take_philox_state(seqlen_q, seqlen_k, p.philox_seed, p.philox_offset);
+    take_philox_state(seqlen_q, seqlen_k, p);
     p.dropout_p = static_cast<float>(dropout_p);
     p.rng_seed_out = seed_t.data_ptr<int64_t>();
     p.rng_offset_out = offset_t.data_ptr<int64_t>();
@@ -632,7 +641,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   at::Tensor seed_t = at::empty({}, q.options().dtype(at::kLong));
   at::Tensor offset_t = at::empty({}, q.options().dtype(at::kLong));
   if (dropout_p > 0.0) {
-    take_philox_state(Sq, Sk, p.philox_seed, p.philox_offset);
+    take_philox_state(Sq, Sk, p);
     p.dropout_p = static_cast<float>(dropout_p);
     p.rng_seed_out = seed_t.data_ptr<int64_t>();
     p.rng_offset_out = offset_t.data_ptr<int64_t>();

@@ -40,6 +40,8 @@ struct KArgs {
   uint32_t drop_thr;  // dropout: an element is kept iff its byte <= drop_thr
   float drop_rp;      // 1 / (1 - p)
   uint64_t seed, offset;
+  const int64_t* seed_ptr;    // optional: the seed is *seed_ptr and *offset_ptr is added to offset (graph capture)
+  const int64_t* offset_ptr;
   int64_t* rng_seed_out;
   int64_t* rng_offset_out;
   unsigned char* dmask;  // debug mask [batch][heads_q][seqlen_q][seqlen_k] elements, or null

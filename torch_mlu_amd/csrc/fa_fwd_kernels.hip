@@ -80,7 +80,35 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   // `split` of n_splits takes a contiguous range of a block's tiles and leaves unnormalised partials (m, l, O) in
   // the workspace, which fa_merge_rows_kernel combines.
   int split = 0;
-  if (a.cu_q) {
+  int pk_blk = -1;  // packed, paired: the heavy block of this workgroup's pair
+  if (a.cu_q && a.pair) {
+    // Packed and causal, lengths known only here: every workgroup finds its own work.  A sequence of n blocks is cut
+    // into the pairs (i, n-1-i), n-1 >= i >= (n-1)/2, which all cost the same; the pairs of all sequences are ordered
+    // by i, largest first (so the pairs of the longest sequences run first and the short ones fill the end), then by
+    // sequence, and workgroup number `item` takes pair number `item` of that order.  One lane per sequence (at most
+    // 64, checked by the launcher) votes "I have a pair with this i"; the workgroups beyond the last pair are the
+    // last ones of the grid and exit.
+    const int item = lid / a.heads_q;
+    bh = -1;
+    int nb = 0;
+    if (lane < a.batch) nb = (a.cu_q[lane + 1] - a.cu_q[lane] + BM - 1) / BM;
+    int left = item;
+    for (int i = a.n_mblk - 1; i >= 0; --i) {
+      const bool mine = i < nb && 2 * i >= nb - 1;
+      const uint64_t votes = __builtin_amdgcn_ballot_w64(mine);
+      const int cnt = __builtin_popcountll(votes);
+      if (left < cnt) {
+        const int before = __builtin_amdgcn_mbcnt_hi((uint32_t)(votes >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)votes, 0));
+        const uint64_t sel = __builtin_amdgcn_ballot_w64(mine && before == left);
+        bh = (__builtin_ctzll(sel)) * a.heads_q + lid % a.heads_q;
+        pk_blk = i;
+        break;
+      }
+      left -= cnt;
+    }
+    if (bh < 0) return;
+    pslot = 0;
+  } else if (a.cu_q) {
     if (a.n_splits > 1) {
       split = lid % a.n_splits;
       lid /= a.n_splits;
@@ -111,10 +139,13 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   const int hk = h / a.group;
   uint32_t drop_key = 0;
   if constexpr (DROP) {
-    drop_key = drop_head_key(a.seed, a.offset, (uint32_t)bh);
+    // the two numbers of the mask: by value, or (a launch recorded into a graph) read now from the generator's state
+    const uint64_t seed = a.seed_ptr ? (uint64_t)*a.seed_ptr : a.seed;
+    const uint64_t offset = a.offset_ptr ? (uint64_t)*a.offset_ptr + a.offset : a.offset;
+    drop_key = drop_head_key(seed, offset, (uint32_t)bh);
     if (blockIdx.x == 0 && tid == 0) {
-      if (a.rng_seed_out) *a.rng_seed_out = (int64_t)a.seed;
-      if (a.rng_offset_out) *a.rng_offset_out = (int64_t)a.offset;
+      if (a.rng_seed_out) *a.rng_seed_out = (int64_t)seed;
+      if (a.rng_offset_out) *a.rng_offset_out = (int64_t)offset;
     }
   }
 
@@ -134,9 +165,10 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   // so that every workgroup of a sequence has the same number of tiles; unpaired -> one block, heavy blocks first
   // (packed: counted down from the longest possible sequence so that equal slots mean equal block indices)
   const int nblk = (Lq + BM - 1) / BM;
-  const int blk_first = (a.cu_q ? a.n_mblk : nblk) - 1 - pslot;
-  if (a.pair ? (2 * pslot >= nblk) : (blk_first < 0 || blk_first >= nblk)) return;
-  const int n_own = (DP != 256 && a.pair && blk_first != pslot) ? 2 : 1;  // head_dim 256 never pairs (registers)
+  const int blk_first = pk_blk >= 0 ? pk_blk : (a.cu_q ? a.n_mblk : nblk) - 1 - pslot;
+  const int blk_second = pk_blk >= 0 ? nblk - 1 - pk_blk : pslot;
+  if (pk_blk < 0 && (a.pair ? (2 * pslot >= nblk) : (blk_first < 0 || blk_first >= nblk))) return;
+  const int n_own = (DP != 256 && a.pair && blk_first != blk_second) ? 2 : 1;  // head_dim 256 never pairs (registers)
   const int off = a.causal_tl ? 0 : Lk - Lq;  // causal: col visible iff col <= row + off
 
   const unsigned char* qp = a.q + qb + (int64_t)q0 * a.q_ss + (int64_t)h * a.q_sh;
@@ -210,7 +242,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   const float lazy = kLazyLog2 / c;  // threshold in score units
 
   for (int own = 0; own < n_own; ++own) {
-  const int m0 = (own == 0 ? blk_first : pslot) * BM;
+  const int m0 = (own == 0 ? blk_first : blk_second) * BM;
   int n_end = Lk;
   if (a.is_causal) n_end = min(Lk, m0 + BM + off);
   if (n_end < 0) n_end = 0;
@@ -487,11 +519,13 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     if (row < Lq && row < a.seqlen_q) {
       const int64_t slot = (((int64_t)b * a.heads_q + h) * a.seqlen_q + row) * a.n_splits + split;
       float* dst = a.ws_o + slot * D;
+      int g_e = g;  // (kept out of loop-invariant hoisting, as below)
+      asm volatile("" : "+v"(g_e));
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int v4 = 0; v4 < 4; ++v4) {
-          const int d = 32 * mb + 8 * v4 + 4 * g;
+          const int d = 32 * mb + 8 * v4 + 4 * g_e;
           if (d < D) *(f32x4*)(dst + d) = f32x4{o[mb][4 * v4 + 0], o[mb][4 * v4 + 1], o[mb][4 * v4 + 2], o[mb][4 * v4 + 3]};
         }
       if (g == 0) {
@@ -503,12 +537,16 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   }
   const float inv = (l_run > 0.f) ? (DROP ? a.drop_rp : 1.f) / l_run : 0.f;
   if (row < Lq) {
+    // (the lane's column group passes through an empty asm statement so that the 16 store offsets and their
+    // `d < D` predicates are formed here and not once ahead of all loops, where they would be spilled)
+    int g_e = g;
+    asm volatile("" : "+v"(g_e));
     unsigned char* orow = a.out + ob + (int64_t)(q0 + row) * a.o_ss + (int64_t)h * a.o_sh;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int v4 = 0; v4 < 4; ++v4) {
-        const int d = 32 * mb + 8 * v4 + 4 * g;
+        const int d = 32 * mb + 8 * v4 + 4 * g_e;
         if (d < D) {
           u32x2 w;
           w[0] = Mma<T>::pack2(o[mb][4 * v4 + 0] * inv, o[mb][4 * v4 + 1] * inv);
@@ -899,6 +937,7 @@ KArgs make_args(const fa_fwd_params* p, int kern, int ns, void* ws) {
   a.drop_thr = (uint32_t)floorf(p_keep * 255.f);
   a.drop_rp = 1.f / p_keep;
   a.seed = p->philox_seed; a.offset = p->philox_offset;
+  a.seed_ptr = p->philox_seed_ptr; a.offset_ptr = p->philox_offset_ptr;
   a.rng_seed_out = p->rng_seed_out; a.rng_offset_out = p->rng_offset_out;
   a.dmask = (unsigned char*)p->dropout_mask;
   a.ws_o = nullptr;
@@ -917,9 +956,11 @@ int launch_tile(KArgs a, hipStream_t st) {
   constexpr auto kfn = fa_tile_kernel<T, DP, MINB, BIAS, DROP, DMASK>;
   if (!ensure_dynamic_lds<kfn>(lds)) return FA_ERR_LAUNCH;
   const int nblk = (a.seqlen_q + 127) / 128;
-  a.pair = (DP != 256 && !a.cu_q && a.n_splits == 1 && a.is_causal && nblk >= 2 &&
+  a.pair = (DP != 256 && a.n_splits == 1 && a.is_causal && nblk >= 2 &&
             (int64_t)a.batch * a.heads_q * ((nblk + 1) / 2) >= 1024) ? 1 : 0;
-  a.n_mblk = a.pair ? (nblk + 1) / 2 : nblk;
+  // packed: the kernel finds the pairs itself with one lane per sequence, in a loop over the block index
+  if (a.cu_q && (a.batch > 64 || nblk > 1024)) a.pair = 0;
+  a.n_mblk = (a.pair && !a.cu_q) ? (nblk + 1) / 2 : nblk;
   a.hgroup = 1;
   if (BIAS && !a.cu_q && a.bias_sh == 0)
     for (int gsz = FA_HGROUP; gsz > 1; gsz >>= 1)
@@ -927,7 +968,8 @@ int launch_tile(KArgs a, hipStream_t st) {
         a.hgroup = gsz;
         break;
       }
-  const int64_t grid = (int64_t)a.batch * a.heads_q * a.n_mblk * a.n_splits;
+  // (packed and paired: at most (n + 1) / 2 pairs per sequence; what the shorter sequences leave over exits)
+  const int64_t grid = (int64_t)a.batch * a.heads_q * ((a.pair && a.cu_q) ? (nblk + 1) / 2 : a.n_mblk) * a.n_splits;
   if (grid <= 0) return FA_OK;
   if (grid > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kfn, dim3((unsigned)grid), dim3(256), lds, st, a);

@@ -60,6 +60,8 @@ inline int validate(const fa_fwd_params* p) {
     if (p->kernel == FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
     if (p->dropout_mask && ((uintptr_t)p->dropout_mask & 3)) return FA_ERR_BAD_ARG;
     if (((uintptr_t)p->rng_seed_out | (uintptr_t)p->rng_offset_out) & 7) return FA_ERR_BAD_ARG;
+    if (((uintptr_t)p->philox_seed_ptr | (uintptr_t)p->philox_offset_ptr) & 7) return FA_ERR_BAD_ARG;
+    if (!p->philox_seed_ptr != !p->philox_offset_ptr) return FA_ERR_BAD_ARG;  // both or neither
   }
   if ((uintptr_t)p->seqused_k & 3) return FA_ERR_BAD_ARG;
   if (p->bias) {
