@@ -83,28 +83,42 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   int pk_blk = -1;  // packed, paired: the heavy block of this workgroup's pair
   if (a.cu_q && a.pair) {
     // Packed and causal, lengths known only here: every workgroup finds its own work.  A sequence of n blocks is cut
-    // into the pairs (i, n-1-i), n-1 >= i >= (n-1)/2, which all cost the same; the pairs of all sequences are ordered
-    // by i, largest first (so the pairs of the longest sequences run first and the short ones fill the end), then by
-    // sequence, and workgroup number `item` takes pair number `item` of that order.  One lane per sequence (at most
-    // 64, checked by the launcher) votes "I have a pair with this i"; the workgroups beyond the last pair are the
-    // last ones of the grid and exit.
-    const int item = lid / a.heads_q;
-    bh = -1;
+    // into (n + 1) / 2 pairs (n-1-p, p), which all cost the same, about n + 1 tiles.  The sequences are taken longest
+    // first (so the short ones fill the end of the launch), and within a sequence the pairs of 8 kv heads (all query
+    // heads of their groups) form one run of consecutive workgroups, kv head fastest: consecutive workgroups go to
+    // the 8 XCDs in turn, so everything that reads one (sequence, kv head) lands on one XCD at about the same time
+    // and shares its L2 for K and V.  One lane per sequence
+    // (at most 64, checked by the launcher) works out its rank and where its run of workgroups starts; the
+    // workgroups beyond the last pair are the last ones of the grid and exit.
     int nb = 0;
     if (lane < a.batch) nb = (a.cu_q[lane + 1] - a.cu_q[lane] + BM - 1) / BM;
-    int left = item;
-    for (int i = a.n_mblk - 1; i >= 0; --i) {
-      const bool mine = i < nb && 2 * i >= nb - 1;
-      const uint64_t votes = __builtin_amdgcn_ballot_w64(mine);
-      const int cnt = __builtin_popcountll(votes);
-      if (left < cnt) {
-        const int before = __builtin_amdgcn_mbcnt_hi((uint32_t)(votes >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)votes, 0));
-        const uint64_t sel = __builtin_amdgcn_ballot_w64(mine && before == left);
-        bh = (__builtin_ctzll(sel)) * a.heads_q + lid % a.heads_q;
-        pk_blk = i;
-        break;
+    const int np = (nb + 1) >> 1;  // pairs of this lane's sequence
+    int start = 0;                 // pairs of the sequences that come before it
+    for (int o = 0; o < a.batch; ++o) {
+      const int nbo = __builtin_amdgcn_readlane(nb, o);
+      const bool first = nbo > nb || (nbo == nb && o < lane);
+      start += first ? (nbo + 1) >> 1 : 0;
+    }
+    const int H = a.heads_q;
+    const bool mine = lane < a.batch && lid >= start * H && lid < (start + np) * H;
+    const uint64_t sel = __builtin_amdgcn_ballot_w64(mine);
+    bh = -1;
+    if (sel != 0) {
+      const int sb = __builtin_ctzll(sel);
+      const int np_b = __builtin_amdgcn_readlane(np, sb);
+      const int r = lid - __builtin_amdgcn_readlane(start, sb) * H;
+      int hh, pp;
+      if ((a.heads_k & 7) == 0) {
+        const int run = 8 * a.group * np_b;  // workgroups of 8 kv heads: (pair, head of the group) x 8 kv heads
+        const int t = (r % run) >> 3;
+        hh = ((r / run) * 8 + (r & 7)) * a.group + t % a.group;
+        pp = t / a.group;
+      } else {
+        hh = r % H;
+        pp = r / H;
       }
-      left -= cnt;
+      bh = sb * H + hh;
+      pk_blk = __builtin_amdgcn_readlane(nb, sb) - 1 - pp;
     }
     if (bh < 0) return;
     pslot = 0;
@@ -258,19 +272,36 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   if (ntiles > jt0) issue_tile(jt0, 0);
 
   // ---- Q fragments (B operand): lane (c32, g) holds Q[row][16 ks + 8 g .. +8] -----------------------------
+  // The block's 128 rows come in through LDS like two K tiles (rows 0-63 into K buffer 1, rows 64-127 into V buffer
+  // 1, same swizzle, whole rows per DMA instruction; rows beyond the sequence repeat its last row) and each lane
+  // picks its fragments up from there: loading them straight from global memory takes 16 bytes from each of 32 rows
+  // per instruction, measured at 3.7 us per block.
   s16x8 qf[KS];
   {
-    const int qr = min(row, Lq - 1);
-    const unsigned char* qrow = qp + (int64_t)qr * a.q_ss;
+    const unsigned char* qt = qp + (int64_t)m0 * a.q_ss;
+    const int rmaxq = Lq - 1 - m0;  // >= 0: the block exists
+    const unsigned q_ss = (unsigned)a.q_ss;
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const unsigned r = (unsigned)min(64 * half + dma_r + i * 4 * RPI, rmaxq);
+        dma16s(qt, r * q_ss + ((DP == 256 && (i & 1)) ? lck_odd : lck) * 16, lds0 + (half ? 3 * TILE : TILE) + i * 4096);
+      }
+    WAIT_VMCNT(0);
+    __syncthreads();
+    const unsigned char* qs = smem + ((wave >> 1) ? 3 * TILE : TILE) + (wave & 1) * 32 * ROWB;
     const unsigned flip = a.neg_scale ? 0x80008000u : 0u;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const int ch = 2 * ks + g;
-      u32x4 x = {0, 0, 0, 0};
-      if (ch * 8 < D) x = *(const u32x4*)(qrow + ch * 16);
+      u32x4 x = *(const u32x4*)(qs + kaddr[ks]);
+      if ((2 * ks + g) * 8 >= D) x = u32x4{0, 0, 0, 0};  // pad chunks hold a copy of chunk 0
       x ^= flip;
       qf[ks] = __builtin_bit_cast(s16x8, x);
     }
+    // the fragments are in registers before any wavefront passes the first tile's barrier and sends the second
+    // tile into these two buffers
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
 
   f32x16 o[MB];
@@ -536,24 +567,35 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     continue;
   }
   const float inv = (l_run > 0.f) ? (DROP ? a.drop_rp : 1.f) / l_run : 0.f;
-  if (row < Lq) {
-    // (the lane's column group passes through an empty asm statement so that the 16 store offsets and their
-    // `d < D` predicates are formed here and not once ahead of all loops, where they would be spilled)
-    int g_e = g;
-    asm volatile("" : "+v"(g_e));
-    unsigned char* orow = a.out + ob + (int64_t)(q0 + row) * a.o_ss + (int64_t)h * a.o_sh;
+  // O goes out through LDS: in the accumulator layout a store instruction would write 16 bytes into each of 32 rows
+  // (every cache line of the block in 8 pieces, measured at 3.8 us per block); staged, it writes whole rows.  Each
+  // wavefront stages its own 32 rows (row stride padded by 16 bytes: the 8-byte writes of rows r and r + 16 share a
+  // bank, the 16-byte reads are conflict-free).
+  __syncthreads();  // every wavefront is done with the K/V buffers of the last tile
+  {
+    constexpr int OSTR = ROWB + 16;
+    unsigned char* stage = smem + wave * (32 * OSTR);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int v4 = 0; v4 < 4; ++v4) {
-        const int d = 32 * mb + 8 * v4 + 4 * g_e;
-        if (d < D) {
-          u32x2 w;
-          w[0] = Mma<T>::pack2(o[mb][4 * v4 + 0] * inv, o[mb][4 * v4 + 1] * inv);
-          w[1] = Mma<T>::pack2(o[mb][4 * v4 + 2] * inv, o[mb][4 * v4 + 3] * inv);
-          *(u32x2*)(orow + d * 2) = w;
-        }
+        u32x2 w;
+        w[0] = Mma<T>::pack2(o[mb][4 * v4 + 0] * inv, o[mb][4 * v4 + 1] * inv);
+        w[1] = Mma<T>::pack2(o[mb][4 * v4 + 2] * inv, o[mb][4 * v4 + 3] * inv);
+        *(u32x2*)(stage + c32 * OSTR + (32 * mb + 8 * v4 + 4 * g) * 2) = w;
       }
+    constexpr int RPS = 64 / CPR;  // rows per store instruction
+    unsigned char* oblk = a.out + ob + (int64_t)(q0 + m0 + 32 * wave) * a.o_ss + (int64_t)h * a.o_sh;
+    const int sr = lane / CPR, sch = lane % CPR;
+    const int rows_left = Lq - (m0 + 32 * wave);  // rows of this wavefront that exist
+#pragma unroll
+    for (int i = 0; i < 32 / RPS; ++i) {
+      const int r = i * RPS + sr;
+      const u32x4 x = *(const u32x4*)(stage + r * OSTR + sch * 16);
+      if (r < rows_left && sch * 8 < D) *(u32x4*)(oblk + (int64_t)r * a.o_ss + sch * 16) = x;
+    }
+  }
+  if (row < Lq) {
     if (g == 0) {
       const float lse = (l_run > 0.f) ? (m_run * c + __builtin_log2f(l_run)) * kLn2 : INFINITY;
       a.lse[lb + (int64_t)h * a.lse_sh + (int64_t)(q0 + row) * a.lse_ss] = lse;

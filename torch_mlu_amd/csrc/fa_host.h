@@ -53,7 +53,9 @@ inline int validate(const fa_fwd_params* p) {
   }
   if (p->lse_stride_h < 0 || p->lse_stride_s < 0) return FA_ERR_BAD_ARG;
   // the kernels form per-lane byte offsets inside a tile (up to 128 rows) as 32-bit row x 32-bit stride
-  if (p->k_stride_s > kMaxRowStrideBytes / 2 || p->v_stride_s > kMaxRowStrideBytes / 2) return FA_ERR_UNSUPPORTED;
+  if (p->k_stride_s > kMaxRowStrideBytes / 2 || p->v_stride_s > kMaxRowStrideBytes / 2 ||
+      p->q_stride_s > kMaxRowStrideBytes / 2)
+    return FA_ERR_UNSUPPORTED;
   if (p->is_causal < FA_MASK_NONE || p->is_causal > FA_MASK_CAUSAL_TOP_LEFT) return FA_ERR_BAD_ARG;
   if (p->reserved2 != 0 || !(p->dropout_p >= 0.f && p->dropout_p < 1.f)) return FA_ERR_BAD_ARG;
   if (p->dropout_p > 0.f) {
