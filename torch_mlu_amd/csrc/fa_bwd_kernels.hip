@@ -506,21 +506,32 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
       for (int t = 0; t < 4; ++t) store_dbias(j, t, u32x4{0, 0, 0, 0});
   }
 
-  if (row < Lq) {
-    unsigned char* orow = a.dq + dqb + (int64_t)(q0 + row) * a.dq_ss + (int64_t)h * a.dq_sh;
+  // dQ goes out through LDS, as O does in the forward kernel: staged per wavefront (32 rows, row stride padded by
+  // 16 bytes) and stored as whole rows instead of 8-byte pieces of 32 rows per instruction.
+  __syncthreads();  // every wavefront is done with the K/V buffers of the last tile
+  {
+    constexpr int OSTR = ROWB + 16;
+    unsigned char* stage = smem + wave * (32 * OSTR);
     const float sc = a.scale;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int v4 = 0; v4 < 4; ++v4) {
-        const int d = 32 * mb + 8 * v4 + 4 * g;
-        if (d < D) {
-          u32x2 w;
-          w[0] = Mma<T>::pack2(acc[mb][4 * v4 + 0] * sc, acc[mb][4 * v4 + 1] * sc);
-          w[1] = Mma<T>::pack2(acc[mb][4 * v4 + 2] * sc, acc[mb][4 * v4 + 3] * sc);
-          *(u32x2*)(orow + d * 2) = w;
-        }
+        u32x2 w;
+        w[0] = Mma<T>::pack2(acc[mb][4 * v4 + 0] * sc, acc[mb][4 * v4 + 1] * sc);
+        w[1] = Mma<T>::pack2(acc[mb][4 * v4 + 2] * sc, acc[mb][4 * v4 + 3] * sc);
+        *(u32x2*)(stage + c32 * OSTR + (32 * mb + 8 * v4 + 4 * g) * 2) = w;
       }
+    constexpr int RPS = 64 / CPR;  // rows per store instruction
+    unsigned char* oblk = a.dq + dqb + (int64_t)(q0 + m0 + 32 * wave) * a.dq_ss + (int64_t)h * a.dq_sh;
+    const int sr = lane / CPR, sch = lane % CPR;
+    const int rows_left = Lq - (m0 + 32 * wave);
+#pragma unroll
+    for (int i = 0; i < 32 / RPS; ++i) {
+      const int r = i * RPS + sr;
+      const u32x4 x = *(const u32x4*)(stage + r * OSTR + sch * 16);
+      if (r < rows_left && sch * 8 < D) *(u32x4*)(oblk + (int64_t)r * a.dq_ss + sch * 16) = x;
+    }
   }
 }
 
@@ -994,29 +1005,49 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
     }
   }
 
-  if (kvrow < Lk) {
-    unsigned char* krow = a.dk + dkb + (int64_t)(k0 + kvrow) * a.dk_ss + (int64_t)hk * a.dk_sh;
-    unsigned char* vrow = a.dv + dvb + (int64_t)(k0 + kvrow) * a.dv_ss + (int64_t)hk * a.dv_sh;
+  // dK and dV go out through LDS like the forward's O: staged per wavefront (its 32 key rows, row stride padded by 16
+  // bytes), then stored as whole rows.  One staging area per wavefront serves dK, then dV (LDS operations of a
+  // wavefront run in order).
+  __syncthreads();  // every wavefront is done with the Q / dO buffers of the last tile
+  {
+    constexpr int OSTR = ROWB + 16;
+    unsigned char* stage = smem + wave * (32 * OSTR);
+    constexpr int RPS = 64 / CPR;  // rows per store instruction
+    const int sr = lane / CPR, sch = lane % CPR;
+    const int rows_left = Lk - (n0 + 32 * wave);
     const float sc = a.scale;
+    auto flush = [&](unsigned char* base, int64_t row_stride) __attribute__((always_inline)) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int v4 = 0; v4 < 4; ++v4) {
-        const int d = 32 * mb + 8 * v4 + 4 * g;
-        if (d < D) {
-          u32x2 w;
-          if constexpr (DO_K) {
-            w[0] = Mma<T>::pack2(dk[mb][4 * v4 + 0] * sc, dk[mb][4 * v4 + 1] * sc);
-            w[1] = Mma<T>::pack2(dk[mb][4 * v4 + 2] * sc, dk[mb][4 * v4 + 3] * sc);
-            *(u32x2*)(krow + d * 2) = w;
-          }
-          if constexpr (DO_V) {
-            w[0] = Mma<T>::pack2(dv[mb][4 * v4 + 0], dv[mb][4 * v4 + 1]);
-            w[1] = Mma<T>::pack2(dv[mb][4 * v4 + 2], dv[mb][4 * v4 + 3]);
-            *(u32x2*)(vrow + d * 2) = w;
-          }
-        }
+      for (int i = 0; i < 32 / RPS; ++i) {
+        const int r = i * RPS + sr;
+        const u32x4 x = *(const u32x4*)(stage + r * OSTR + sch * 16);
+        if (r < rows_left && sch * 8 < D) *(u32x4*)(base + (int64_t)r * row_stride + sch * 16) = x;
       }
+    };
+    if constexpr (DO_K) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {
+          u32x2 w;
+          w[0] = Mma<T>::pack2(dk[mb][4 * v4 + 0] * sc, dk[mb][4 * v4 + 1] * sc);
+          w[1] = Mma<T>::pack2(dk[mb][4 * v4 + 2] * sc, dk[mb][4 * v4 + 3] * sc);
+          *(u32x2*)(stage + c32 * OSTR + (32 * mb + 8 * v4 + 4 * g) * 2) = w;
+        }
+      flush(a.dk + dkb + (int64_t)(k0 + n0 + 32 * wave) * a.dk_ss + (int64_t)hk * a.dk_sh, a.dk_ss);
+    }
+    if constexpr (DO_V) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {
+          u32x2 w;
+          w[0] = Mma<T>::pack2(dv[mb][4 * v4 + 0], dv[mb][4 * v4 + 1]);
+          w[1] = Mma<T>::pack2(dv[mb][4 * v4 + 2], dv[mb][4 * v4 + 3]);
+          *(u32x2*)(stage + c32 * OSTR + (32 * mb + 8 * v4 + 4 * g) * 2) = w;
+        }
+      flush(a.dv + dvb + (int64_t)(k0 + n0 + 32 * wave) * a.dv_ss + (int64_t)hk * a.dv_sh, a.dv_ss);
+    }
   }
 }
 
