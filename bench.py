@@ -27,15 +27,21 @@ PEAK_MFMA_TFLOPS = 2500.0  # dense bf16 / fp16
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same file,
 # each scaled by what the same counter reads for the 1 GiB copy of --config copy1g (2.000 and 1.000); the runs and
-# their commands are recorded under profiles/.  Counters cannot be read from inside a timed run, so these are the
-# recorded values (None: not profiled).
+# their commands are recorded under profiles/ (all of one session on one box, after the last kernel change).  Counters
+# cannot be read from inside a timed run, so these are the recorded values (None: not profiled).
 TRAFFIC_BYTES = {
-    "cfg2": int((522.2 + 130.0) * 2 ** 20),
+    "cfg2": int((525.2 + 130.0) * 2 ** 20),
+    "cfg3": int((212.1 + 130.0) * 2 ** 20),
+    "cfg4": int((286.1 + 68.2) * 2 ** 20),
     "cfg5": int(2.0006 * 2 ** 30 + 0.52 * 2 ** 20),
-    "cfg2_bwd": int((1828.3 + 388.2) * 2 ** 20),  # the three launches of one backward together
-    "cfg2_mask": int(2.17 * 2 ** 30 + 199.5 * 2 ** 20),
-    "cfg2_drop": int((518.6 + 130.0) * 2 ** 20),
-    "cfg2_mask_bwd": int((2.80 + 2.24 + 2.00) * 2 ** 30 + (148.1 + 128.6 + 128.0) * 2 ** 20),  # three launches
+    "cfg2_bwd": int((1849.0 + 388.0) * 2 ** 20),  # the three launches of one backward together
+    "cfg2_mask": int(2.10 * 2 ** 30 + 130.0 * 2 ** 20),
+    "cfg2_drop": int((517.2 + 130.0) * 2 ** 20),
+    "cfg2_mask_bwd": int((3.84 + 2.24 + 1.97) * 2 ** 30 + (156.0 + 128.0 + 128.0) * 2 ** 20),  # three launches
+    "cfg2_tile256": int((686.7 + 130.0) * 2 ** 20),
+    "cfg2_tile256w": int((659.4 + 130.0) * 2 ** 20),
+    "spec4": int(1.0011 * 2 ** 30 + (2.1 + 2.1 + 0.3) * 2 ** 20),  # split-KV + merge launches
+    "chunk256": int((182.0 + 32.6 + 32.6 + 2.1) * 2 ** 20),        # sliced tile + merge launches
 }
 
 

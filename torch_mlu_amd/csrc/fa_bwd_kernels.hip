@@ -25,7 +25,6 @@
 #include "fa_device.h"
 #include "fa_host.h"
 
-// ring depths of the two operand prefetch loops of the dK/dV kernel, by what the instantiation computes
 // ring depths of the two operand prefetch loops of the dQ kernel
 #ifndef FA_RQ
 #define FA_RQ 2
@@ -33,14 +32,16 @@
 #ifndef FA_RA
 #define FA_RA 2
 #endif
+// ring depths of the two operand prefetch loops of the dK/dV kernel, by what the instantiation computes
 #ifndef FA_RS
 #define FA_RS(DO_K, DO_V) ((DO_K) ? 2 : 4)
 #endif
-#ifndef FA_HGROUP
-#define FA_HGROUP 4
-#endif
 #ifndef FA_RT
 #define FA_RT(DO_K, DO_V) ((DO_K) && (DO_V) ? 2 : 4)
+#endif
+// heads whose workgroups are interleaved when a bias is broadcast over heads
+#ifndef FA_HGROUP
+#define FA_HGROUP 4
 #endif
 // dV-only kernel: all 64 query rows of a tile in one pass (needs 16 more registers)
 #ifndef FA_WIDE

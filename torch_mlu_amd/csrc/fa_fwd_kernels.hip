@@ -68,12 +68,10 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   const int g = lane >> 5, c32 = lane & 31;
 
   // ---- which (sequence, head, query block): XCD-aware, heavy blocks first -------------------------------
-  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical ids so that
-  // all query blocks of one (sequence, kv head) share that XCD's L2.
   // Dense: workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical ids so that
   // all query blocks of one (sequence, kv head) share that XCD's L2.  Packed (ragged lengths, known only on the
-  // device): block-major order instead, i.e. the last (heaviest) blocks of all sequences first and sequences
-  // shorter than that exit at once — longest-processing-time-first without knowing the lengths on the host.
+  // device): causal calls that can pair blocks search their pair below; the others go block-major, i.e. the last
+  // (heaviest) blocks of all sequences first and sequences shorter than that exit at once.
   int lid = blockIdx.x;
   int pslot, bh;
   // Sliced mode (few query blocks against a long K/V: chunked prefill, speculative decoding): workgroup
