@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the flash-attention forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop|cfg2_mask_bwd|spec4|chunk256|cfg2_tile256|cfg2_tile256w] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop|cfg2_mask_bwd|spec4|chunk256|cfg2_tile256|cfg2_tile256w|cfg5_paged] [--no-extras] [--no-cpu-baseline]
 
 A "step" is one call of the registered op on one batch of seeded synthetic input that is already resident in HBM.
 The headline workload is BASELINE.json configs[1] (causal prefill, bf16 MHA, B=4 H=32 S=4096 D=128); the other
@@ -210,6 +210,38 @@ def make_workload(name, dev):
         return dict(call=call, check=check, flops=4 * B * Hq * Sk * D, bytes_kv=2 * B * Hk * Sk * D * 2,
                     desc=f"decode bf16 GQA B={B} Hq={Hq} Hkv={Hk} Sq=1 Skv={Sk} D={D}", dtype="bf16", bound="hbm",
                     kernel="fa_splitkv_kernel")
+    if name == "cfg5_paged":
+        # cfg5's decode against the same amount of K/V held in 256-row pages that are scattered over a pool and found
+        # through a block table (fa_fwd_params.block_table, C ABI); three pools in turn, as cfg5 rotates its K/V sets
+        from torch_mlu_amd import capi
+        B, Hq, Hk, Sk, D, page = 64, 32, 8, 8192, 128, 256
+        q = seeded((B, Hq, 1, D), 4, bf).to(dev)
+        per_seq = Sk // page
+        g = torch.Generator().manual_seed(7)
+        pools = []
+        k0 = seeded((B * per_seq, page, Hk, D), 5, bf).to(dev)
+        v0 = seeded((B * per_seq, page, Hk, D), 6, bf).to(dev)
+        for r in range(3):
+            table = torch.randperm(B * per_seq, generator=g).reshape(B, per_seq).to(torch.int32).to(dev)
+            pools.append((torch.roll(k0, 7 * r, dims=0) if r else k0, torch.roll(v0, 7 * r, dims=0) if r else v0, table))
+        used = torch.full((B,), Sk, dtype=torch.int32, device=dev)
+        state = {"i": 0}
+
+        def call():
+            kk, vv, tt = pools[state["i"] % 3]
+            state["i"] += 1
+            return capi.fa_forward_paged(q, kk, vv, tt, used)
+
+        def check():
+            kk, vv, tt = pools[0]
+            out, lse = capi.fa_forward_paged(q, kk, vv, tt, used)
+            kf = kk[tt.long()].reshape(B, Sk, Hk, D).transpose(1, 2)
+            vf = vv[tt.long()].reshape(B, Sk, Hk, D).transpose(1, 2)
+            return _check_heads(q, kf, vf, out, lse, False, [(0, 0), (B - 1, Hq - 1)])
+
+        return dict(call=call, check=check, flops=4 * B * Hq * Sk * D, bytes_kv=2 * B * Hk * Sk * D * 2,
+                    desc=f"decode bf16 GQA B={B} Hq={Hq} Hkv={Hk} Sq=1 Skv={Sk} D={D}, K/V in scattered {page}-row pages "
+                         "through a block table (fa_fwd_launch)", dtype="bf16", bound="hbm", kernel="fa_splitkv_kernel")
     if name in ("spec4", "chunk256"):
         # serving shapes beside the BASELINE configs (extras only): 4 speculative tokens per sequence against a 32k
         # KV cache (rides the split-KV kernel, HBM-bound) and a 256-token prefill chunk of one sequence against a
@@ -404,7 +436,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "spec4", "chunk256", "copy1g",
-                             "cfg2_tile256", "cfg2_tile256w"])
+                             "cfg2_tile256", "cfg2_tile256w", "cfg5_paged"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -427,7 +459,7 @@ def main():
         n0 = torch_mlu_amd.launch_count()
         eo, el = w["check"]()
         wall, ev_mean, ev_med, ev_min = time_steps(w["call"], steps, warmup)
-        assert name in ("copy1g", "cfg2_tile256", "cfg2_tile256w") or torch_mlu_amd.launch_count() >= n0 + steps + warmup, \
+        assert name in ("copy1g", "cfg2_tile256", "cfg2_tile256w", "cfg5_paged") or torch_mlu_amd.launch_count() >= n0 + steps + warmup, \
             "the registered HIP path did not run"
         r = {"config": name, "workload": w["desc"], "ms_per_step": wall, "kernel_ms_mean": ev_mean,
              "kernel_ms_median": ev_med, "kernel_ms_min": ev_min, "tflops": w["flops"] / wall / 1e9,
@@ -451,11 +483,11 @@ def main():
     extras = []
     if not args.no_extras:
         for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd",
-                     "spec4", "chunk256"):
+                     "spec4", "chunk256", "cfg5_paged"):
             if name != args.config:
                 extras.append(run(name, args.steps, args.warmup))
 
-    is_decode = args.config in ("cfg5", "spec4", "copy1g")
+    is_decode = args.config in ("cfg5", "spec4", "copy1g", "cfg5_paged")
     line = {
         "metric": "fwd attn TFLOP/s + % MFMA peak (bf16 S=4096 D=128); decode HBM GB/s",
         "value": main_r.get("kv_gbs") if is_decode else main_r["tflops"],
@@ -473,6 +505,7 @@ def main():
                    "entry": {"cfg4": "aten::_flash_attention_forward", "spec4": "aten::_flash_attention_forward",
                              "chunk256": "aten::_flash_attention_forward",
                              "cfg2_tile256": "fa_fwd_launch (C ABI)", "cfg2_tile256w": "fa_fwd_launch (C ABI)",
+                             "cfg5_paged": "fa_fwd_launch (C ABI)",
                              "cfg2_bwd": "aten::_scaled_dot_product_flash_attention_backward",
                              "cfg2_mask": "aten::_scaled_dot_product_efficient_attention",
                              "cfg2_mask_bwd": "aten::_scaled_dot_product_efficient_attention_backward"}.get(

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FA_FWD_ABI_VERSION 7
+#define FA_FWD_ABI_VERSION 8
 
 /* element types accepted for q/k/v/out (FlashAttention_internal.cpp:73-80 allows exactly these two) */
 #define FA_DTYPE_FP16 0
@@ -146,6 +146,18 @@ typedef struct fa_fwd_params {
      rng_seed_out / rng_offset_out receive the resolved numbers. */
   const int64_t* philox_seed_ptr;
   const int64_t* philox_offset_ptr;
+  /* optional paged KV cache (NULL = k / v are per-sequence tensors as above).  Dense mode, split-KV kernel only
+     (seqlen_q x heads_q / heads_k <= 16, no bias, no dropout, not top-left causal; anything else: FA_ERR_UNSUPPORTED).
+     k and v then point at pools of pages, [page][row in page][kv head][head_dim]: k_stride_b / v_stride_b are the
+     element strides between pages, k_stride_s / v_stride_s between the rows of a page.  Key row r of sequence b lives
+     in page block_table[b * block_table_stride + r / page_size] at row r % page_size.  seqlen_k is the longest
+     sequence's key count (block_table_stride * page_size at most); seqused_k gives each sequence's own.  page_size
+     must be a multiple of 32.  (No counterpart in the reference, whose ops take whole tensors; this is the block
+     table of serving engines.) */
+  const int32_t* block_table; /* device int32 [batch][block_table_stride] */
+  int64_t block_table_stride;
+  int32_t page_size;
+  int32_t reserved3;          /* must be 0 */
 } fa_fwd_params;
 
 #define FA_MAX_SPLITS 64

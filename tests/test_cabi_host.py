@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_version_and_error_strings():
     L = capi.lib()
-    assert L.fa_fwd_version() == capi.FA_FWD_ABI_VERSION == 7
+    assert L.fa_fwd_version() == capi.FA_FWD_ABI_VERSION == 8
     assert capi.error_string(0) == "ok"
     for rc in (-1, -2, -3, -99):
         assert capi.error_string(rc)

@@ -44,6 +44,7 @@ from . import backends, capi  # noqa: E402
 from .ops import (  # noqa: E402
     flash_attention_forward,
     launch_count,
+    paged_attention,
     scaled_dot_product_flash_attention,
     sdpa,
 )
@@ -54,6 +55,7 @@ __all__ = [
     "flash_attention_forward",
     "launch_count",
     "load",
+    "paged_attention",
     "scaled_dot_product_flash_attention",
     "sdpa",
 ]

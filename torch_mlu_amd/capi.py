@@ -21,7 +21,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libfa_fwd.so")
 
-FA_FWD_ABI_VERSION = 7
+FA_FWD_ABI_VERSION = 8
 FA_DTYPE_FP16 = 0
 FA_DTYPE_BF16 = 1
 FA_OK = 0
@@ -95,6 +95,10 @@ class FaFwdParams(ctypes.Structure):
         ("seqused_k", ctypes.c_void_p),
         ("philox_seed_ptr", ctypes.c_void_p),
         ("philox_offset_ptr", ctypes.c_void_p),
+        ("block_table", ctypes.c_void_p),
+        ("block_table_stride", ctypes.c_int64),
+        ("page_size", ctypes.c_int32),
+        ("reserved3", ctypes.c_int32),
     ]
 
 
@@ -233,6 +237,7 @@ def make_params(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Te
     # int64[2] on the device: (seed, offset base) read by the kernel when it runs; philox_offset is added to the base
     p.philox_seed_ptr = philox_state[0:].data_ptr() if philox_state is not None else None
     p.philox_offset_ptr = philox_state[1:].data_ptr() if philox_state is not None else None
+    p.block_table, p.block_table_stride, p.page_size, p.reserved3 = None, 0, 0, 0
     return p
 
 
@@ -268,6 +273,30 @@ def fa_forward_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, is_ca
                     is_causal=is_causal, kernel=kernel, num_splits=num_splits, bias=bias, dropout_p=dropout_p,
                     philox_seed=philox_seed, philox_offset=philox_offset, rng_out=rng_out, dropout_mask=dropout_mask,
                     seqused_k=seqused_k, philox_state=philox_state)
+    launch(p, q.device)
+    return out.transpose(1, 2), lse
+
+
+def fa_forward_paged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                     seqused_k: torch.Tensor, *, is_causal=False, scale: Optional[float] = None,
+                     num_splits: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Decode / speculative tokens against a paged KV cache.  q [B, Hq, Sq, D] with Sq * (Hq / Hk) <= 16;
+    k_pages / v_pages [pages, page_size, Hk, D] (any strides, contiguous last dim; page_size a multiple of 32);
+    block_table int32 [B, max_pages] on the device: the pages of each sequence in order; seqused_k int32 [B]: how many
+    keys each sequence holds.  -> out [B, Hq, Sq, D], lse [B, Hq, Sq].  Bottom-right causal when `is_causal`."""
+    B, Hq, Sq, D = q.shape
+    page_size, Hk = k_pages.shape[1], k_pages.shape[2]
+    assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] == B
+    assert block_table.stride(1) == 1
+    out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    # k / v stand in as [B, seqlen_k, Hk, D] views for the stride fields: batch stride = page stride
+    p = make_params(q.transpose(1, 2), k_pages, v_pages, out, lse, scale=scale, is_causal=is_causal,
+                    kernel=FA_KERNEL_SPLITKV, num_splits=num_splits, seqused_k=seqused_k)
+    p.seqlen_k = block_table.shape[1] * page_size
+    p.block_table = block_table.data_ptr()
+    p.block_table_stride = block_table.stride(0)
+    p.page_size = page_size
     launch(p, q.device)
     return out.transpose(1, 2), lse
 

@@ -35,6 +35,9 @@ struct KArgs {
   float scale_abs;    // |scale| (bias path)
   int32_t causal_tl;  // causal mask aligned to the top-left corner (col <= row) instead of the bottom-right one
   const int32_t* seqused_k;   // optional: keys of sequence b beyond seqused_k[b] do not exist
+  const int32_t* block_table; // optional (split-KV kernel): paged K/V, page of key row r = table[b * bt_stride + r / page_size]
+  int64_t bt_stride;
+  int32_t page_size;
   const unsigned char* bias;  // optional additive bias, dense mode: [b][h][row][col] through byte strides
   int64_t bias_sb, bias_sh, bias_sq;
   uint32_t drop_thr;  // dropout: an element is kept iff its byte <= drop_thr

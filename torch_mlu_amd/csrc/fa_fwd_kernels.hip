@@ -684,29 +684,45 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
   unsigned char* ring = smem + wave * SplitCfg<DP>::RING;
   const int dma_r = lane / CPR, dma_pc = lane % CPR;
 
-  auto issue_block = [&](int blk, int stage) {
+  // Paged cache: a 32-row block lies inside one page (page_size is a multiple of 32), so the page is one scalar
+  // table entry per block; `page` is that entry (fetched an iteration ahead of its use) and the rows count from the
+  // page's first row.  Without a table `page` is 0 and the rows count from the sequence's first key.
+  const int32_t* tbl = a.block_table ? a.block_table + (int64_t)b * a.bt_stride : nullptr;
+  const int psz = a.page_size;
+  auto page_of = [&](int blk_) -> int { return tbl ? tbl[min(blk_ * 32, last_k) / psz] : 0; };
+  auto issue_block = [&](int blk, int stage, int page) {
     unsigned char* kdst = ring + stage * SplitCfg<DP>::STAGE;
     unsigned char* vdst = kdst + BLK;
+    const unsigned char* kpg = kp;
+    const unsigned char* vpg = vp;
+    int row0 = 0;  // first key row of what kpg / vpg point at
+    if (tbl) {
+      kpg = a.k + (int64_t)page * a.k_sb + (int64_t)hk * a.k_sh;
+      vpg = a.v + (int64_t)page * a.v_sb + (int64_t)hk * a.v_sh;
+      row0 = min(blk * 32, last_k) / psz * psz;
+    }
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int r = dma_r + i * RPI;
       int lc = dma_pc ^ swzKd<DP>(r);
       if (lc * 8 >= D) lc = 0;
-      const int gr = min(blk * 32 + r, last_k);
-      dma16(kp + (uint64_t)(unsigned)gr * k_ss + lc * 16, kdst + i * 1024);
+      const int gr = min(blk * 32 + r, last_k) - row0;
+      dma16(kpg + (uint64_t)(unsigned)gr * k_ss + lc * 16, kdst + i * 1024);
     }
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int r = dma_r + i * RPI;
       int lc = dma_pc ^ swzVd<DP>(r);
       if (lc * 8 >= D) lc = 0;
-      const int gr = min(blk * 32 + r, last_k);
-      dma16(vp + (uint64_t)(unsigned)gr * v_ss + lc * 16, vdst + i * 1024);
+      const int gr = min(blk * 32 + r, last_k) - row0;
+      dma16(vpg + (uint64_t)(unsigned)gr * v_ss + lc * 16, vdst + i * 1024);
     }
   };
 
   int blk = blk_begin + wave;
-  if (blk < blk_end && Lq > 0) issue_block(blk, 0);
+  const bool any = blk < blk_end && Lq > 0;
+  if (any) issue_block(blk, 0, page_of(blk));
+  int page_next = (any && blk + NW < blk_end) ? page_of(blk + NW) : 0;  // the table entry of the next block to fetch
 
   // Q^T as B operand of 16x16x32: lane (q slot = L, G) holds Q[row][head][32 ks + 8 G .. +8] of its slot
   s16x8 qf[KS];
@@ -741,7 +757,8 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
   for (; blk < blk_end && Lq > 0; blk += NW) {
     const int nxt = blk + NW;
     if (nxt < blk_end) {
-      issue_block(nxt, stage ^ 1);
+      issue_block(nxt, stage ^ 1, page_next);
+      page_next = (nxt + NW < blk_end) ? page_of(nxt + NW) : 0;
       if constexpr (NI == 4) WAIT_VMCNT(8);
       else if constexpr (NI == 8) WAIT_VMCNT(16);
       else WAIT_VMCNT(32);
@@ -965,6 +982,7 @@ KArgs make_args(const fa_fwd_params* p, int kern, int ns, void* ws) {
   a.is_causal = p->is_causal ? 1 : 0;
   a.causal_tl = p->is_causal == FA_MASK_CAUSAL_TOP_LEFT ? 1 : 0;
   a.seqused_k = p->seqused_k;
+  a.block_table = p->block_table; a.bt_stride = p->block_table_stride; a.page_size = p->page_size;
   a.bias = (const unsigned char*)p->bias;
   a.bias_sb = p->bias_stride_b * 2; a.bias_sh = p->bias_stride_h * 2; a.bias_sq = p->bias_stride_q * 2;
   a.neg_scale = p->scale < 0.f ? 1 : 0;

@@ -66,6 +66,18 @@ inline int validate(const fa_fwd_params* p) {
     if (!p->philox_seed_ptr != !p->philox_offset_ptr) return FA_ERR_BAD_ARG;  // both or neither
   }
   if ((uintptr_t)p->seqused_k & 3) return FA_ERR_BAD_ARG;
+  if (p->reserved3 != 0) return FA_ERR_BAD_ARG;
+  if (p->block_table) {
+    // paged K/V: dense mode, a shape the split-KV kernel takes, pages of whole 32-row blocks, a table wide enough
+    if ((uintptr_t)p->block_table & 3) return FA_ERR_BAD_ARG;
+    if (p->page_size <= 0 || p->block_table_stride < 0) return FA_ERR_BAD_ARG;
+    if (p->page_size % 32) return FA_ERR_UNSUPPORTED;
+    if (p->block_table_stride < ((int64_t)p->seqlen_k + p->page_size - 1) / p->page_size) return FA_ERR_BAD_ARG;
+    if (p->cu_seqlens_q || p->bias || p->dropout_p > 0.f || p->is_causal == FA_MASK_CAUSAL_TOP_LEFT)
+      return FA_ERR_UNSUPPORTED;
+    if (p->kernel != FA_KERNEL_AUTO && p->kernel != FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
+    if (p->seqlen_q < 1 || (int64_t)p->seqlen_q * (p->heads_q / p->heads_k) > 16) return FA_ERR_UNSUPPORTED;
+  }
   if (p->bias) {
     if (((uintptr_t)p->bias & 7) || p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_q < 0 ||
         ((p->bias_stride_b | p->bias_stride_h | p->bias_stride_q) & 3))
@@ -84,6 +96,7 @@ inline void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   int kern = p->kernel;
   const int group = p->heads_q / p->heads_k;
   if (kern == FA_KERNEL_TILE128 || kern == FA_KERNEL_TILE256 || kern == FA_KERNEL_TILE256W) kern = FA_KERNEL_TILE;  // the family; tile_rows() picks
+  if (p->block_table) kern = FA_KERNEL_SPLITKV;  // the only kernel that reads a page table (validate() checked the shape)
   if (kern == FA_KERNEL_AUTO)
     kern = (p->seqlen_q >= 1 && (int64_t)p->seqlen_q * group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT && !(p->dropout_p > 0.f))
                ? FA_KERNEL_SPLITKV

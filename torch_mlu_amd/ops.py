@@ -39,6 +39,17 @@ def sdpa(query, key, value, *, is_causal: bool = False, scale: Optional[float] =
                                               enable_gqa=enable_gqa)
 
 
+def paged_attention(query, key_pages, value_pages, block_table, seqused_k, *, is_causal: bool = False,
+                    scale: Optional[float] = None):
+    """Decode (or a few speculative tokens: Sq * Hq / Hk <= 16) against a paged KV cache, through the C ABI
+    (`fa_fwd_params.block_table`; the reference's ops have no such argument).  query [B, Hq, Sq, D]; key_pages /
+    value_pages [pages, page_size, Hk, D] with page_size a multiple of 32; block_table int32 [B, max_pages] and
+    seqused_k int32 [B] on the device.  -> (out [B, Hq, Sq, D], logsumexp [B, Hq, Sq]).  Inference only."""
+    from . import capi
+
+    return capi.fa_forward_paged(query, key_pages, value_pages, block_table, seqused_k, is_causal=is_causal, scale=scale)
+
+
 def launch_count() -> int:
     """How many times this build's HIP kernels were enqueued through the registered ops."""
     return torch.ops.torch_mlu_amd._launch_count()
