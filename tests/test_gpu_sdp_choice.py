@@ -138,3 +138,62 @@ def test_flash_only_refusals_warn_and_raise(build, msg):
                     F.scaled_dot_product_attention(q, k, v, mask, 0.0, False)
         finally:
             torch.backends.cuda.enable_cudnn_sdp(prev)
+
+
+def _nested(lens, H, D, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    parts = [(torch.randn(L, H, D, generator=g) * 0.5).to(dtype) for L in lens]
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        return parts, torch.nested.nested_tensor(parts).to(DEV)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_nested_tensors_reach_the_packed_kernel(causal):
+    """Nested (ragged) q / k / v: the selector answers flash, PyTorch's nested-tensor kernel of the flash op packs them
+    and calls aten::_flash_attention_forward with cu_seqlens - this build's packed op (the reference's selector has the
+    same nested branch, sdp_utils.h:168-200, 322-370).  Forward values per sequence against the oracle, and the
+    gradients through the same route."""
+    H, D, lens = 4, 64, [37, 128, 5, 200]
+    qp, q = _nested(lens, H, D, HF, 1)
+    kp, k = _nested(lens, H, D, HF, 2)
+    vp, v = _nested(lens, H, D, HF, 3)
+    qt, kt, vt = (x.transpose(1, 2) for x in (q, k, v))          # [B, H, ragged, D]
+    assert torch._fused_sdp_choice(qt, kt, vt, None, 0.0, causal) == SDPBackend.FLASH_ATTENTION
+    n0 = torch_mlu_amd.launch_count()
+    out = F.scaled_dot_product_attention(qt, kt, vt, is_causal=causal)
+    assert torch_mlu_amd.launch_count() == n0 + 1 and out.is_nested
+    for i, o in enumerate(out.transpose(1, 2).unbind()):
+        qi, ki, vi = (p[i].transpose(0, 1)[None] for p in (qp, kp, vp))
+        ref, _ = oracle.sdpa_oracle(qi, ki, vi, is_causal=causal)
+        out_close(o.transpose(0, 1)[None].float().cpu().numpy(), ref, HF)
+    # training: the backward of the nested op calls aten::_flash_attention_backward, also this build's
+    leaves = [torch.nested.nested_tensor(p).to(DEV).requires_grad_() for p in (qp, kp, vp)]
+    n0 = torch_mlu_amd.launch_count()
+    o = F.scaled_dot_product_attention(*(x.transpose(1, 2) for x in leaves), is_causal=causal)
+    sum(t.sum() for t in o.unbind()).backward()
+    assert torch_mlu_amd.launch_count() == n0 + 2
+    for i in range(len(lens)):
+        qi, ki, vi = (p[i].transpose(0, 1)[None] for p in (qp, kp, vp))
+        want = oracle.sdpa_backward_oracle(qi, ki, vi, torch.ones_like(qi), is_causal=causal)
+        for leaf, w in zip(leaves, want):
+            got = leaf.grad.unbind()[i].transpose(0, 1)[None].float().cpu().numpy()
+            assert np.abs(got - w).max() <= 2 * 2.0 ** -11 * max(np.abs(w).max(), 0.25)
+
+
+def test_nested_refusals():
+    """An empty sequence and a mask are refused for nested inputs with the reference's messages; with only the flash
+    backend allowed the call then raises."""
+    H, D = 2, 64
+    _, q = _nested([10, 0, 7], H, D, HF, 4)
+    qt = q.transpose(1, 2)
+    with sdp_kernel(enable_flash=True, enable_math=False, enable_mem_efficient=False):
+        with pytest.warns(UserWarning, match="Fused kernels do not support seq_len == 0"):
+            with pytest.raises(RuntimeError, match="No available kernel"):
+                F.scaled_dot_product_attention(qt, qt, qt)
+    _, q = _nested([10, 3, 7], H, D, HF, 5)
+    _, k2 = _nested([10, 3], H, D, HF, 6)
+    with sdp_kernel(enable_flash=True, enable_math=False, enable_mem_efficient=False):
+        with pytest.warns(UserWarning, match="broadcastable batch size"):
+            with pytest.raises(RuntimeError, match="No available kernel"):
+                F.scaled_dot_product_attention(q.transpose(1, 2), k2.transpose(1, 2), k2.transpose(1, 2))

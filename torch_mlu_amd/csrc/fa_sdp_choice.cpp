@@ -10,12 +10,14 @@
 // choice among its remaining backends.
 #include <ATen/ATen.h>
 #include <ATen/Context.h>
+#include <ATen/NestedTensorImpl.h>
 #include <ATen/core/LegacyTypeDispatch.h>
 #include <ATen/native/DispatchStub.h>
 #include <ATen/native/transformers/attention.h>
 #include <c10/util/Exception.h>
 #include <torch/library.h>
 
+#include <algorithm>
 #include <array>
 #include <sstream>
 
@@ -48,10 +50,63 @@ bool check_runtime_disabled_flash(const sdp_params&, bool debug) {
   return true;
 }
 
+bool has_nested_inputs(const sdp_params& p) { return p.query.is_nested() || p.key.is_nested() || p.value.is_nested(); }
+
+// The mem-efficient entry points of this build take dense tensors only.
 bool check_not_nested(const sdp_params& p, bool debug) {
-  if (p.query.is_nested() || p.key.is_nested() || p.value.is_nested()) {
-    if (debug) TORCH_WARN("The flash kernels of this build take dense tensors only; packed sequences go through "
-                          "aten::_flash_attention_forward with cu_seqlens.");
+  if (has_nested_inputs(p)) {
+    if (debug) TORCH_WARN("The mem-efficient kernels of this build take dense tensors only; nested tensors go through "
+                          "the flash kernels.");
+    return false;
+  }
+  return true;
+}
+
+// Nested inputs (sdp_utils.h:168-200, 283-370): PyTorch's nested-tensor kernel of the flash op packs them and calls
+// aten::_flash_attention_forward with cu_seqlens, i.e. this build's packed op.  What it cannot pack is refused here,
+// with the reference's messages: a ragged head count, an empty sequence, batch sizes or head counts that are neither
+// equal nor 1.
+bool check_nested_sizes_one(const at::Tensor& t, const char* name, bool debug) {
+  if (!t.is_nested()) return true;
+  const auto* impl = at::native::get_nested_tensor_impl(t);
+  if (!impl->opt_size(1).has_value()) {
+    if (debug) TORCH_WARN("Fused kernels do not support ragged num_head_dims, ", name, "has a ragged num_heads.");
+    return false;
+  }
+  const at::Tensor& sizes = impl->get_nested_sizes();
+  const int64_t* ptr = sizes.data_ptr<int64_t>();
+  const int64_t n = t.size(0), stride = sizes.stride(0);
+  for (int64_t i = 0; i < n; ++i)
+    if (ptr[i * stride + 1] == 0) {
+      if (debug) TORCH_WARN("Fused kernels do not support seq_len == 0, ", name, "has a seq len of 0.");
+      return false;
+    }
+  return true;
+}
+
+bool broadcastable(int64_t q, int64_t k, int64_t v, const char* what, bool debug) {
+  const int64_t mx = std::max(q, std::max(k, v));
+  if ((q != mx && q != 1) || (k != mx && k != 1) || (v != mx && v != 1)) {
+    if (debug)
+      TORCH_WARN("Both fused kernels require query, key and value to have broadcastable ", what, "got Query ", what, q,
+                 ", Key ", what, k, ", Value ", what, v, " instead.");
+    return false;
+  }
+  return true;
+}
+
+bool check_nested_inputs(const sdp_params& p, bool debug) {
+  if (!check_nested_sizes_one(p.query, "query ", debug) || !check_nested_sizes_one(p.key, "key ", debug) ||
+      !check_nested_sizes_one(p.value, "value ", debug))
+    return false;
+  if (!broadcastable(p.query.size(0), p.key.size(0), p.value.size(0), "batch size ", debug)) return false;
+  if (!broadcastable(p.query.size(1), p.key.size(1), p.value.size(1), "num heads ", debug)) return false;
+  if (!p.query.is_cuda() || !p.key.is_cuda() || !p.value.is_cuda()) {
+    if (debug) TORCH_WARN("The flash kernels of this build need all inputs on the HIP device.");
+    return false;
+  }
+  if (!(p.dropout >= 0.0 && p.dropout < 1.0)) {
+    if (debug) TORCH_WARN("The flash kernels of this build need 0 <= dropout_p < 1.");
     return false;
   }
   return true;
@@ -164,10 +219,20 @@ bool check_this_build(const sdp_params& p, bool debug) {
 }
 
 bool use_flash_attention(const sdp_params& p, bool debug) {
-  constexpr std::array<bool (*)(const sdp_params&, bool), 10> constraints{
-      check_runtime_disabled_flash,   check_not_nested,    check_tensor_shapes,
-      check_batch_size_and_num_heads, check_for_attn_mask, check_head_dim_size,
-      check_nonzero_sequence_lengths, check_last_dim_stride_equals_1, check_tensor_dtype, check_this_build};
+  if (has_nested_inputs(p)) {
+    // (sdp_utils.cpp:97-147: the general constraints, then the nested ones; the causal alignment of ragged sequences
+    // is the packed op's bottom-right one, as in PyTorch's own nested path)
+    constexpr std::array<bool (*)(const sdp_params&, bool), 6> nested{
+        check_runtime_disabled_flash, check_tensor_shapes, check_for_attn_mask,
+        check_head_dim_size,          check_tensor_dtype,  check_nested_inputs};
+    for (auto c : nested)
+      if (!c(p, debug)) return false;
+    return true;
+  }
+  constexpr std::array<bool (*)(const sdp_params&, bool), 9> constraints{
+      check_runtime_disabled_flash,   check_tensor_shapes, check_batch_size_and_num_heads,
+      check_for_attn_mask,            check_head_dim_size, check_nonzero_sequence_lengths,
+      check_last_dim_stride_equals_1, check_tensor_dtype,  check_this_build};
   for (auto c : constraints)
     if (!c(p, debug)) return false;
   return true;
