@@ -120,3 +120,32 @@ def test_meta_shape_contract_of_installed_torch():
     cu = torch.empty(3, dtype=torch.int32, device="meta")
     r = torch.ops.aten._flash_attention_forward(p, p, p, cu, cu, 6, 6, 0.0, False, False)
     assert r[0].shape == (10, 4, 64) and r[1].shape == (4, 10)
+
+
+def test_extension_host_code_is_clean_under_ubsan():
+    """fa_aten.cpp + fa_sdp_choice.cpp built with the undefined-behaviour sanitizer (no recovery) and put through the
+    host-side tests of the ops and of the selector in a fresh interpreter: signed overflow, misaligned or null
+    accesses, bad shifts and the like in the argument checks, stride arithmetic and the cum_seq cache abort the run.
+    (The address sanitizer needs its runtime loaded before the interpreter's own libraries and is used on the launchers'
+    host half instead, tests/test_cabi_host.py.)"""
+    import os
+    import shutil
+    import subprocess
+    import sys
+    import tempfile
+
+    if shutil.which("g++") is None:
+        pytest.skip("no host C++ compiler")
+    from torch_mlu_amd import _build
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with tempfile.TemporaryDirectory() as d:
+        lib = _build.build_aten(out=os.path.join(d, "libfa_aten_ubsan.so"),
+                                extra_flags=("-fsanitize=undefined", "-fno-sanitize-recover=all", "-g", "-O1"))
+        env = dict(os.environ, TORCH_MLU_AMD_ATEN_LIB=lib, UBSAN_OPTIONS="print_stacktrace=1:halt_on_error=1")
+        res = subprocess.run([sys.executable, "-m", "pytest", "-x", "-q", "-m", "not gpu", "-p", "no:cacheprovider",
+                              "tests/test_aten_host.py", "tests/test_sdp_choice_host.py",
+                              "--deselect", "tests/test_aten_host.py::test_extension_host_code_is_clean_under_ubsan"],
+                             cwd=root, env=env, capture_output=True, text=True)
+    assert res.returncode == 0, (res.stdout[-1500:], res.stderr[-1500:])
+    assert "runtime error" not in res.stderr

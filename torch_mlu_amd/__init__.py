@@ -18,7 +18,8 @@ import torch
 __version__ = "0.1.0"
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-ATEN_LIB_PATH = os.path.join(_HERE, "lib", "libfa_aten.so")
+# TORCH_MLU_AMD_ATEN_LIB: another build of the same extension (an instrumented one); there is still no fallback
+ATEN_LIB_PATH = os.environ.get("TORCH_MLU_AMD_ATEN_LIB") or os.path.join(_HERE, "lib", "libfa_aten.so")
 KERNEL_LIB_PATH = os.path.join(_HERE, "lib", "libfa_fwd.so")
 
 _loaded = False

@@ -102,14 +102,15 @@ def build_kernels(verbose: bool = False) -> str:
     return out
 
 
-def build_aten(verbose: bool = False) -> str:
+def build_aten(verbose: bool = False, out: str = None, extra_flags=()) -> str:
     """g++: csrc/fa_aten.cpp + csrc/fa_sdp_choice.cpp -> lib/libfa_aten.so (registers the forward and backward aten ops
-    and the SDPA backend selector; links libfa_fwd.so by $ORIGIN)."""
+    and the SDPA backend selector; links libfa_fwd.so by $ORIGIN).  `out` / `extra_flags`: an instrumented build next
+    to the real one (the sanitizer test), which finds libfa_fwd.so through an rpath to lib/."""
     import torch
     from torch.utils import cpp_extension as ce
 
     os.makedirs(LIBDIR, exist_ok=True)
-    out = os.path.join(LIBDIR, "libfa_aten.so")
+    out = out or os.path.join(LIBDIR, "libfa_aten.so")
     tmp = out + ".tmp"
     tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
     inc = [f"-I{p}" for p in ce.include_paths("cuda")] + [f"-I{INCLUDE}"]
@@ -119,7 +120,7 @@ def build_aten(verbose: bool = False) -> str:
         "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
         *inc, os.path.join(CSRC, "fa_aten.cpp"), os.path.join(CSRC, "fa_sdp_choice.cpp"), "-o", tmp,
         f"-L{LIBDIR}", "-lfa_fwd", f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
-        "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}", "-Wl,--no-as-needed",
+        "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{LIBDIR}", f"-Wl,-rpath,{tlib}", "-Wl,--no-as-needed", *extra_flags,
     ]
     log = _run(cmd)
     os.replace(tmp, out)
