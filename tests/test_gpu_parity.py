@@ -331,6 +331,42 @@ def test_packed_equals_per_sequence_dense():
     lse_close(lse.cpu().numpy(), rl)
 
 
+@pytest.mark.parametrize("B,Hq,Hk,D,maxlen,dtype", [(32, 16, 16, 64, 512, HF),    # 8 kv heads at a time, MHA
+                                                    (64, 8, 2, 64, 1024, BF),     # kv heads not a multiple of 8, group 4
+                                                    (40, 32, 8, 128, 300, BF),    # kv heads a multiple of 8, group 4
+                                                    (64, 16, 16, 128, 257, HF)])  # 64 sequences, many of one block
+def test_packed_causal_pairs_equal_per_sequence_dense(B, Hq, Hk, D, maxlen, dtype):
+    """Packed causal calls with enough workgroups are cut into heavy / light block pairs that every workgroup looks up
+    for itself (longest sequence first, kv head fastest).  Ragged lengths with empty sequences, single rows, odd block
+    counts and different query / key lengths: every sequence bit-equal to its own dense call, every row written."""
+    g = torch.Generator().manual_seed(B * 1000 + Hq)
+    lq = torch.randint(1, maxlen + 1, (B,), generator=g).tolist()
+    lq[0], lq[1], lq[2], lq[-1] = maxlen, 0, 1, 129
+    lk = [L + int(x) for L, x in zip(lq, torch.randint(0, 70, (B,), generator=g))]   # keys >= rows: bottom-right causal
+    lk[1] = 0
+    cq = torch.tensor([0] + list(np.cumsum(lq)), dtype=torch.int32)
+    ck = torch.tensor([0] + list(np.cumsum(lk)), dtype=torch.int32)
+    q = seeded((int(cq[-1]), Hq, D), 850, dtype).to(DEV)
+    k, v = seeded((int(ck[-1]), Hk, D), 851, dtype).to(DEV), seeded((int(ck[-1]), Hk, D), 852, dtype).to(DEV)
+    out = torch.full((int(cq[-1]), Hq, D), float("nan"), dtype=dtype, device=DEV)
+    lse = torch.full((Hq, int(cq[-1])), float("nan"), dtype=torch.float32, device=DEV)
+    p = capi.make_params(q, k, v, out, lse, cu_seqlens_q=cq.to(DEV), cu_seqlens_k=ck.to(DEV), max_seqlen_q=max(lq),
+                         max_seqlen_k=max(lk), is_causal=True)
+    capi.launch(p, torch.device(DEV))
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    for b in sorted(range(B), key=lambda i: -lq[i])[:6] + [2, B - 1]:
+        if lq[b] == 0:
+            continue
+        s, e, ks, ke = int(cq[b]), int(cq[b + 1]), int(ck[b]), int(ck[b + 1])
+        o, l = capi.fa_forward_dense(q[s:e].transpose(0, 1)[None], k[ks:ke].transpose(0, 1)[None],
+                                     v[ks:ke].transpose(0, 1)[None], is_causal=True, kernel=capi.FA_KERNEL_TILE128)
+        assert torch.equal(out[s:e], o[0].transpose(0, 1)) and torch.equal(lse[:, s:e], l[0]), b
+    ro, rl = oracle.varlen_oracle(q[:int(cq[3])].cpu(), k[:int(ck[3])].cpu(), v[:int(ck[3])].cpu(), cq[:4], ck[:4],
+                                  is_causal=True)
+    out_close(out[:int(cq[3])].float().cpu().numpy(), ro, dtype)
+    lse_close(lse[:, :int(cq[3])].cpu().numpy(), rl)
+
+
 def test_packed_with_empty_sequences_and_ragged_kv():
     lq, lk = [0, 7, 3, 0, 40], [5, 0, 90, 0, 40]
     cq = torch.tensor([0] + list(np.cumsum(lq)), dtype=torch.int32)
