@@ -11,6 +11,8 @@ from .attention_oracle import (  # noqa: F401
     default_atol,
     default_rtol,
     dropout_keep_mask,
+    dropout_keys,
+    dropout_patch_words,
     get_tolerances,
     sdpa_backward_oracle,
     sdpa_oracle,

@@ -229,6 +229,42 @@ def _mix32(h):
     return h
 
 
+def _mix32_keyed(h, key2):
+    """The same finaliser with `key2` added (mod 2^32) between its two multiplications."""
+    h = h & _M32
+    h ^= h >> np.uint64(16)
+    h = (h * np.uint64(0x85EBCA6B)) & _M32
+    h = ((h ^ (h >> np.uint64(13))) + key2) & _M32
+    h = (h * np.uint64(0xC2B2AE35)) & _M32
+    h ^= h >> np.uint64(16)
+    return h
+
+
+def dropout_keys(seed: int, offset: int, bh: int):
+    """The two 32-bit keys of sequence-and-head index bh = b * heads_q + h for (philox_seed, philox_offset)."""
+    u = np.uint64
+    seed, offset = int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1)
+    k = (_mix32(u((seed & 0xFFFFFFFF) ^ 0x2545F491)) + u(seed >> 32)) & _M32
+    k = _mix32(k) ^ u(offset & 0xFFFFFFFF)
+    k = (_mix32(k) + u(offset >> 32)) & _M32
+    key1 = _mix32(k ^ u((bh * 0x9E3779B1 + 0x7F4A7C15) & 0xFFFFFFFF))
+    m = (_mix32(u((seed >> 32) ^ 0x3C6EF372)) + u(seed & 0xFFFFFFFF)) & _M32
+    m = _mix32(m) ^ u(offset >> 32)
+    m = (_mix32(m) + u(offset & 0xFFFFFFFF)) & _M32
+    key2 = _mix32(m ^ u((bh * 0x85EBCA77 + 0x165667B1) & 0xFFFFFFFF))
+    return key1, key2
+
+
+def dropout_patch_words(key1, key2, rowpairs, colpairs):
+    """Patch words [len(rowpairs), len(colpairs)] for the given row-pair and column-pair indices (uint64 arrays)."""
+    u = np.uint64
+    rp = np.asarray(rowpairs, dtype=np.uint64)[:, None]
+    cp = np.asarray(colpairs, dtype=np.uint64)[None, :]
+    row_term = ((rp << u(16)) & _M32) ^ (((rp >> u(16)) * u(0x9E3779B1)) & _M32)
+    col_term = (cp & u(0xFFFF)) ^ (((cp >> u(16)) * u(0x7F4A7C15)) & _M32)
+    return _mix32_keyed(key1 ^ row_term ^ col_term, key2)
+
+
 def dropout_keep_mask(seed: int, offset: int, bh: int, seqlen_q: int, seqlen_k: int, dropout_p: float) -> np.ndarray:
     """The keep-mask [seqlen_q, seqlen_k] (True = kept) the HIP kernels use for sequence-and-head index
     bh = b * heads_q + h of a call with (philox_seed, philox_offset) = (seed, offset).
@@ -236,19 +272,13 @@ def dropout_keep_mask(seed: int, offset: int, bh: int, seqlen_q: int, seqlen_k: 
     The reference's mask comes out of the closed vendor kernel and cannot be reproduced (its tests only ever feed the
     returned mask back into `attention_ref`, test_scaled_dot_product_attention.py:1049-1070); this restates THIS
     build's definition so that the tests can check that forward, debug mask and backward all use one and the same
-    mask: one 32-bit word per 2 x 2 patch, word = mix(key ^ row_term(row >> 1) ^ col_term(col >> 1)), element kept
-    iff byte 2 (row & 1) + (col & 1) of the word <= floor((1 - p) * 255)."""
+    mask: one 32-bit word per 2 x 2 patch, word = mix(key1 ^ row_term(row >> 1) ^ col_term(col >> 1)) with key2 added
+    between the finaliser's two multiplications, element kept iff byte 2 (row & 1) + (col & 1) of the word
+    <= floor((1 - p) * 255)."""
     u = np.uint64
-    seed, offset = int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1)
-    k = (_mix32(u((seed & 0xFFFFFFFF) ^ 0x2545F491)) + u(seed >> 32)) & _M32
-    k = _mix32(k) ^ u(offset & 0xFFFFFFFF)
-    k = (_mix32(k) + u(offset >> 32)) & _M32
-    key = _mix32(k ^ u((bh * 0x9E3779B1 + 0x7F4A7C15) & 0xFFFFFFFF))
-    rp = (np.arange(seqlen_q, dtype=np.uint64) >> u(1))[:, None]
-    cp = (np.arange(seqlen_k, dtype=np.uint64) >> u(1))[None, :]
-    row_term = ((rp << u(16)) & _M32) ^ (((rp >> u(16)) * u(0x9E3779B1)) & _M32)
-    col_term = (cp & u(0xFFFF)) ^ (((cp >> u(16)) * u(0x7F4A7C15)) & _M32)
-    word = _mix32(key ^ row_term ^ col_term)
+    key1, key2 = dropout_keys(seed, offset, bh)
+    word = dropout_patch_words(key1, key2, np.arange(seqlen_q, dtype=np.uint64) >> u(1),
+                               np.arange(seqlen_k, dtype=np.uint64) >> u(1))
     sel = (u(2) * (np.arange(seqlen_q, dtype=np.uint64) & u(1)))[:, None] + (np.arange(seqlen_k, dtype=np.uint64) & u(1))[None, :]
     byte = (word >> (u(8) * sel)) & u(0xFF)
     # the threshold is formed in float32, as the launcher does from its float dropout_p

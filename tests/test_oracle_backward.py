@@ -198,6 +198,35 @@ def test_dropout_mask_restatement_properties():
     assert abs(oracle.dropout_keep_mask(1, 0, 0, 512, 512, 0.6).mean() - 102 / 256) < 5e-3
 
 
+def test_dropout_masks_of_two_heads_are_not_translates():
+    """With a single key XORed into the patch counter, head h' would see head h's word table with its row-pair and
+    column-pair indices XORed by the constant key(h) ^ key(h'); the second key breaks that.  Checked on the word
+    function itself, at the translated positions, for several head pairs and both key paths (seed, offset)."""
+    rp = np.arange(0, 256, dtype=np.uint64)
+    cp = np.arange(0, 256, dtype=np.uint64)
+    for (s0, o0, bh0), (s1, o1, bh1) in (((7, 0, 0), (7, 0, 1)), ((7, 0, 5), (7, 0, 77)), ((7, 0, 3), (7, 4, 3)),
+                                         ((7, 0, 3), (8, 0, 3)), ((2 ** 40 + 1, 2 ** 33, 9), (2 ** 40 + 1, 2 ** 33, 10))):
+        k1a, k2a = oracle.dropout_keys(s0, o0, bh0)
+        k1b, k2b = oracle.dropout_keys(s1, o1, bh1)
+        assert k1a != k1b and k2a != k2b
+        delta = int(k1a) ^ int(k1b)
+        wa = oracle.dropout_patch_words(k1a, k2a, rp, cp)
+        # head b at the positions that the XOR by delta maps onto head a's: counter_b = counter_a
+        wb = oracle.dropout_patch_words(k1b, k2b, rp ^ np.uint64(delta >> 16), cp ^ np.uint64(delta & 0xFFFF))
+        assert (wa == wb).mean() < 1e-3
+        # and their bytes agree as often as independent bytes do
+        agree = ((wa & np.uint64(0xFF)) == (wb & np.uint64(0xFF))).mean()
+        assert agree < 3e-2
+
+
+def test_dropout_mean_keep_rate_over_thresholds_and_heads():
+    """Realised keep rate = (floor((1 - p) 255) + 1) / 256 for every p, pooled over heads."""
+    for p in (0.001, 0.1, 0.5, 0.9):
+        want = (int(np.floor((np.float32(1.0) - np.float32(p)) * np.float32(255.0))) + 1) / 256
+        got = np.mean([oracle.dropout_keep_mask(11, 16, bh, 256, 256, p).mean() for bh in range(8)])
+        assert abs(got - want) < 3e-3, (p, got, want)
+
+
 # ---- additive bias, top-left causal mask, gradient of the bias (the mem-efficient backward's additions) -------------
 @pytest.mark.parametrize("causal_tl", [False, True])
 @pytest.mark.parametrize("bshape", ["full", "row", "head"])

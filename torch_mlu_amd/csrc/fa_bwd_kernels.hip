@@ -300,9 +300,12 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
   const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
   // dropout: the forward's mask, regenerated (same patch words, same lane layout as the forward's scores)
-  uint32_t drop_row = 0;
-  if constexpr (DROP)
-    drop_row = drop_head_key((uint64_t)*a.seed_ptr, (uint64_t)*a.offset_ptr, (uint32_t)bh) ^ drop_row_term((uint32_t)row >> 1);
+  uint32_t drop_row = 0, drop_key2 = 0;
+  if constexpr (DROP) {
+    const DropKeys dk = drop_head_keys((uint64_t)*a.seed_ptr, (uint64_t)*a.offset_ptr, (uint32_t)bh);
+    drop_row = dk.k1 ^ drop_row_term((uint32_t)row >> 1);
+    drop_key2 = dk.k2;
+  }
   const int drop_sh = 16 * (row & 1);
   // bias / dBias of this lane's row, at its first key group (4 g)
   const unsigned char* brow = nullptr;
@@ -446,7 +449,7 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
         uint32_t word = 0;
         if constexpr (DROP) {
           const int v0 = 8 * (t & 1) + 2 * e2;
-          word = drop_mix(drop_tile ^ (uint32_t)(16 * (t >> 1) + 4 * (v0 >> 2) + ((v0 & 3) >> 1))) >> drop_sh;
+          word = drop_word(drop_tile ^ (uint32_t)(16 * (t >> 1) + 4 * (v0 >> 2) + ((v0 & 3) >> 1)), drop_key2) >> drop_sh;
         }
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
@@ -760,10 +763,12 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
     if (a.is_causal && qlo + BQ - 1 + off < wave_kv_lo) continue;
     // dropout: key of this iteration's query head ^ column term ^ row term of the tile's first row pair (+ 2 g);
     // the row pair of registers (v, v + 1) adds a compile-time constant with disjoint bits
-    uint32_t drop_tile = 0;
-    if constexpr (DROP)
-      drop_tile = drop_head_key(drop_seed, drop_offset, (uint32_t)(b * a.heads_q + hk * a.group + it / nq)) ^ drop_col ^
-                  drop_row_term((uint32_t)(qlo / 2 + 2 * g));
+    uint32_t drop_tile = 0, drop_key2 = 0;
+    if constexpr (DROP) {
+      const DropKeys dk = drop_head_keys(drop_seed, drop_offset, (uint32_t)(b * a.heads_q + hk * a.group + it / nq));
+      drop_tile = dk.k1 ^ drop_col ^ drop_row_term((uint32_t)(qlo / 2 + 2 * g));
+      drop_key2 = dk.k2;
+    }
 
     const unsigned char* qt = smem + buf * TILE;
     const unsigned char* dt = smem + 2 * TILE + buf * TILE;
@@ -844,7 +849,7 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
           float p0 = fast_exp2(s2[qbk][v] * c - l0), p1 = fast_exp2(s2[qbk][v + 1] * c - l1);
           if constexpr (DROP) {
             const uint32_t rp_const = 16 * qbk + 4 * (v >> 2) + ((v & 3) >> 1);
-            const uint32_t word = drop_mix(drop_tile ^ (rp_const << 16)) >> drop_sh;
+            const uint32_t word = drop_word(drop_tile ^ (rp_const << 16), drop_key2) >> drop_sh;
             p0 = ((word & 0xffu) <= a.drop_thr) ? p0 * a.drop_rp : 0.f;
             p1 = (((word >> 16) & 0xffu) <= a.drop_thr) ? p1 * a.drop_rp : 0.f;
           }
@@ -959,7 +964,7 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
           float pv0 = p0, pv1 = p1;  // what multiplies dO in dV: P o M / (1 - p)
           if constexpr (DROP) {
             const uint32_t rp_const = 16 * qbk + 4 * (v >> 2) + ((v & 3) >> 1);
-            const uint32_t word = drop_mix(drop_tile ^ (rp_const << 16)) >> drop_sh;
+            const uint32_t word = drop_word(drop_tile ^ (rp_const << 16), drop_key2) >> drop_sh;
             const bool k0 = (word & 0xffu) <= a.drop_thr, k1 = ((word >> 16) & 0xffu) <= a.drop_thr;
             pv0 = k0 ? p0 * a.drop_rp : 0.f;
             pv1 = k1 ? p1 * a.drop_rp : 0.f;

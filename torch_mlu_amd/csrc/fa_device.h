@@ -140,7 +140,10 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
 // probability iff byte 2 (row & 1) + (col & 1) of the patch's word is <= the threshold.  The word is a murmur3
 // finaliser over a counter that is unique per patch while both pair indices are below 65536 (beyond that the high
 // parts are folded in), so forward and backward — whose lanes own different elements — regenerate the same mask from
-// (seed, offset, sequence, head, row, col) alone.
+// (seed, offset, sequence, head, row, col) alone.  A (sequence, head) has two 32-bit keys: the first is XORed into the
+// counter, the second is added between the finaliser's two multiplications, so the masks of two heads are not
+// translates of one another (with the first key alone, head h' would see head h's table with its row and column pair
+// indices XORed by a constant).
 __device__ __forceinline__ uint32_t drop_mix(uint32_t h) {
   h ^= h >> 16;
   h *= 0x85ebca6bu;
@@ -149,12 +152,27 @@ __device__ __forceinline__ uint32_t drop_mix(uint32_t h) {
   h ^= h >> 16;
   return h;
 }
-// key of one (sequence b, query head h) of one call: bh = b * heads_q + h
-__device__ __forceinline__ uint32_t drop_head_key(uint64_t seed, uint64_t offset, uint32_t bh) {
+__device__ __forceinline__ uint32_t drop_word(uint32_t counter, uint32_t key2) {
+  uint32_t h = counter;
+  h ^= h >> 16;
+  h *= 0x85ebca6bu;
+  h = (h ^ (h >> 13)) + key2;
+  h *= 0xc2b2ae35u;
+  h ^= h >> 16;
+  return h;
+}
+// keys of one (sequence b, query head h) of one call: bh = b * heads_q + h
+struct DropKeys {
+  uint32_t k1, k2;
+};
+__device__ __forceinline__ DropKeys drop_head_keys(uint64_t seed, uint64_t offset, uint32_t bh) {
   uint32_t k = drop_mix((uint32_t)seed ^ 0x2545f491u) + (uint32_t)(seed >> 32);
   k = drop_mix(k) ^ (uint32_t)offset;
   k = drop_mix(k) + (uint32_t)(offset >> 32);
-  return drop_mix(k ^ (bh * 0x9e3779b1u + 0x7f4a7c15u));
+  uint32_t m = drop_mix((uint32_t)(seed >> 32) ^ 0x3c6ef372u) + (uint32_t)seed;
+  m = drop_mix(m) ^ (uint32_t)(offset >> 32);
+  m = drop_mix(m) + (uint32_t)offset;
+  return DropKeys{drop_mix(k ^ (bh * 0x9e3779b1u + 0x7f4a7c15u)), drop_mix(m ^ (bh * 0x85ebca77u + 0x165667b1u))};
 }
 // the part of a patch's counter that depends on its row pair / on its column pair; the counter is their XOR with the key
 __device__ __forceinline__ uint32_t drop_row_term(uint32_t rowpair) { return (rowpair << 16) ^ ((rowpair >> 16) * 0x9e3779b1u); }

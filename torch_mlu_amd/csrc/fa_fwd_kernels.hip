@@ -149,12 +149,14 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   }
   const int h = bh % a.heads_q, b = bh / a.heads_q;
   const int hk = h / a.group;
-  uint32_t drop_key = 0;
+  uint32_t drop_key = 0, drop_key2 = 0;
   if constexpr (DROP) {
     // the two numbers of the mask: by value, or (a launch recorded into a graph) read now from the generator's state
     const uint64_t seed = a.seed_ptr ? (uint64_t)*a.seed_ptr : a.seed;
     const uint64_t offset = a.offset_ptr ? (uint64_t)*a.offset_ptr + a.offset : a.offset;
-    drop_key = drop_head_key(seed, offset, (uint32_t)bh);
+    const DropKeys dk = drop_head_keys(seed, offset, (uint32_t)bh);
+    drop_key = dk.k1;
+    drop_key2 = dk.k2;
     if (blockIdx.x == 0 && tid == 0) {
       if (a.rng_seed_out) *a.rng_seed_out = (int64_t)seed;
       if (a.rng_offset_out) *a.rng_offset_out = (int64_t)offset;
@@ -500,7 +502,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
         if constexpr (DROP) {
           // keys j BN + 32 (t >> 1) + 8 (v >> 2) + 4 g + (v & 3), + 1: one column pair, one patch word
           const uint32_t cp_const = 16 * (t >> 1) + 4 * (v >> 2) + ((v & 3) >> 1);
-          const uint32_t word = drop_mix(drop_tile ^ cp_const) >> drop_sh;
+          const uint32_t word = drop_word(drop_tile ^ cp_const, drop_key2) >> drop_sh;
           const bool k0 = (word & 0xffu) <= a.drop_thr, k1 = ((word >> 8) & 0xffu) <= a.drop_thr;
           if (DMASK && a.dmask) {
             const int col = j * BN + 32 * (t >> 1) + 8 * (v >> 2) + 4 * g + (v & 3);
