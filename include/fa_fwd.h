@@ -119,8 +119,9 @@ typedef struct fa_fwd_params {
   const void* bias;  /* device or NULL */
   int64_t bias_stride_b, bias_stride_h, bias_stride_q;
 
-  /* dropout on the softmax probabilities (tile kernel only; 0 = off).  The mask is a pure function of
-     (philox_seed, philox_offset, sequence, query head, row, col), so the backward regenerates it from the two numbers. */
+  /* dropout on the softmax probabilities (0 = off; both forward kernels).  The mask is a pure function of
+     (philox_seed, philox_offset, sequence, query head, row, col), so the backward regenerates it from the two numbers
+     and the tile and split-KV kernels drop the same elements. */
   float dropout_p;         /* 0 <= p < 1.  An element is kept iff one byte of a hash word is <= floor((1 - p) 255), i.e.
                               with probability (floor((1 - p) 255) + 1) / 256, and kept elements are scaled by
                               1 / (1 - p) exactly as the reference's oracle scales them: the expectation of the output
@@ -133,7 +134,9 @@ typedef struct fa_fwd_params {
   void* dropout_mask;      /* device or NULL: debug output, dense [batch][heads_q][seqlen_q][seqlen_k] elements of
                               `dtype`, +1 kept / -1 dropped, positions outside a sequence or masked left untouched
                               (packed mode: seqlen_q / seqlen_k are the maxima, rows and keys count from each
-                              sequence's start, as FlashAttention_internal.cpp:141-146 shapes it) */
+                              sequence's start, as FlashAttention_internal.cpp:141-146 shapes it).  Written by the
+                              tile kernel only: a call that wants it is planned onto the tile kernel, and with
+                              kernel = FA_KERNEL_SPLITKV or a page table it is FA_ERR_UNSUPPORTED */
   /* optional (NULL = all of them): device int32[batch]; only the first min(seqused_k[b], its length) keys of sequence b
      exist — a KV cache that is allocated to seqlen_k rows but filled to a per-sequence length (the `seqused_k` of
      aten::_flash_attention_forward, the `seqlen_k` of aten::_efficient_attention_forward).  The causal mask aligns to
@@ -147,7 +150,7 @@ typedef struct fa_fwd_params {
   const int64_t* philox_seed_ptr;
   const int64_t* philox_offset_ptr;
   /* optional paged KV cache (NULL = k / v are per-sequence tensors as above).  Dense mode, split-KV kernel only
-     (seqlen_q x heads_q / heads_k <= 16, no bias, no dropout, not top-left causal; anything else: FA_ERR_UNSUPPORTED).
+     (seqlen_q x heads_q / heads_k <= 16, no bias, no dropout_mask, not top-left causal; anything else: FA_ERR_UNSUPPORTED).
      k and v then point at pools of pages, [page][row in page][kv head][head_dim]: k_stride_b / v_stride_b are the
      element strides between pages, k_stride_s / v_stride_s between the rows of a page.  Key row r of sequence b lives
      in page block_table[b * block_table_stride + r / page_size] at row r % page_size.  seqlen_k is the longest

@@ -212,3 +212,120 @@ def test_dropout_under_graph_capture_draws_a_new_mask_per_replay():
         eager = aten._scaled_dot_product_flash_attention(qd, kd, vd, 0.0, True, False)[0]
         assert torch.isfinite(eager.float()).all()
     assert len({o for _, o in seen}) == 3 and len({s for s, _ in seen}) == 1
+
+
+def _plan_of(q, k, v, **kw):
+    import ctypes
+    B, Hq, Sq, D = q.shape
+    out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    p = capi.make_params(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), out, lse, **kw)
+    kern, ns = ctypes.c_int32(), ctypes.c_int32()
+    assert capi.lib().fa_fwd_plan(ctypes.byref(p), ctypes.byref(kern), ctypes.byref(ns)) == capi.FA_OK
+    return kern.value, ns.value
+
+
+@pytest.mark.parametrize("dtype,D", [(BF, 128), (HF, 64), (BF, 256), (HF, 72)])
+@pytest.mark.parametrize("Sq,group,causal", [(1, 4, False), (4, 4, True), (3, 1, True), (16, 1, False), (1, 16, False)])
+def test_split_kv_kernel_drops_the_same_elements_as_the_tile_kernel(dtype, D, Sq, group, causal):
+    """Few query rows against a long K/V with dropout run the split-KV kernel (the plan says so); its mask is the
+    documented function — the oracle fed with that mask agrees —, LSE ignores it, forced slice counts (merge kernel)
+    agree, and the tile kernel asked for by name gives the same answer.  A call that wants the debug mask is planned
+    onto the tile kernel."""
+    B, Hk, Sk, p = 2, 2, 700, 0.3
+    Hq = Hk * group
+    q, k, v, _ = _inputs(B, Hq, Hk, Sq, Sk, D, dtype, 900 + D + Sq + group)
+    qd, kd, vd = (t.to(DEV) for t in (q, k, v))
+    seed, offset = 0x0BAD_5EED_0000_0001 + D, 8 * Sq + (group << 36)
+    assert _plan_of(qd, kd, vd, is_causal=causal, dropout_p=p, philox_seed=seed, philox_offset=offset)[0] == capi.FA_KERNEL_SPLITKV
+    dm = torch.zeros(B, Hq, Sq, Sk, dtype=dtype, device=DEV)
+    assert _plan_of(qd, kd, vd, is_causal=causal, dropout_p=p, philox_seed=seed, philox_offset=offset,
+                    dropout_mask=dm)[0] == capi.FA_KERNEL_TILE
+    keep = _expected_mask(seed, offset, B, Hq, Sq, Sk, p)
+    ro, rl = oracle.sdpa_oracle(q, k, v, is_causal=causal, dropout_p=p, dropout_mask=keep)
+    tol = 2 * EPS[dtype] * max(1.0, float(np.abs(ro).max()))
+    outs = []
+    for ns in (0, 1, 3):
+        rng = torch.zeros(2, dtype=torch.int64, device=DEV)
+        out, lse = capi.fa_forward_dense(qd, kd, vd, is_causal=causal, dropout_p=p, philox_seed=seed,
+                                         philox_offset=offset, rng_out=rng, kernel=capi.FA_KERNEL_SPLITKV, num_splits=ns)
+        assert rng.tolist() == [seed, offset]
+        out_close(out.float().cpu().numpy(), ro, dtype, tol=tol)
+        lse_close(lse.cpu().numpy(), rl)
+        outs.append(out)
+    out_t, lse_t = capi.fa_forward_dense(qd, kd, vd, is_causal=causal, dropout_p=p, philox_seed=seed,
+                                         philox_offset=offset, kernel=capi.FA_KERNEL_TILE)
+    out_close(out_t.float().cpu().numpy(), ro, dtype, tol=tol)
+    # both kernels drop the same elements: their outputs differ by rounding only (a different mask would move them
+    # by whole probabilities)
+    assert (out_t.float() - outs[1].float()).abs().max().item() <= tol
+    # and without dropout the split-KV kernel's answer is another one
+    plain, _ = capi.fa_forward_dense(qd, kd, vd, is_causal=causal, kernel=capi.FA_KERNEL_SPLITKV)
+    assert (plain.float() - outs[1].float()).abs().max().item() > 2 * tol
+
+
+def test_split_kv_dropout_paged_packed_and_through_the_op():
+    """Dropout on the split-KV kernel with a paged cache (bit-equal to the contiguous cache: same keys, same mask), in
+    packed mode (one query row per sequence, rows and keys counted from each sequence's start), and through
+    F.scaled_dot_product_attention in training mode on a decode-shaped call (forward on the split-KV kernel, backward
+    regenerates the mask)."""
+    from tests.test_gpu_paged import _paged_case
+    B, Hq, Hk, Sq, D, page, p = 3, 8, 2, 2, 128, 64, 0.25
+    lens = [5 * page + 17, page, 300]
+    q, kp, vp, table, used, kf, vf = _paged_case(B, Hq, Hk, Sq, D, page, lens, BF, 31)
+    qd, kpd, vpd, td, ud, kfd, vfd = (t.to(DEV) for t in (q, kp, vp, table, used, kf, vf))
+    seed, offset = 77, 1 << 33
+    # capi.fa_forward_paged has no dropout arguments: fill the block by hand
+    out_p = torch.empty((B, Sq, Hq, D), dtype=BF, device=DEV)
+    lse_p = torch.empty((B, Hq, Sq), dtype=torch.float32, device=DEV)
+    pp = capi.make_params(qd.transpose(1, 2), kpd, vpd, out_p, lse_p, is_causal=True, seqused_k=ud, dropout_p=p,
+                          philox_seed=seed, philox_offset=offset)
+    pp.seqlen_k = table.shape[1] * page
+    pp.block_table, pp.block_table_stride, pp.page_size = td.data_ptr(), td.stride(0), page
+    capi.launch(pp, torch.device(DEV))
+    out_c, lse_c = capi.fa_forward_dense(qd, kfd, vfd, is_causal=True, dropout_p=p, philox_seed=seed, philox_offset=offset,
+                                         kernel=capi.FA_KERNEL_SPLITKV, seqused_k=ud)
+    assert torch.equal(out_p.transpose(1, 2), out_c) and torch.equal(lse_p, lse_c)
+    for b in range(B):
+        keep = _expected_mask(seed, offset, B, Hq, Sq, lens[b], p)[b:b + 1]
+        ro, rl = oracle.sdpa_oracle(q[b:b + 1], kf[b:b + 1, :, :lens[b]], vf[b:b + 1, :, :lens[b]], is_causal=True,
+                                    dropout_p=p, dropout_mask=keep)
+        out_close(out_c[b:b + 1].float().cpu().numpy(), ro, BF, tol=2 * EPS[BF] * max(1.0, float(np.abs(ro).max())))
+        lse_close(lse_c[b:b + 1].cpu().numpy(), rl)
+
+    # packed: one query row per sequence
+    lens_k = [300, 0, 1000, 257]
+    cu_q = torch.tensor([0, 1, 2, 3, 4], dtype=torch.int32, device=DEV)
+    cu_k = torch.tensor(np.concatenate([[0], np.cumsum(lens_k)]), dtype=torch.int32, device=DEV)
+    Hq2, Hk2, D2 = 8, 2, 64
+    qk = seeded((4, Hq2, D2), 51, HF); kk = seeded((sum(lens_k), Hk2, D2), 52, HF); vk = seeded((sum(lens_k), Hk2, D2), 53, HF)
+    rng = torch.zeros(2, dtype=torch.int64, device=DEV)
+    out_k, lse_k = capi.fa_forward_packed(qk.to(DEV), kk.to(DEV), vk.to(DEV), cu_q, cu_k, 1, max(lens_k), dropout_p=p,
+                                          philox_seed=seed, philox_offset=offset, rng_out=rng, kernel=capi.FA_KERNEL_SPLITKV)
+    assert rng.tolist() == [seed, offset]
+    ck = cu_k.cpu().numpy()
+    for b, n in enumerate(lens_k):
+        if n == 0:
+            assert out_k[b].abs().max().item() == 0
+            continue
+        keep = np.stack([oracle.dropout_keep_mask(seed, offset, b * Hq2 + h, 1, n, p) for h in range(Hq2)])[None]
+        ro, rl = oracle.sdpa_oracle(qk[b:b + 1].transpose(0, 1)[None], kk[ck[b]:ck[b + 1]].transpose(0, 1)[None],
+                                    vk[ck[b]:ck[b + 1]].transpose(0, 1)[None], dropout_p=p, dropout_mask=keep)
+        out_close(out_k[b:b + 1].transpose(0, 1)[None].float().cpu().numpy(), ro, HF,
+                  tol=2 * EPS[HF] * max(1.0, float(np.abs(ro).max())))
+
+    # the op: a decode-shaped training call
+    torch.manual_seed(5)
+    qo, ko, vo = (seeded(s, 60 + i, BF).to(DEV).requires_grad_() for i, s in enumerate([(2, 8, 2, 64), (2, 2, 512, 64), (2, 2, 512, 64)]))
+    n0 = torch_mlu_amd.launch_count()
+    res = aten._scaled_dot_product_flash_attention(qo, ko, vo, 0.2, False, False)
+    out_o, lse_o, sd, of = res[0], res[1], res[6], res[7]
+    assert torch_mlu_amd.launch_count() == n0 + 1
+    keep = _expected_mask(int(sd), int(of), 2, 8, 2, 512, 0.2)
+    ro, _ = oracle.sdpa_oracle(qo.detach().cpu(), ko.detach().cpu(), vo.detach().cpu(), dropout_p=0.2, dropout_mask=keep)
+    out_close(out_o.float().detach().cpu().numpy(), ro, BF, tol=2 * EPS[BF] * max(1.0, float(np.abs(ro).max())))
+    do = seeded((2, 8, 2, 64), 70, BF).to(DEV)
+    out_o.backward(do)
+    want = oracle.sdpa_backward_oracle(qo.detach().cpu(), ko.detach().cpu(), vo.detach().cpu(), do.cpu(), dropout_p=0.2,
+                                       dropout_mask=keep)
+    _grad_check((qo.grad, ko.grad, vo.grad), want, BF)

@@ -626,7 +626,7 @@ struct SplitCfg {
   static constexpr int LDS = NW * RING;
 };
 
-template <typename T, int DP>
+template <typename T, int DP, bool DROP = false>
 __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(const KArgs a) {
   constexpr int NW = SplitCfg<DP>::NW;
   constexpr int CPR = DP / 8;
@@ -671,6 +671,20 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
   // keys this lane's slot may see: bottom-right causal lets row r see keys <= Lk - Lq + r
   const int slot_lim = a.is_causal ? min(Lk - 1, Lk - Lq + slot_r) : Lk - 1;
   const int mask_from = a.is_causal ? Lk - (Lq - 1) : Lk;  // first key that some slot does not see
+  // dropout: the tile kernel's mask (same patch words): this lane's slot is one (head, row), its registers are keys
+  uint32_t drop_row = 0, drop_key2 = 0;
+  const int drop_sh = 16 * (slot_r & 1);
+  if constexpr (DROP) {
+    const uint64_t seed = a.seed_ptr ? (uint64_t)*a.seed_ptr : a.seed;
+    const uint64_t offset = a.offset_ptr ? (uint64_t)*a.offset_ptr + a.offset : a.offset;
+    const DropKeys dk = drop_head_keys(seed, offset, (uint32_t)(b * a.heads_q + h0 + slot_g));
+    drop_row = dk.k1 ^ drop_row_term((uint32_t)slot_r >> 1);
+    drop_key2 = dk.k2;
+    if (blockIdx.x == 0 && tid == 0) {
+      if (a.rng_seed_out) *a.rng_seed_out = (int64_t)seed;
+      if (a.rng_offset_out) *a.rng_offset_out = (int64_t)offset;
+    }
+  }
 
   // slice of 32-row blocks owned by this workgroup, then by this wavefront (interleaved)
   const int nblk = (Lk + 31) >> 5;
@@ -807,6 +821,25 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
     l_run = l_run * alpha + rs;
 #pragma unroll
     for (int i = 0; i < MB; ++i) o[i] *= alpha;
+    if constexpr (DROP) {
+      // row sums are those of the undropped probabilities.  Registers (2 pr, 2 pr + 1) of sa / sb hold keys
+      // 32 blk + 16 half + 4 G + 2 pr, + 1: column pair 16 blk + 8 half + 2 G + pr
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr) {
+          const uint32_t cp = (uint32_t)(16 * blk + 8 * half + 2 * G + pr);
+          const uint32_t word = drop_word(drop_row ^ drop_col_term(cp), drop_key2) >> drop_sh;
+          const bool k0 = (word & 0xffu) <= a.drop_thr, k1 = ((word >> 8) & 0xffu) <= a.drop_thr;
+          if (half) {
+            sb[2 * pr] = k0 ? sb[2 * pr] : 0.f;
+            sb[2 * pr + 1] = k1 ? sb[2 * pr + 1] : 0.f;
+          } else {
+            sa[2 * pr] = k0 ? sa[2 * pr] : 0.f;
+            sa[2 * pr + 1] = k1 ? sa[2 * pr + 1] : 0.f;
+          }
+        }
+    }
 
     u32x4 w;
     w[0] = Mma<T>::pack2(sa[0], sa[1]);
@@ -865,7 +898,7 @@ __global__ void __launch_bounds__(SplitCfg<DP>::NW * 64, 1) fa_splitkv_kernel(co
     const int qr = qs / group;  // query row of this slot (0 in packed mode)
     const int h = h0 + qs % group;
     if (a.n_splits == 1) {
-      const float inv = (lsum > 0.f) ? 1.f / lsum : 0.f;
+      const float inv = (lsum > 0.f) ? (DROP ? a.drop_rp : 1.f) / lsum : 0.f;
       if (d0 < D) {
         unsigned char* orow = a.out + ob + (int64_t)(q0 + qr) * a.o_ss + (int64_t)h * a.o_sh + d0 * 2;
         u32x4 w0, w1;
@@ -946,7 +979,7 @@ __global__ void __launch_bounds__(256) fa_merge_rows_kernel(const KArgs a) {
       if (d < D) acc[i] += po[(int64_t)s * D + d] * sc;
     }
   }
-  const float inv = (lsum > 0.f) ? 1.f / lsum : 0.f;
+  const float inv = (lsum > 0.f) ? a.drop_rp / lsum : 0.f;  // 1 / (1 - p): the split-KV kernel's partials under dropout
   T* orow = (T*)(a.out + orow_off + (int64_t)h * a.o_sh);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -1042,10 +1075,10 @@ int launch_tile(KArgs a, hipStream_t st) {
   return FA_OK;
 }
 
-template <typename T, int DP>
+template <typename T, int DP, bool DROP>
 int launch_splitkv(const KArgs& a, hipStream_t st) {
   constexpr int lds = SplitCfg<DP>::LDS;
-  constexpr auto kfn = fa_splitkv_kernel<T, DP>;
+  constexpr auto kfn = fa_splitkv_kernel<T, DP, DROP>;
   if (!ensure_dynamic_lds<kfn>(lds)) return FA_ERR_LAUNCH;
   const int64_t grid = (int64_t)a.batch * a.heads_k * a.n_splits;
   if (grid > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
@@ -1063,9 +1096,14 @@ template <typename T>
 int dispatch(const KArgs& a, int kern, hipStream_t st) {
   const int dp = padded_dim(a.head_dim);
   if (kern == FA_KERNEL_SPLITKV) {
-    if (dp == 64) return launch_splitkv<T, 64>(a, st);
-    if (dp == 128) return launch_splitkv<T, 128>(a, st);
-    return launch_splitkv<T, 256>(a, st);
+    if (a.drop_thr < 255u) {  // dropout_p > 0
+      if (dp == 64) return launch_splitkv<T, 64, true>(a, st);
+      if (dp == 128) return launch_splitkv<T, 128, true>(a, st);
+      return launch_splitkv<T, 256, true>(a, st);
+    }
+    if (dp == 64) return launch_splitkv<T, 64, false>(a, st);
+    if (dp == 128) return launch_splitkv<T, 128, false>(a, st);
+    return launch_splitkv<T, 256, false>(a, st);
   }
   if (a.drop_thr < 255u && a.dmask) {  // dropout_p > 0 and the keep-mask is wanted (tests)
     if (a.bias) {

@@ -59,7 +59,7 @@ inline int validate(const fa_fwd_params* p) {
   if (p->is_causal < FA_MASK_NONE || p->is_causal > FA_MASK_CAUSAL_TOP_LEFT) return FA_ERR_BAD_ARG;
   if (p->reserved2 != 0 || !(p->dropout_p >= 0.f && p->dropout_p < 1.f)) return FA_ERR_BAD_ARG;
   if (p->dropout_p > 0.f) {
-    if (p->kernel == FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
+    if (p->kernel == FA_KERNEL_SPLITKV && p->dropout_mask) return FA_ERR_UNSUPPORTED;  // only the tile kernel writes the debug mask
     if (p->dropout_mask && ((uintptr_t)p->dropout_mask & 3)) return FA_ERR_BAD_ARG;
     if (((uintptr_t)p->rng_seed_out | (uintptr_t)p->rng_offset_out) & 7) return FA_ERR_BAD_ARG;
     if (((uintptr_t)p->philox_seed_ptr | (uintptr_t)p->philox_offset_ptr) & 7) return FA_ERR_BAD_ARG;
@@ -73,7 +73,7 @@ inline int validate(const fa_fwd_params* p) {
     if (p->page_size <= 0 || p->block_table_stride < 0) return FA_ERR_BAD_ARG;
     if (p->page_size % 32) return FA_ERR_UNSUPPORTED;
     if (p->block_table_stride < ((int64_t)p->seqlen_k + p->page_size - 1) / p->page_size) return FA_ERR_BAD_ARG;
-    if (p->cu_seqlens_q || p->bias || p->dropout_p > 0.f || p->is_causal == FA_MASK_CAUSAL_TOP_LEFT)
+    if (p->cu_seqlens_q || p->bias || (p->dropout_p > 0.f && p->dropout_mask) || p->is_causal == FA_MASK_CAUSAL_TOP_LEFT)
       return FA_ERR_UNSUPPORTED;
     if (p->kernel != FA_KERNEL_AUTO && p->kernel != FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
     if (p->seqlen_q < 1 || (int64_t)p->seqlen_q * (p->heads_q / p->heads_k) > 16) return FA_ERR_UNSUPPORTED;
@@ -98,7 +98,7 @@ inline void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   if (kern == FA_KERNEL_TILE128 || kern == FA_KERNEL_TILE256 || kern == FA_KERNEL_TILE256W) kern = FA_KERNEL_TILE;  // the family; tile_rows() picks
   if (p->block_table) kern = FA_KERNEL_SPLITKV;  // the only kernel that reads a page table (validate() checked the shape)
   if (kern == FA_KERNEL_AUTO)
-    kern = (p->seqlen_q >= 1 && (int64_t)p->seqlen_q * group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT && !(p->dropout_p > 0.f))
+    kern = (p->seqlen_q >= 1 && (int64_t)p->seqlen_q * group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT && !(p->dropout_p > 0.f && p->dropout_mask))
                ? FA_KERNEL_SPLITKV
                : FA_KERNEL_TILE;
   int ns = 1;
