@@ -298,6 +298,18 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dq_kernel(const 
   for (int i = 0; i < MB; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+  if constexpr (DP == 256) {
+    // One wavefront per SIMD, 512 registers: of those only 256 are vector registers proper.  The operands that
+    // nothing but MFMAs touch (the Q and dO fragments, the dQ accumulators: 256 registers) are sent to the
+    // accumulation half here, which leaves the vector half to the scores.
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      asm volatile("" : "+a"(qf[ks]));
+      asm volatile("" : "+a"(dof[ks]));
+    }
+#pragma unroll
+    for (int i = 0; i < MB; ++i) asm volatile("" : "+a"(acc[i]));
+  }
   const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
   // dropout: the forward's mask, regenerated (same patch words, same lane layout as the forward's scores)
   uint32_t drop_row = 0, drop_key2 = 0;
@@ -763,6 +775,17 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
   for (int i = 0; i < MB; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) { dk[i][v] = 0.f; dv[i][v] = 0.f; }
+  if constexpr (DP == 256 && DO_K) {
+    // as in the dQ kernel: the K and V fragments and the dK accumulators (256 registers that only MFMAs touch) go to
+    // the accumulation half of the 512 registers a lone wavefront per SIMD has
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      asm volatile("" : "+a"(kf[ks]));
+      asm volatile("" : "+a"(vf[ks]));
+    }
+#pragma unroll
+    for (int i = 0; i < MB; ++i) asm volatile("" : "+a"(dk[i]));
+  }
 
   for (int it = 0; it < niter; ++it) {
     const int buf = it & 1;
