@@ -372,3 +372,33 @@ def test_host_glue_is_clean_under_asan_and_ubsan():
         res = subprocess.run([exe], capture_output=True, text=True)
     assert res.returncode == 0, res.stderr[-2000:]
     assert re.match(r"\d+ blocks", res.stdout)
+
+
+def test_build_refuses_spilling_or_register_clashing_kernels():
+    """The two build-time checks on compiler output, fed with made-up compiler text: head_dim-256 backward kernels must
+    not use scratch memory, and the 256-row forward kernels must neither spill nor see the compiler use one of their
+    hand-assigned accumulation registers."""
+    from torch_mlu_amd import _build
+
+    def remarks(name, scratch):
+        return (f"x.hip:130:1: remark: Function Name: {name} [-Rpass-analysis=kernel-resource-usage]\n"
+                "  130 | __global__ void k() {\n      | ^\n"
+                "x.hip:130:1: remark:     VGPRs: 256 [-Rpass-analysis=kernel-resource-usage]\n"
+                f"x.hip:130:1: remark:     ScratchSize [bytes/lane]: {scratch} [-Rpass-analysis=kernel-resource-usage]\n")
+
+    dq256 = "_ZN12_GLOBAL__N_116fa_bwd_dq_kernelIDF16bLi256ELb0ELi0EEEvNS_5BArgsE"
+    dkv256 = "_ZN12_GLOBAL__N_117fa_bwd_dkv_kernelIDF16_Li256ELi1ELb0ELb0EEEvNS_5BArgsE"
+    dq128 = "_ZN12_GLOBAL__N_116fa_bwd_dq_kernelIDF16bLi128ELb0ELi2EEEvNS_5BArgsE"
+    _build.check_bwd256_scratch(remarks(dq256, 0) + remarks(dkv256, 0) + remarks(dq128, 28))   # 128: not this check's business
+    with pytest.raises(RuntimeError, match="spills 76 bytes"):
+        _build.check_bwd256_scratch(remarks(dq256, 0) + remarks(dkv256, 76))
+    with pytest.raises(RuntimeError, match="check not run"):
+        _build.check_bwd256_scratch(remarks(dq128, 0))
+
+    head = "_ZN2fa12_GLOBAL__N_117fa_tile256_kernelIDF16bLi128ELi2EEEvNS_5KArgsE:\n"
+    ok = head + "\tv_accvgpr_write_b32 a3, v1\n\t;;#ASMSTART\n\tv_mfma_f32_32x32x16_bf16 a[64:79], v[0:3], v[4:7], a[64:79]\n\t;;#ASMEND\n.Lfunc_end0:\n; ScratchSize: 0\n"
+    _build.check_tile256_registers(ok)
+    with pytest.raises(RuntimeError, match="hand-assigned"):
+        _build.check_tile256_registers(ok.replace("a3, v1", "a70, v1"))
+    with pytest.raises(RuntimeError, match="scratch"):
+        _build.check_tile256_registers(ok.replace("ScratchSize: 0", "ScratchSize: 16"))

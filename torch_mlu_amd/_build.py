@@ -67,6 +67,29 @@ def check_tile256_registers(asm_text: str) -> None:
             raise RuntimeError("fa_fwd_tile256: vector registers spill to scratch memory")
 
 
+def check_bwd256_scratch(remarks: str) -> None:
+    """The head_dim-256 backward kernels run one wavefront per SIMD with their MFMA-only operands pinned to the
+    accumulation registers; without the pins the compiler spilled up to 91 vector registers in them and they ran 1.5 x
+    slower.  `remarks` is what hipcc -Rpass-analysis=kernel-resource-usage printed for fa_bwd_kernels.hip; a build in
+    which one of those kernels uses scratch memory again is refused."""
+    import re
+
+    name = None
+    seen = 0
+    for line in remarks.splitlines():
+        m = re.search(r"remark: Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            continue
+        m = re.search(r"remark:\s+ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and name and re.search(r"fa_bwd_(dq|dkv)_kernelIDF16[b_]Li256E", name):
+            seen += 1
+            if int(m.group(1)) != 0:
+                raise RuntimeError(f"fa_bwd_kernels: {name} spills {m.group(1)} bytes per lane to scratch memory")
+    if seen == 0:
+        raise RuntimeError("fa_bwd_kernels: no resource remarks for the head_dim-256 kernels (check not run)")
+
+
 def build_kernels(verbose: bool = False) -> str:
     """hipcc: csrc/fa_fwd_kernels.hip + csrc/fa_fwd_tile256.hip + csrc/fa_bwd_kernels.hip -> lib/libfa_fwd.so (the C ABI of
     include/fa_fwd.h and include/fa_bwd.h)."""
@@ -76,7 +99,10 @@ def build_kernels(verbose: bool = False) -> str:
     srcs = [os.path.join(CSRC, f) for f in KERNEL_SOURCES]
     objs = [os.path.join(LIBDIR, os.path.splitext(f)[0] + ".o") for f in KERNEL_SOURCES]
     # one hipcc process per translation unit, side by side
-    procs = [(src, subprocess.Popen([HIPCC, *HIP_FLAGS, "-c", f"-I{INCLUDE}", f"-I{CSRC}", src, "-o", obj],
+    def extra(src):  # the backward file reports its kernels' registers and scratch (checked below)
+        return ["-Rpass-analysis=kernel-resource-usage"] if src.endswith("fa_bwd_kernels.hip") else []
+
+    procs = [(src, subprocess.Popen([HIPCC, *HIP_FLAGS, *extra(src), "-c", f"-I{INCLUDE}", f"-I{CSRC}", src, "-o", obj],
                                     stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
              for src, obj in zip(srcs, objs)]
     # the same device code as text, for the register check of the 256-row kernel
@@ -92,6 +118,17 @@ def build_kernels(verbose: bool = False) -> str:
         o = "\n".join(l for l in o.splitlines() if "is not a recognized feature for this target" not in l)
         if pr.returncode != 0:
             raise RuntimeError("build step failed: hipcc -c " + src + "\n" + o)
+        if extra(src):
+            check_bwd256_scratch(o)
+            kept, skip = [], 0  # a remark is three lines: the message, the source line, the caret
+            for l in o.splitlines():
+                if "-Rpass-analysis=kernel-resource-usage" in l:
+                    skip = 2
+                elif skip:
+                    skip -= 1
+                else:
+                    kept.append(l)
+            o = "\n".join(kept)
         log += o
     log += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp])
     os.replace(tmp, out)
