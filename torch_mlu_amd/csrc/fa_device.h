@@ -99,13 +99,24 @@ __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 LDS_AS*)p);
 }
 
+// the same through a pointer that is already an LDS address
+__device__ __forceinline__ s16x4 lds_read_tr_lds(LDS_AS const unsigned char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 LDS_AS*)p);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// max of two as one instruction (fmaxf first canonicalises both operands: three instructions)
+__device__ __forceinline__ float max2(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
 // max over the lane pair (l, l ^ 32)
 __device__ __forceinline__ float pair_max32(float x) {
   unsigned u = __builtin_bit_cast(unsigned, x);
   auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+  return max2(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
 }
 __device__ __forceinline__ float pair_sum32(float x) {
   unsigned u = __builtin_bit_cast(unsigned, x);

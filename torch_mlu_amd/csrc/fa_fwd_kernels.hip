@@ -250,6 +250,22 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
     vaddr[mb] = v_row * ROWB + (L & 1) * 8 + (((4 * mb + 2 * (G & 1) + ((L & 3) >> 1)) ^ swzV<DP>(v_row)) * 16);
+  // The same offsets as LDS pointers held in registers (the compiler otherwise re-adds the LDS base, a link-time
+  // constant it cannot fold, to every fragment address of every tile: 8 + 4 vector adds per tile); buffer and
+  // row-block displacements are immediates of the read instructions.  The bias variants have no registers to spare
+  // for that and keep the adds; so does head_dim 256 (measured: 2 % slower with the pointers).
+  LDS_AS const unsigned char* kptr[KS];
+  LDS_AS const unsigned char* vptr[MB];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    kptr[ks] = (LDS_AS const unsigned char*)smem + kaddr[ks];
+    if constexpr (BIAS == 0 && DP <= 128) asm volatile("" : "+v"(kptr[ks]));
+  }
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    vptr[mb] = (LDS_AS const unsigned char*)smem + 2 * TILE + vaddr[mb];
+    if constexpr (BIAS == 0 && DP <= 128) asm volatile("" : "+v"(vptr[mb]));
+  }
   // without a bias the scores stay raw and scale * log2(e) is folded into the exponent's FMA; with one they become
   // scale * s + bias when the bias is added, and the factor from there on is log2(e)
   const float c = BIAS ? kLog2e : a.scale_log2;
@@ -309,7 +325,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   for (int i = 0; i < MB; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = -INFINITY, l_run = 0.f, mc_run = 0.f;
 
   const int causal_row_lim = a.is_causal ? row + off : 0x7fffffff;
   const int wave_row_lo = m0 + 32 * wave, wave_row_hi = wave_row_lo + 31;
@@ -360,8 +376,6 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     // wavefront-uniform skip: every score of this tile is masked for all 32 rows of this wavefront
     if (a.is_causal && j * BN > wave_row_hi + off) return;
 
-    const unsigned char* kt = smem + BUF * TILE;
-    const unsigned char* vt = smem + 2 * TILE + BUF * TILE;
 
     // bias of a full tile: 8 loads of 4 keys each, issued now and consumed after the S MFMAs
     const bool full_tile = j * BN + BN <= Lk;
@@ -382,8 +396,8 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
       s16x8 ka[2][2];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
-        ka[ks][0] = *(const s16x8*)(kt + kaddr[ks]);
-        ka[ks][1] = *(const s16x8*)(kt + kaddr[ks] + 32 * ROWB);
+        ka[ks][0] = *(LDS_AS const s16x8*)(kptr[ks] + BUF * TILE);
+        ka[ks][1] = *(LDS_AS const s16x8*)(kptr[ks] + BUF * TILE + 32 * ROWB);
       }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
@@ -395,8 +409,8 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
           for (int x = (ks * 2 * NI) / KS; x < ((ks + 1) * 2 * NI) / KS; ++x) issue_one(j + 1, BUF ^ 1, x & 1, x >> 1);
         }
         if (ks + 2 < KS) {
-          ka[ks & 1][0] = *(const s16x8*)(kt + kaddr[ks + 2]);
-          ka[ks & 1][1] = *(const s16x8*)(kt + kaddr[ks + 2] + 32 * ROWB);
+          ka[ks & 1][0] = *(LDS_AS const s16x8*)(kptr[ks + 2] + BUF * TILE);
+          ka[ks & 1][1] = *(LDS_AS const s16x8*)(kptr[ks + 2] + BUF * TILE + 32 * ROWB);
         }
       }
     }
@@ -450,7 +464,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     mx = max3(mx, s0[15], s1[0]);
 #pragma unroll
     for (int v = 1; v < 15; v += 2) mx = max3(mx, s1[v], s1[v + 1]);
-    mx = fmaxf(mx, s1[15]);
+    mx = max2(mx, s1[15]);
     mx = pair_max32(mx);
     if constexpr (BIAS == 2) {
       // the next tile's bias may overwrite this one now: the maximum depends on every value that was read
@@ -462,13 +476,14 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
       const float m_new = grow ? mx : m_run;
       const float alpha = grow ? fast_exp2((m_run - m_new) * c) : 1.0f;  // exp2(-inf) = 0 on the first tile
       m_run = m_new;
+      mc_run = (m_run == -INFINITY) ? 0.f : m_run * c;
       l_run *= alpha;
 #pragma unroll
       for (int i = 0; i < MB; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
     }
-    const float mc = (m_run == -INFINITY) ? 0.f : m_run * c;
+    const float mc = mc_run;  // m_run c, kept alongside m_run (0 while no key has been seen)
     // dropout: counter of a patch = key ^ row term ^ column term; the column pair of this lane's groups is
     // 32 j + 2 g + a compile-time constant with disjoint bits
     const uint32_t drop_tile = DROP ? (drop_row ^ drop_col_term((uint32_t)(j * (BN / 2) + 2 * g))) : 0u;
@@ -476,8 +491,8 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     // ---- per 16-key chunk t: P = exp2(S c - m c), row sums, P^T as B operand, O^T += V^T P^T.  The V^T fragments
     //      of chunk t + 1 are fetched while chunk t's MFMAs run. ----
     auto vfrag = [&](int mb, int t) {
-      const s16x4 lo = lds_read_tr(vt + vaddr[mb] + (16 * t) * ROWB);
-      const s16x4 hi = lds_read_tr(vt + vaddr[mb] + (16 * t + 8) * ROWB);
+      const s16x4 lo = lds_read_tr_lds(vptr[mb] + BUF * TILE + (16 * t) * ROWB);
+      const s16x4 hi = lds_read_tr_lds(vptr[mb] + BUF * TILE + (16 * t + 8) * ROWB);
       return s16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
     s16x8 va[2][MB];
