@@ -145,6 +145,12 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
 }
+// the same, ordered behind the instruction that produced `after` (an input the instruction does not use)
+__device__ __forceinline__ float max3d(float a, float b, float c, float after) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c), "v"(after));
+  return r;
+}
 
 // ---- dropout ---------------------------------------------------------------------------------------------
 // One 32-bit word per 2 x 2 patch of the attention matrix of one (sequence, query head); element (row, col) keeps its

@@ -458,13 +458,29 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     }
 
     // ---- online softmax (one lane = one query row x 32 of the 64 columns) ----
-    float mx = max3(s0[0], s0[1], s0[2]);
+    // The maximum is exact whatever the order: two interleaved chains per product (half the latency of one chain, and
+    // fewer readers right behind their `asm` producer, each of which costs a compiler-inserted wait state).  The MFMA
+    // results must not be read before the matrix pipe has written them, and the compiler only inserts that wait in
+    // front of instructions it knows: the first read of each product's accumulators is therefore a canonicalize
+    // (a `v_max_f32 x, x` the compiler emits itself), and every `asm` maximum of that product depends on it.
+    const float g0 = __builtin_canonicalizef(s0[15]);
+    float c0 = max3d(s0[0], s0[1], s0[2], g0), c1 = max3d(s0[8], s0[9], s0[10], g0);
 #pragma unroll
-    for (int v = 3; v < 15; v += 2) mx = max3(mx, s0[v], s0[v + 1]);
-    mx = max3(mx, s0[15], s1[0]);
+    for (int v = 3; v < 7; v += 2) {
+      c0 = max3(c0, s0[v], s0[v + 1]);
+      c1 = max3(c1, s0[v + 8], s0[v + 9]);
+    }
+    c0 = max3(c0, s0[7], g0);
+    const float g1 = __builtin_canonicalizef(s1[15]);
+    float c2 = max3d(s1[0], s1[1], s1[2], g1), c3 = max3d(s1[8], s1[9], s1[10], g1);
 #pragma unroll
-    for (int v = 1; v < 15; v += 2) mx = max3(mx, s1[v], s1[v + 1]);
-    mx = max2(mx, s1[15]);
+    for (int v = 3; v < 7; v += 2) {
+      c2 = max3(c2, s1[v], s1[v + 1]);
+      c3 = max3(c3, s1[v + 8], s1[v + 9]);
+    }
+    c2 = max3(c2, s1[7], g1);
+    float mx = max3(c0, c1, c2);
+    mx = max2(mx, c3);
     mx = pair_max32(mx);
     if constexpr (BIAS == 2) {
       // the next tile's bias may overwrite this one now: the maximum depends on every value that was read
