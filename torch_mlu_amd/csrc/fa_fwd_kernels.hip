@@ -332,6 +332,9 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   // dropout: key ^ row term of this lane's row pair, and which half of a patch word belongs to this row
   const uint32_t drop_row = DROP ? (drop_key ^ drop_row_term((uint32_t)row >> 1)) : 0u;
   const int drop_sh = 16 * (row & 1);
+  // v_perm_b32 selector: bytes 2 (row & 1) and 2 (row & 1) + 1 of a word into the low bytes of the two halves
+  const uint32_t drop_sel = 0x0c000c00u | (uint32_t)(2 * (row & 1)) | ((uint32_t)(2 * (row & 1) + 1) << 16);
+  const uint32_t drop_thr2 = a.drop_thr | (a.drop_thr << 16);
   const unsigned char* brow = nullptr;  // this lane's bias row, at its first key group (4 g)
   unsigned char* drow = nullptr;  // this lane's row of the debug mask
   if constexpr (DROP && DMASK)
@@ -533,7 +536,20 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
         if constexpr (DROP) {
           // keys j BN + 32 (t >> 1) + 8 (v >> 2) + 4 g + (v & 3), + 1: one column pair, one patch word
           const uint32_t cp_const = 16 * (t >> 1) + 4 * (v >> 2) + ((v & 3) >> 1);
-          const uint32_t word = drop_word(drop_tile ^ cp_const, drop_key2) >> drop_sh;
+          const uint32_t word_full = drop_word(drop_tile ^ cp_const, drop_key2);
+          if constexpr (!DMASK) {
+            // The pair's two bytes go to the low bytes of the two 16-bit halves (one v_perm_b32), threshold minus
+            // byte is negative exactly where the element is dropped, and its sign, spread over the half by an
+            // arithmetic shift, clears that half of the packed pair: 4 instructions for what compare-and-select on
+            // the two floats does in 6.
+            typedef short i16x2 __attribute__((ext_vector_type(2)));
+            const uint32_t bytes = __builtin_amdgcn_perm(word_full, word_full, drop_sel);
+            const i16x2 diff = __builtin_bit_cast(i16x2, drop_thr2) - __builtin_bit_cast(i16x2, bytes);
+            const uint32_t gone = __builtin_bit_cast(uint32_t, diff >> 15);  // 0xffff per dropped half
+            w[e2] = Mma<T>::pack2(p0, p1) & ~gone;
+            continue;
+          }
+          const uint32_t word = word_full >> drop_sh;
           const bool k0 = (word & 0xffu) <= a.drop_thr, k1 = ((word >> 8) & 0xffu) <= a.drop_thr;
           if (DMASK && a.dmask) {
             const int col = j * BN + 32 * (t >> 1) + 8 * (v >> 2) + 4 * g + (v & 3);
