@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the flash-attention forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop|cfg2_mask_bwd|spec4|chunk256|cfg2_tile256|cfg2_tile256w|cfg5_paged] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop|cfg2_mask_bwd|spec4|chunk256|cfg5_paged] [--no-extras] [--no-cpu-baseline]
 
 A "step" is one call of the registered op on one batch of seeded synthetic input that is already resident in HBM.
 The headline workload is BASELINE.json configs[1] (causal prefill, bf16 MHA, B=4 H=32 S=4096 D=128); the other
@@ -38,8 +38,6 @@ TRAFFIC_BYTES = {
     "cfg2_mask": int(2.10 * 2 ** 30 + 130.0 * 2 ** 20),
     "cfg2_drop": int((515.5 + 130.0) * 2 ** 20),
     "cfg2_mask_bwd": int((3.84 + 2.24 + 1.97) * 2 ** 30 + (156.0 + 128.0 + 128.0) * 2 ** 20),  # three launches
-    "cfg2_tile256": int((686.7 + 130.0) * 2 ** 20),
-    "cfg2_tile256w": int((659.4 + 130.0) * 2 ** 20),
     "spec4": int(1.0011 * 2 ** 30 + (2.1 + 2.1 + 0.3) * 2 ** 20),  # split-KV + merge launches
     "chunk256": int((222.3 + 32.6 + 32.6 + 2.1) * 2 ** 20),        # sliced tile + merge launches
 }
@@ -78,25 +76,6 @@ def make_workload(name, dev):
                     desc=f"causal prefill bf16 B={B} Hq={Hq} Hkv={Hk} S={S} D={D}"
                          + (" on [B,S,H,D]-backed views" if name == "cfg2_bshd" else ""), dtype="bf16", bound="mfma",
                     kernel="fa_tile_kernel")
-    if name in ("cfg2_tile256", "cfg2_tile256w"):
-        # the headline workload through the C ABI with one of the 256-row kernels requested (they are not the default
-        # choice: see fa_fwd_tile_rows); 8 wavefronts x 32 rows, or 4 wavefronts x 64 rows
-        from torch_mlu_amd import capi
-        B, H, S, D = 4, 32, 4096, 128
-        q, k, v = (seeded((B, H, S, D), 1 + i, bf).to(dev) for i in range(3))
-        kern = capi.FA_KERNEL_TILE256 if name == "cfg2_tile256" else capi.FA_KERNEL_TILE256W
-
-        def call():
-            return capi.fa_forward_dense(q, k, v, is_causal=True, kernel=kern)
-
-        def check():
-            out, lse = call()
-            return _check_heads(q, k, v, out, lse, True, [(0, 0), (B - 1, H - 1)])
-
-        return dict(call=call, check=check, flops=4 * B * H * S * S * D / 2, bytes_kv=2 * B * H * S * D * 2,
-                    desc=f"causal prefill bf16 B={B} H={H} S={S} D={D}, 256-row kernel "
-                         + ("8 x 32 rows" if name == "cfg2_tile256" else "4 x 64 rows") + " through fa_fwd_launch",
-                    dtype="bf16", bound="mfma", kernel="fa_tile256_kernel")
     if name == "cfg2_bwd":
         # the backward of the headline workload (same shape and inputs, plus a seeded dOut); FLOPs are the five matrix
         # products of the algorithm (2.5 x the forward's), although the two-kernel design executes eight
@@ -304,7 +283,9 @@ def _check_heads(q, k, v, out, lse, causal, heads, bias=None, keep=None, dropout
         l = torch.logsumexp(s, -1)
         pm = torch.exp(s - l[:, None])
         if keep is not None:
-            pm = pm * keep[b, h] / (1.0 - dropout_p)
+            # the mask keeps with probability (floor((1 - p) 255) + 1) / 256 and the kernels scale by its reciprocal
+            thr = int(np.floor((np.float32(1.0) - np.float32(dropout_p)) * np.float32(255.0)))
+            pm = pm * keep[b, h] * (256.0 / (thr + 1))
         o = pm @ v[b, h // g].float()
         eo = max(eo, (out[b, h].float() - o).abs().max().item())
         el = max(el, (lse[b, h] - l).abs().max().item())
@@ -436,7 +417,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "spec4", "chunk256", "copy1g",
-                             "cfg2_tile256", "cfg2_tile256w", "cfg5_paged"])
+                             "cfg5_paged"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -459,7 +440,7 @@ def main():
         n0 = torch_mlu_amd.launch_count()
         eo, el = w["check"]()
         wall, ev_mean, ev_med, ev_min = time_steps(w["call"], steps, warmup)
-        assert name in ("copy1g", "cfg2_tile256", "cfg2_tile256w", "cfg5_paged") or torch_mlu_amd.launch_count() >= n0 + steps + warmup, \
+        assert name in ("copy1g", "cfg5_paged") or torch_mlu_amd.launch_count() >= n0 + steps + warmup, \
             "the registered HIP path did not run"
         r = {"config": name, "workload": w["desc"], "ms_per_step": wall, "kernel_ms_mean": ev_mean,
              "kernel_ms_median": ev_med, "kernel_ms_min": ev_min, "tflops": w["flops"] / wall / 1e9,
@@ -504,7 +485,7 @@ def main():
         "config": {"workload": main_r["workload"], "name": args.config,
                    "entry": {"cfg4": "aten::_flash_attention_forward", "spec4": "aten::_flash_attention_forward",
                              "chunk256": "aten::_flash_attention_forward",
-                             "cfg2_tile256": "fa_fwd_launch (C ABI)", "cfg2_tile256w": "fa_fwd_launch (C ABI)",
+                             
                              "cfg5_paged": "fa_fwd_launch (C ABI)",
                              "cfg2_bwd": "aten::_scaled_dot_product_flash_attention_backward",
                              "cfg2_mask": "aten::_scaled_dot_product_efficient_attention",

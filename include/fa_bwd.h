@@ -13,7 +13,8 @@
  *     dV  = P^T dO
  *     dP  = dO V^T,   delta = rowsum(dO o O),   dS = P o (dP - delta)
  *     dQ  = scale * dS K,   dK = scale * dS^T Q
- * (with dropout: dV = (P o M)^T dO / (1-p) and dP = M o (dO V^T) / (1-p), M regenerated from the forward's seed/offset)
+ * (with dropout: dV = (P o M)^T dO / keep and dP = M o (dO V^T) / keep, M regenerated from the forward's seed/offset,
+ * keep = the mask's keep probability as defined at fa_fwd_params.dropout_p)
  * with the forward's masking (the FA_MASK_* modes of fa_fwd.h) and head grouping (dK, dV of a kv head sum over the
  * query heads that read it).  Same rules as fa_fwd.h: plain C, device pointers, element strides, no allocation,
  * no synchronisation, work is only enqueued on the caller's stream.
@@ -90,7 +91,12 @@ typedef struct fa_bwd_params {
   /* optional additive bias of the forward (same dtype as q; NULL = none):
      element (b, h, row, col) at bias + b*bias_stride_b + h*bias_stride_h + row*bias_stride_q + col, h a query head;
      in packed mode b is the sequence and row, col count from the sequence's first row / key.
-     Strides may be 0 (broadcast) and must be multiples of 4; the pointer must be 8-byte aligned (as in the forward). */
+     Strides may be 0 (broadcast) and must be multiples of 4; the pointer must be 8-byte aligned (as in the forward).
+     Values: finite numbers and -inf (a masked position; a row that is -inf throughout gets zero gradients).  +inf and
+     NaN entries are outside the contract of this backward: the dK / dV kernels bring the bias into the score layout
+     through a matrix product with the identity, where an infinity or NaN spreads over its query row of the 32 x 32
+     block, so the gradients of that row are then undefined (other rows are unaffected).  The reference hands any
+     bias to the vendor call unchecked (FlashAttention_internal.cpp:836-903) and defines nothing for them either. */
   const void* bias;
   int64_t bias_stride_b, bias_stride_h, bias_stride_q;
   /* optional output (needs bias): the gradient of the bias, [batch, heads_q, seqlen_q, seqlen_k] in q's dtype,
@@ -100,14 +106,14 @@ typedef struct fa_bwd_params {
 } fa_bwd_params;
 
 /* Host-only validation: FA_OK or a negative code (FA_ERR_UNSUPPORTED for head_dim > 256). */
-int fa_bwd_validate(const fa_bwd_params* p);
+FA_API int fa_bwd_validate(const fa_bwd_params* p);
 
 /* Bytes of device scratch fa_bwd_launch needs (-rowsum(dO o O) and LSE log2(e), two fp32 per query row and head);
    0 if invalid. */
-size_t fa_bwd_workspace_bytes(const fa_bwd_params* p);
+FA_API size_t fa_bwd_workspace_bytes(const fa_bwd_params* p);
 
 /* Enqueue the backward pass on `stream`; `workspace` must hold fa_bwd_workspace_bytes(p) bytes, 16-byte aligned. */
-int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_bytes, void* stream);
+FA_API int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

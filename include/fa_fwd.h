@@ -24,7 +24,13 @@
 extern "C" {
 #endif
 
-#define FA_FWD_ABI_VERSION 8
+#define FA_FWD_ABI_VERSION 9
+
+/* The library is built with hidden visibility; the entry points declared here and in fa_bwd.h are its whole export
+   list. */
+#ifndef FA_API
+#define FA_API __attribute__((visibility("default")))
+#endif
 
 /* element types accepted for q/k/v/out (FlashAttention_internal.cpp:73-80 allows exactly these two) */
 #define FA_DTYPE_FP16 0
@@ -46,22 +52,17 @@ extern "C" {
 /* kernel selection */
 #define FA_KERNEL_AUTO 0     /* split-KV kernel when seqlen_q * (heads_q/heads_k) <= 16 (decode, a few speculative
                                 tokens; packed mode: seqlen_q is the longest sequence), else the tile kernel */
-#define FA_KERNEL_TILE 1     /* MFMA tile (prefill) kernels; the launcher picks the rows per workgroup (fa_fwd_tile_rows) */
+#define FA_KERNEL_TILE 1     /* MFMA tile (prefill) kernel: 128 query rows per workgroup, two workgroups per CU */
 #define FA_KERNEL_SPLITKV 2  /* HBM-bound split-KV kernel (+ merge): query rows x group heads share one pass over K/V */
-#define FA_KERNEL_TILE128 3  /* tile kernel with 128 query rows per workgroup, two workgroups per CU (every option) */
-#define FA_KERNEL_TILE256 4  /* tile kernel with 256 query rows per workgroup, one per CU, MFMA and softmax overlapped
-                                inside each wavefront (8 wavefronts of 32 rows, two per SIMD): head_dim <= 128, no
-                                bias, no dropout, num_splits <= 1, query / output row stride < 16 MiB
-                                (FA_ERR_UNSUPPORTED otherwise) */
-#define FA_KERNEL_TILE256W 5 /* the same with 4 wavefronts of 64 rows, one per SIMD */
 
 /*
  * One attention-forward problem:  for every sequence b and query head h
  *     S   = scale * Q[b,h] K[b,h/(heads_q/heads_k)]^T      (fp32 accumulate)
  *     S  += bias[b,h]                                      (optional additive bias, mem-efficient entry points)
  *     S   = -inf where is_causal and col > row + Lk_b - Lq_b (bottom-right aligned; FA_MASK_CAUSAL_TOP_LEFT: col > row)
- *     LSE = ln sum_j exp(S[:,j]),   out = softmax_row(S) V      (dropout_p > 0: out = (softmax_row(S) o M) V / (1 - p)
- *                                                          with a keep-mask M; LSE is that of the undropped S)
+ *     LSE = ln sum_j exp(S[:,j]),   out = softmax_row(S) V      (dropout_p > 0: out = (softmax_row(S) o M) V / keep
+ *                                                          with a keep-mask M of keep probability `keep`, see
+ *                                                          dropout_p; LSE is that of the undropped S)
  * which is what cnnlFlashAttentionForward_v2 is asked to compute (FlashAttention_internal.cpp:147-161,231-258; with
  * the bias descriptor of the mem-efficient launcher, :585-590,659-686).
  *
@@ -123,9 +124,10 @@ typedef struct fa_fwd_params {
      (philox_seed, philox_offset, sequence, query head, row, col), so the backward regenerates it from the two numbers
      and the tile and split-KV kernels drop the same elements. */
   float dropout_p;         /* 0 <= p < 1.  An element is kept iff one byte of a hash word is <= floor((1 - p) 255), i.e.
-                              with probability (floor((1 - p) 255) + 1) / 256, and kept elements are scaled by
-                              1 / (1 - p) exactly as the reference's oracle scales them: the expectation of the output
-                              is off by at most 1 / (256 (1 - p)) relative (p = 0.1: 0.18 %) */
+                              with probability keep = (floor((1 - p) 255) + 1) / 256 (1 - p rounded to a multiple of
+                              1 / 256), and kept elements are scaled by 1 / keep — the reference's oracle scales by
+                              1 / (1 - p) with a mask that keeps with probability 1 - p — so that the expectation of
+                              the output over masks is the undropped output; the backward uses the same factor */
   int32_t reserved2;       /* must be 0 */
   uint64_t philox_seed;
   uint64_t philox_offset;
@@ -166,22 +168,22 @@ typedef struct fa_fwd_params {
 #define FA_MAX_SPLITS 64
 
 /* ABI version of the loaded library (== FA_FWD_ABI_VERSION it was built with). */
-int fa_fwd_version(void);
+FA_API int fa_fwd_version(void);
 
 /* Static text for a return code. */
-const char* fa_fwd_error_string(int rc);
+FA_API const char* fa_fwd_error_string(int rc);
 
 /*
  * Validate `p` without touching the GPU.  Returns FA_OK or a negative code; the same checks run inside
  * fa_fwd_workspace_bytes / fa_fwd_launch.  Host-only, so callable on a machine with no device.
  */
-int fa_fwd_validate(const fa_fwd_params* p);
+FA_API int fa_fwd_validate(const fa_fwd_params* p);
 
 /*
  * Bytes of device scratch fa_fwd_launch needs for `p`: partial (m, l, o) per slice — per (sequence, query head, query row) for both
  * kernels (packed mode: seqlen_q rows per sequence); 0 when nothing is sliced.  Mirrors cnnlGetFlashAttentionForwardWorkspaceSize_v2.  Returns 0 also when `p` is invalid.
  */
-size_t fa_fwd_workspace_bytes(const fa_fwd_params* p);
+FA_API size_t fa_fwd_workspace_bytes(const fa_fwd_params* p);
 
 /*
  * Enqueue the forward pass on `stream` (a hipStream_t passed as void*; NULL = the null stream).
@@ -189,7 +191,7 @@ size_t fa_fwd_workspace_bytes(const fa_fwd_params* p);
  * alive until the enqueued work has run; stream-ordered allocators satisfy this.  Never allocates, never
  * synchronises, never throws.  Returns FA_OK or a negative code (nothing is enqueued on error).
  */
-int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_bytes, void* stream);
+FA_API int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * fa_fwd_launch for callers that cannot allocate device memory or pass a workspace (code under HIP graph capture,
@@ -204,20 +206,13 @@ int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_byte
  * between calls: every slot a launch reads it has written first.
  */
 #define FA_STATIC_WORKSPACE_BYTES (64u << 20)
-int fa_fwd_launch_static(const fa_fwd_params* p, void* stream);
+FA_API int fa_fwd_launch_static(const fa_fwd_params* p, void* stream);
 
 /*
  * Which kernel fa_fwd_launch would run for `p` (FA_KERNEL_TILE / FA_KERNEL_SPLITKV) and with how many splits;
  * negative code when `p` is invalid.  Host-only.
  */
-int fa_fwd_plan(const fa_fwd_params* p, int32_t* kernel, int32_t* num_splits);
-
-/*
- * Query rows per workgroup of the tile kernel fa_fwd_launch would run for `p`: 128 or 256; 0 when `p` goes to the
- * split-KV kernel; negative code when `p` is invalid or asks for FA_KERNEL_TILE256 with an option that kernel lacks.
- * Host-only.  (No counterpart in the reference: its kernel choice is inside the vendor library.)
- */
-int fa_fwd_tile_rows(const fa_fwd_params* p);
+FA_API int fa_fwd_plan(const fa_fwd_params* p, int32_t* kernel, int32_t* num_splits);
 
 #ifdef __cplusplus
 }

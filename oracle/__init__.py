@@ -10,6 +10,7 @@ from .attention_oracle import (  # noqa: F401
     cpu_sdpa_flash,
     default_atol,
     default_rtol,
+    dropout_effective_p,
     dropout_keep_mask,
     dropout_keys,
     dropout_patch_words,

@@ -286,6 +286,15 @@ def dropout_keep_mask(seed: int, offset: int, bh: int, seqlen_q: int, seqlen_k: 
     return byte <= u(thr)
 
 
+def dropout_effective_p(dropout_p: float) -> float:
+    """The drop probability this build's mask realises for a requested `dropout_p`: 1 - (floor((1 - p) 255) + 1) / 256,
+    the threshold formed in float32 as the launcher forms it.  The kernels scale kept probabilities by the reciprocal of
+    the realised keep probability, so the reference's formula (attention_ref: P o M / (1 - p),
+    test_scaled_dot_product_attention.py:152-158) describes their output when it is given this value as p."""
+    thr = int(np.floor((np.float32(1.0) - np.float32(dropout_p)) * np.float32(255.0)))
+    return 1.0 - (thr + 1) / 256.0
+
+
 def get_tolerances(true_value, computed_value, dtype_name: str, fudge_factor: Optional[float] = 2.0
                    ) -> Tuple[float, float]:
     """Restates test_scaled_dot_product_attention.py:166-204: the allowed error is `fudge_factor` times the error

@@ -319,8 +319,11 @@ def _reference_grid_case(dtype, B, Sq, Sk, D, l1, causal, p):
     keep = (dbg > 0) if p > 0 else None
     out.backward(do)
     assert torch_mlu_amd.launch_count() == n0 + 2
-    ref = _torch_attention_ref(q, k, v, do, scale, causal, keep, p, torch.float32)
-    lp = _torch_attention_ref(q, k, v, do, scale, causal, keep, p, dtype)
+    # (the returned mask keeps with probability 1 - pe, 1 - p rounded to a multiple of 1 / 256, and the kernels scale by
+    # 1 / (1 - pe): the reference's formula with the drop probability the mask realises)
+    pe = oracle.dropout_effective_p(p)
+    ref = _torch_attention_ref(q, k, v, do, scale, causal, keep, pe, torch.float32)
+    lp = _torch_attention_ref(q, k, v, do, scale, causal, keep, pe, dtype)
     for name, got, r, l, fudge in zip(("out", "dq", "dk", "dv"), (out, qd.grad, kd.grad, vd.grad), ref, lp,
                                       (2.0, 4.0, 2.0, 2.0)):
         # the rule's tolerances, computed on the device: atol = fudge * max(|ref - lp|, default), rtol likewise

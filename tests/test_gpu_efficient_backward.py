@@ -408,7 +408,7 @@ def test_bias_with_dropout_through_c_abi(dtype, D, mask):
         assert rng.tolist() == [seed, offset]
         keep = _keep(seed, offset, B, Hq, Sq, Sk, p)
         okw = dict(is_causal=mask != "none", causal_top_left=mask == "tl", attn_bias=fb[..., :Sk].double().numpy(),
-                   dropout_p=p, dropout_mask=keep)
+                   dropout_p=oracle.dropout_effective_p(p), dropout_mask=keep)
         ro, rl = oracle.sdpa_oracle(q, k, v, **okw)
         got_o = out.float().cpu().double().numpy()
         assert np.isfinite(got_o).all()
@@ -434,7 +434,7 @@ def test_efficient_ops_with_dropout_return_state_and_train():
     out, lse, seed, offset = aten._scaled_dot_product_efficient_attention(qd, kd, vd, be, True, p, False)
     assert seed.is_cuda and seed.dtype == torch.int64 and seed.dim() == 0 and seed.item() == 77
     keep = _keep(seed.item(), offset.item(), B, H, Sq, Sk, p)
-    okw = dict(attn_bias=bias.double().numpy(), dropout_p=p, dropout_mask=keep)
+    okw = dict(attn_bias=bias.double().numpy(), dropout_p=oracle.dropout_effective_p(p), dropout_mask=keep)
     ro, _ = oracle.sdpa_oracle(q, k, v, **okw)
     assert np.abs(out.float().cpu().double().numpy() - ro).max() <= 2 * EPS[HF] * max(1.0, float(np.abs(ro).max()))
     gq, gk, gv, gb = aten._scaled_dot_product_efficient_attention_backward(

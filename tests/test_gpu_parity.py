@@ -359,7 +359,7 @@ def test_packed_causal_pairs_equal_per_sequence_dense(B, Hq, Hk, D, maxlen, dtyp
             continue
         s, e, ks, ke = int(cq[b]), int(cq[b + 1]), int(ck[b]), int(ck[b + 1])
         o, l = capi.fa_forward_dense(q[s:e].transpose(0, 1)[None], k[ks:ke].transpose(0, 1)[None],
-                                     v[ks:ke].transpose(0, 1)[None], is_causal=True, kernel=capi.FA_KERNEL_TILE128)
+                                     v[ks:ke].transpose(0, 1)[None], is_causal=True, kernel=capi.FA_KERNEL_TILE)
         assert torch.equal(out[s:e], o[0].transpose(0, 1)) and torch.equal(lse[:, s:e], l[0]), b
     ro, rl = oracle.varlen_oracle(q[:int(cq[3])].cpu(), k[:int(ck[3])].cpu(), v[:int(ck[3])].cpu(), cq[:4], ck[:4],
                                   is_causal=True)

@@ -72,7 +72,7 @@ def test_dense_sweep(chunk):
             kw.update(dropout_p=p, philox_seed=seed, philox_offset=offset, rng_out=rng_t)
             keep = np.stack([np.stack([oracle.dropout_keep_mask(seed, offset, b * Hq + h, Sq, Sk, p) for h in range(Hq)])
                              for b in range(B)])
-            okw.update(dropout_p=p, dropout_mask=keep)
+            okw.update(dropout_p=oracle.dropout_effective_p(p), dropout_mask=keep)
         out, lse = capi.fa_forward_dense(qd, kd, vd, **kw)
         ro, rl = oracle.sdpa_oracle(q, k, v, **okw)
         got = out.float().cpu().numpy()

@@ -19,12 +19,13 @@ INCLUDE = os.path.join(ROOT, "include")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # Packed-fp32 VALU forms are switched off for all device code.
 HIP_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wno-inline-asm", "-Wno-unused-command-line-argument",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wno-inline-asm",
+    "-Wno-unused-command-line-argument",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
 
-KERNEL_SOURCES = ("fa_fwd_kernels.hip", "fa_fwd_tile256.hip", "fa_bwd_kernels.hip")
+KERNEL_SOURCES = ("fa_fwd_kernels.hip", "fa_bwd_kernels.hip")
 
 
 def _run(cmd, **kw):
@@ -33,38 +34,6 @@ def _run(cmd, **kw):
     if r.returncode != 0:
         raise RuntimeError("build step failed: " + " ".join(cmd) + "\n" + out)
     return out
-
-
-def check_tile256_registers(asm_text: str) -> None:
-    """fa_fwd_tile256.hip assigns accumulation registers by hand inside inline assembly: a64 .. a255 in the kernels with
-    two 32-row halves per wavefront (last template argument 2), a32 .. a127 in those with one.  The compiler may use
-    accumulation registers of its own (it takes them from a0 upwards); one inside the hand-assigned range outside the
-    assembly statements would silently corrupt the O accumulators or the Q fragments, and vector registers that
-    spill to scratch memory would ruin the kernel's speed, so such a build is refused."""
-    import re
-
-    in_asm = False
-    first_own = None  # first hand-assigned register of the kernel being read
-    for line in asm_text.splitlines():
-        t = line.strip()
-        m = re.match(r"^_ZN2fa.*fa_tile256_kernel\w*Li(\d+)EEEvNS_5KArgsE:", line)
-        if m:
-            first_own = 64 if m.group(1) == "2" else 32
-        elif line.startswith(".Lfunc_end"):
-            first_own = None
-        if t.startswith(";;#ASMSTART"):
-            in_asm = True
-        elif t.startswith(";;#ASMEND"):
-            in_asm = False
-        elif first_own is not None and not in_asm and t and not t.startswith((";", ".")):
-            code = t.split(";")[0]
-            for m in re.finditer(r"\ba(\d+)\b|\ba\[(\d+):(\d+)\]", code):
-                hi = int(m.group(1) if m.group(1) is not None else m.group(3))
-                if hi >= first_own:
-                    raise RuntimeError("fa_fwd_tile256: the compiler allocated a hand-assigned accumulation register: " + t)
-    for m in re.finditer(r"; ScratchSize: (\d+)", asm_text):
-        if int(m.group(1)) != 0:
-            raise RuntimeError("fa_fwd_tile256: vector registers spill to scratch memory")
 
 
 def check_bwd256_scratch(remarks: str) -> None:
@@ -91,7 +60,7 @@ def check_bwd256_scratch(remarks: str) -> None:
 
 
 def build_kernels(verbose: bool = False) -> str:
-    """hipcc: csrc/fa_fwd_kernels.hip + csrc/fa_fwd_tile256.hip + csrc/fa_bwd_kernels.hip -> lib/libfa_fwd.so (the C ABI of
+    """hipcc: csrc/fa_fwd_kernels.hip + csrc/fa_bwd_kernels.hip -> lib/libfa_fwd.so (the C ABI of
     include/fa_fwd.h and include/fa_bwd.h)."""
     os.makedirs(LIBDIR, exist_ok=True)
     out = os.path.join(LIBDIR, "libfa_fwd.so")
@@ -105,13 +74,6 @@ def build_kernels(verbose: bool = False) -> str:
     procs = [(src, subprocess.Popen([HIPCC, *HIP_FLAGS, *extra(src), "-c", f"-I{INCLUDE}", f"-I{CSRC}", src, "-o", obj],
                                     stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
              for src, obj in zip(srcs, objs)]
-    # the same device code as text, for the register check of the 256-row kernel
-    asm_path = os.path.join(LIBDIR, "fa_fwd_tile256.s")
-    t256 = os.path.join(CSRC, "fa_fwd_tile256.hip")
-    _run([HIPCC, *HIP_FLAGS, "--offload-device-only", "-S", f"-I{INCLUDE}", f"-I{CSRC}", t256, "-o", asm_path])
-    with open(asm_path) as f:
-        check_tile256_registers(f.read())
-    os.remove(asm_path)
     log = ""
     for src, pr in procs:
         o, _ = pr.communicate()
@@ -130,8 +92,14 @@ def build_kernels(verbose: bool = False) -> str:
                     kept.append(l)
             o = "\n".join(kept)
         log += o
-    log += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp])
+    # the export list is the C ABI and nothing else (hidden visibility covers the C++ internals, the version script
+    # the per-translation-unit marker symbols that hipcc emits)
+    vs = os.path.join(LIBDIR, "exports.map")
+    with open(vs, "w") as f:
+        f.write("{ global: fa_fwd_*; fa_bwd_*; local: *; };\n")
+    log += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", f"-Wl,--version-script={vs}", *objs, "-o", tmp])
     os.replace(tmp, out)
+    os.remove(vs)
     for obj in objs:
         os.remove(obj)
     if verbose and log.strip():

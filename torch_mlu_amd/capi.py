@@ -21,7 +21,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libfa_fwd.so")
 
-FA_FWD_ABI_VERSION = 8
+FA_FWD_ABI_VERSION = 9
 FA_DTYPE_FP16 = 0
 FA_DTYPE_BF16 = 1
 FA_OK = 0
@@ -34,9 +34,6 @@ FA_MASK_NONE, FA_MASK_CAUSAL_BOTTOM_RIGHT, FA_MASK_CAUSAL_TOP_LEFT = 0, 1, 2
 FA_KERNEL_AUTO = 0
 FA_KERNEL_TILE = 1
 FA_KERNEL_SPLITKV = 2
-FA_KERNEL_TILE128 = 3
-FA_KERNEL_TILE256 = 4
-FA_KERNEL_TILE256W = 5
 FA_MAX_SPLITS = 64
 
 # every symbol include/fa_fwd.h declares
@@ -48,7 +45,6 @@ EXPORTED_SYMBOLS = (
     "fa_fwd_launch",
     "fa_fwd_launch_static",
     "fa_fwd_plan",
-    "fa_fwd_tile_rows",
     "fa_bwd_validate",
     "fa_bwd_workspace_bytes",
     "fa_bwd_launch",

@@ -86,7 +86,7 @@ struct BArgs {
   float scale;       // signed softmax scale
   float scale_log2;  // scale * log2(e), signed
   uint32_t drop_thr;  // dropout: an element was kept iff its byte <= drop_thr
-  float drop_rp;      // 1 / (1 - p)
+  float drop_rp;      // 256 / (drop_thr + 1): one over the realised keep probability
   const int64_t* seed_ptr;    // the forward's philox_seed / philox_offset slots (device)
   const int64_t* offset_ptr;
   int32_t causal_tl;          // causal mask aligned to the top-left corner (col <= row) instead of the bottom-right one
@@ -996,7 +996,7 @@ __global__ void __launch_bounds__(256, DP > 128 ? 1 : 2) fa_bwd_dkv_kernel(const
           const float d1 = (DO_K && !DELTA_INIT) ? dl[v >> 2][(v & 3) + 1] : 0.f;
           float p0 = fast_exp2(s[v] * c - l0), p1 = fast_exp2(s[v + 1] * c - l1);
           float dp0 = DO_K ? dp[v] : 0.f, dp1 = DO_K ? dp[v + 1] : 0.f;
-          float pv0 = p0, pv1 = p1;  // what multiplies dO in dV: P o M / (1 - p)
+          float pv0 = p0, pv1 = p1;  // what multiplies dO in dV: P o M / keep
           if constexpr (DROP) {
             const uint32_t rp_const = 16 * qbk + 4 * (v >> 2) + ((v & 3) >> 1);
             const uint32_t word = drop_word(drop_tile ^ (rp_const << 16), drop_key2) >> drop_sh;
@@ -1213,7 +1213,7 @@ int fa_bwd_launch(const fa_bwd_params* p, void* workspace, size_t workspace_byte
   if (a.scale_log2 == 0.f) a.scale_log2 = 1e-30f;  // scale 0: uniform probabilities, and -inf * c stays -inf
   const float p_keep = 1.f - p->dropout_p;
   a.drop_thr = (uint32_t)floorf(p_keep * 255.f);
-  a.drop_rp = 1.f / p_keep;
+  a.drop_rp = 256.f / (float)(a.drop_thr + 1u);  // the reciprocal of the keep probability the mask realises
   a.seed_ptr = p->philox_seed;
   a.offset_ptr = p->philox_offset;
   hipStream_t st = (hipStream_t)stream;

@@ -41,7 +41,7 @@ struct KArgs {
   const unsigned char* bias;  // optional additive bias, dense mode: [b][h][row][col] through byte strides
   int64_t bias_sb, bias_sh, bias_sq;
   uint32_t drop_thr;  // dropout: an element is kept iff its byte <= drop_thr
-  float drop_rp;      // 1 / (1 - p)
+  float drop_rp;      // 256 / (drop_thr + 1): one over the realised keep probability
   uint64_t seed, offset;
   const int64_t* seed_ptr;    // optional: the seed is *seed_ptr and *offset_ptr is added to offset (graph capture)
   const int64_t* offset_ptr;
@@ -75,12 +75,6 @@ __device__ __forceinline__ int swzV(int row) {
 // depend on which maximum was in use.
 constexpr float kLazyLog2 = 8.0f;
 
-
-// The 256-row tile kernels (fa_fwd_tile256.hip): one workgroup owns 256 query rows; `halves` = 32-row halves per
-// wavefront: 1 (8 wavefronts, two per SIMD) or 2 (4 wavefronts, one per SIMD).
-// Eligible problems: head_dim padded to 64 or 128, no bias, no dropout, not sliced.  Returns an FA_* code.
-bool tile256_eligible(const KArgs& a);
-int launch_tile256(const KArgs& a, int dtype, int halves, hipStream_t st);
 
 }  // namespace fa
 

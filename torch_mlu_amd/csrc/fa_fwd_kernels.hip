@@ -47,7 +47,7 @@ using namespace fa;
 // aligned and seqlen_k a multiple of 8) and read from there: the loads of mode 1 are issued only 16 MFMAs before
 // their use, which leaves most of an L2 miss exposed.
 // DROP: dropout on the probabilities.  The row sums (and LSE) are those of the undropped probabilities; dropped
-// entries are zeroed in the P operand of the PV product and 1 / (1 - p) is folded into the final normalisation.
+// entries are zeroed in the P operand of the PV product and 1 / (keep probability) is folded into the final normalisation.
 // DMASK (with DROP): also write the keep-mask out for tests; a variant of its own because the extra stores cost
 // registers (30 spilled at head_dim 128) that the plain dropout kernel does not have to pay.
 template <typename T, int DP, int MINB, int BIAS, bool DROP = false, bool DMASK = false>
@@ -338,7 +338,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   const unsigned char* brow = nullptr;  // this lane's bias row, at its first key group (4 g)
   unsigned char* drow = nullptr;  // this lane's row of the debug mask
   if constexpr (DROP && DMASK)
-    if (a.dmask) drow = a.dmask + (((int64_t)b * a.heads_q + h) * a.seqlen_q + min(row, Lq - 1)) * (int64_t)a.seqlen_k * 2;
+    if (a.dmask) drow = a.dmask + (((int64_t)b * a.heads_q + h) * a.seqlen_q + min(row, min(Lq, a.seqlen_q) - 1)) * (int64_t)a.seqlen_k * 2;
   if constexpr (BIAS == 1)
     brow = a.bias + (int64_t)b * a.bias_sb + (int64_t)h * a.bias_sh + (int64_t)min(row, Lq - 1) * a.bias_sq + 8 * g;
   // BIAS == 2: this wavefront's 32 rows x 64 keys of the bias tile (4 KiB) go through a private LDS area by DMA, one
@@ -553,9 +553,13 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
           const bool k0 = (word & 0xffu) <= a.drop_thr, k1 = ((word >> 8) & 0xffu) <= a.drop_thr;
           if (DMASK && a.dmask) {
             const int col = j * BN + 32 * (t >> 1) + 8 * (v >> 2) + 4 * g + (v & 3);
-            if (row < Lq && col + 1 <= min(last_k, causal_row_lim)) {
+            // (packed: a sequence longer than the seqlen_q x seqlen_k the caller stated gets its first rows and keys
+            // only; nothing is stored outside the [seqlen_q, seqlen_k] plane of this (sequence, head))
+            const bool row_in = row < Lq && row < a.seqlen_q;
+            const int col_lim = min(min(last_k, causal_row_lim), a.seqlen_k - 1);
+            if (row_in && col + 1 <= col_lim) {
               *(unsigned*)(drow + (int64_t)col * 2) = Mma<T>::pack2(k0 ? 1.f : -1.f, k1 ? 1.f : -1.f);
-            } else if (row < Lq && col <= min(last_k, causal_row_lim)) {
+            } else if (row_in && col <= col_lim) {
               *(T*)(drow + (int64_t)col * 2) = (T)(k0 ? 1.f : -1.f);
             }
           }
@@ -1026,7 +1030,7 @@ __global__ void __launch_bounds__(256) fa_merge_rows_kernel(const KArgs a) {
       if (d < D) acc[i] += po[(int64_t)s * D + d] * sc;
     }
   }
-  const float inv = (lsum > 0.f) ? a.drop_rp / lsum : 0.f;  // 1 / (1 - p): the split-KV kernel's partials under dropout
+  const float inv = (lsum > 0.f) ? a.drop_rp / lsum : 0.f;  // 1 / keep: the split-KV kernel's partials under dropout
   T* orow = (T*)(a.out + orow_off + (int64_t)h * a.o_sh);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -1075,7 +1079,7 @@ KArgs make_args(const fa_fwd_params* p, int kern, int ns, void* ws) {
   a.scale_abs = a.scale_log2 * kLn2;
   const float p_keep = 1.f - p->dropout_p;
   a.drop_thr = (uint32_t)floorf(p_keep * 255.f);
-  a.drop_rp = 1.f / p_keep;
+  a.drop_rp = 256.f / (float)(a.drop_thr + 1u);  // the reciprocal of the keep probability the mask realises
   a.seed = p->philox_seed; a.offset = p->philox_offset;
   a.seed_ptr = p->philox_seed_ptr; a.offset_ptr = p->philox_offset_ptr;
   a.rng_seed_out = p->rng_seed_out; a.rng_offset_out = p->rng_offset_out;
@@ -1218,16 +1222,6 @@ int fa_fwd_plan(const fa_fwd_params* p, int32_t* kernel, int32_t* num_splits) {
   return FA_OK;
 }
 
-int fa_fwd_tile_rows(const fa_fwd_params* p) {
-  const int rc = validate(p);
-  if (rc != FA_OK) return rc;
-  int k, s;
-  plan(p, &k, &s);
-  if (k != FA_KERNEL_TILE) return 0;
-  const int rows = tile_rows(p, s);
-  return rows ? rows : FA_ERR_UNSUPPORTED;
-}
-
 size_t fa_fwd_workspace_bytes(const fa_fwd_params* p) {
   if (validate(p) != FA_OK) return 0;
   int k, s;
@@ -1288,14 +1282,6 @@ int fa_fwd_launch(const fa_fwd_params* p, void* workspace, size_t workspace_byte
   if (p->seqlen_q == 0) return FA_OK;  // nothing to write
   const KArgs a = make_args(p, kern, ns, workspace);
   hipStream_t st = (hipStream_t)stream;
-  if (kern == FA_KERNEL_TILE) {
-    const int rows = tile_rows(p, ns);
-    if (rows == 0) return FA_ERR_UNSUPPORTED;
-    if (rows == 256) {
-      if (!tile256_eligible(a)) return FA_ERR_UNSUPPORTED;
-      return launch_tile256(a, p->dtype, p->kernel == FA_KERNEL_TILE256W ? 2 : 1, st);
-    }
-  }
   return p->dtype == FA_DTYPE_BF16 ? dispatch<__bf16>(a, kern, st) : dispatch<_Float16>(a, kern, st);
 }
 

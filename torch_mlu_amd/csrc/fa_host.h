@@ -35,7 +35,7 @@ inline int validate(const fa_fwd_params* p) {
   // sizes) and the 64-bit products below from overflowing
   if (p->seqlen_q > kMaxSeqlen || p->seqlen_k > kMaxSeqlen) return FA_ERR_UNSUPPORTED;
   if ((int64_t)p->batch * p->heads_q > 0x7fffffffLL) return FA_ERR_UNSUPPORTED;
-  if (p->kernel < FA_KERNEL_AUTO || p->kernel > FA_KERNEL_TILE256W) return FA_ERR_BAD_ARG;
+  if (p->kernel < FA_KERNEL_AUTO || p->kernel > FA_KERNEL_SPLITKV) return FA_ERR_BAD_ARG;
   if (p->num_splits < 0 || p->num_splits > FA_MAX_SPLITS) return FA_ERR_BAD_ARG;
   // 16-byte vector access on every row: base pointers and row strides must be multiples of 8 elements
   const uintptr_t al = (uintptr_t)p->q | (uintptr_t)p->k | (uintptr_t)p->v | (uintptr_t)p->out;
@@ -95,7 +95,6 @@ inline int validate(const fa_fwd_params* p) {
 inline void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   int kern = p->kernel;
   const int group = p->heads_q / p->heads_k;
-  if (kern == FA_KERNEL_TILE128 || kern == FA_KERNEL_TILE256 || kern == FA_KERNEL_TILE256W) kern = FA_KERNEL_TILE;  // the family; tile_rows() picks
   if (p->block_table) kern = FA_KERNEL_SPLITKV;  // the only kernel that reads a page table (validate() checked the shape)
   if (kern == FA_KERNEL_AUTO)
     kern = (p->seqlen_q >= 1 && (int64_t)p->seqlen_q * group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT && !(p->dropout_p > 0.f && p->dropout_mask))
@@ -131,7 +130,6 @@ inline void plan(const fa_fwd_params* p, int* kernel, int* splits) {
     if (ns == 0) {
       ns = 1;
       while (ns * 2 <= FA_MAX_SPLITS && wgs * ns * 2 <= 512 && ntiles / (ns * 2) >= min_tiles) ns *= 2;
-      if (p->kernel == FA_KERNEL_TILE256 || p->kernel == FA_KERNEL_TILE256W) ns = 1;  // the 256-row kernels are never sliced
     }
     if (ns > ntiles) ns = ntiles > 0 ? ntiles : 1;
     // keep the partials (fp32, one slot per query row and slice) within 1 GiB
@@ -153,21 +151,6 @@ inline size_t workspace_bytes(const fa_fwd_params* p, int kern, int ns) {
   if (ns <= 1) return 0;
   const size_t slots = partial_slots(p, kern, ns);
   return slots * (size_t)p->head_dim * 4 + slots * 8;
-}
-
-// Rows per workgroup of the tile kernel that runs `p` (plan() chose the tile family with ns slices): the 256-row
-// kernel takes what it can (head_dim <= 128, no bias, no dropout, not sliced) once there are enough query blocks to
-// give every CU two of its workgroups, one after the other; smaller problems spread better in 128-row workgroups, two
-// per CU.
-inline int tile_rows(const fa_fwd_params* p, int ns) {
-  // (the 256-row kernels address a query block's rows with 32-bit offsets from its first row)
-  const int64_t lim256 = 0xffffffffLL / 256 / 2;  // elements
-  const bool can256 = p->head_dim <= 128 && !p->bias && !(p->dropout_p > 0.f) && ns == 1 &&
-                      p->q_stride_s <= lim256 && p->o_stride_s <= lim256;
-  if (p->kernel == FA_KERNEL_TILE128) return 128;
-  if (p->kernel == FA_KERNEL_TILE256 || p->kernel == FA_KERNEL_TILE256W) return can256 ? 256 : 0;
-  if (!can256) return 128;
-  return 128;  // the 256-row kernel only on request while it is being tuned
 }
 
 // ---- backward -----------------------------------------------------------------------------------------------
