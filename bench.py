@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the flash-attention forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop|cfg2_mask_bwd|spec4|chunk256|cfg5_paged] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2|cfg3|cfg4|cfg5|cfg2_bwd|cfg2_mask|cfg2_drop|cfg2_mask_bwd|spec4|chunk256|chunk256_paged|cfg5_paged] [--no-extras] [--no-cpu-baseline]
 
 A "step" is one call of the registered op on one batch of seeded synthetic input that is already resident in HBM.
 The headline workload is BASELINE.json configs[1] (causal prefill, bf16 MHA, B=4 H=32 S=4096 D=128); the other
@@ -221,6 +221,32 @@ def make_workload(name, dev):
         return dict(call=call, check=check, flops=4 * B * Hq * Sk * D, bytes_kv=2 * B * Hk * Sk * D * 2,
                     desc=f"decode bf16 GQA B={B} Hq={Hq} Hkv={Hk} Sq=1 Skv={Sk} D={D}, K/V in scattered {page}-row pages "
                          "through a block table (fa_fwd_launch)", dtype="bf16", bound="hbm", kernel="fa_splitkv_kernel")
+    if name == "chunk256_paged":
+        # chunk256's prefill chunk against the same cache held in scattered 256-row pages (the tile kernel's paged
+        # variant through the C ABI, sliced over the key range like chunk256)
+        from torch_mlu_amd import capi
+        B, Hq, Hk, Sq, Sk, D, page = 1, 32, 8, 256, 32768, 128, 256
+        q = seeded((B, Hq, Sq, D), 40, bf).to(dev)
+        per_seq = Sk // page
+        kk = seeded((B * per_seq, page, Hk, D), 41, bf).to(dev)
+        vv = seeded((B * per_seq, page, Hk, D), 42, bf).to(dev)
+        tt = torch.randperm(B * per_seq, generator=torch.Generator().manual_seed(7)).reshape(B, per_seq).to(torch.int32).to(dev)
+        used = torch.full((B,), Sk, dtype=torch.int32, device=dev)
+
+        def call():
+            return capi.fa_forward_paged(q, kk, vv, tt, used, is_causal=True)
+
+        def check():
+            out, lse = call()
+            kf = kk[tt.long()].reshape(B, Sk, Hk, D).transpose(1, 2)
+            vf = vv[tt.long()].reshape(B, Sk, Hk, D).transpose(1, 2)
+            return _check_heads(q, kf, vf, out, lse, True, [(0, 0), (B - 1, Hq - 1)])
+
+        visible = Sq * (Sk - Sq + 1) + Sq * (Sq - 1) // 2
+        return dict(call=call, check=check, flops=4 * B * Hq * visible * D, bytes_kv=2 * B * Hk * Sk * D * 2,
+                    desc=f"{Sq}-token prefill chunk against a {Sk}-key cache in scattered {page}-row pages, causal, bf16 "
+                         f"GQA B={B} Hq={Hq} Hkv={Hk} D={D} (fa_fwd_launch)", dtype="bf16", bound="mfma",
+                    kernel="fa_tile_kernel")
     if name in ("spec4", "chunk256"):
         # serving shapes beside the BASELINE configs (extras only): 4 speculative tokens per sequence against a 32k
         # KV cache (rides the split-KV kernel, HBM-bound) and a 256-token prefill chunk of one sequence against a
@@ -416,7 +442,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "spec4", "chunk256", "copy1g",
+    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "spec4", "chunk256", "chunk256_paged", "copy1g",
                              "cfg5_paged"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -440,7 +466,7 @@ def main():
         n0 = torch_mlu_amd.launch_count()
         eo, el = w["check"]()
         wall, ev_mean, ev_med, ev_min = time_steps(w["call"], steps, warmup)
-        assert name in ("copy1g", "cfg5_paged") or torch_mlu_amd.launch_count() >= n0 + steps + warmup, \
+        assert name in ("copy1g", "cfg5_paged", "chunk256_paged") or torch_mlu_amd.launch_count() >= n0 + steps + warmup, \
             "the registered HIP path did not run"
         r = {"config": name, "workload": w["desc"], "ms_per_step": wall, "kernel_ms_mean": ev_mean,
              "kernel_ms_median": ev_med, "kernel_ms_min": ev_min, "tflops": w["flops"] / wall / 1e9,
@@ -464,7 +490,7 @@ def main():
     extras = []
     if not args.no_extras:
         for name in ("cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd",
-                     "spec4", "chunk256", "cfg5_paged"):
+                     "spec4", "chunk256", "chunk256_paged", "cfg5_paged"):
             if name != args.config:
                 extras.append(run(name, args.steps, args.warmup))
 
@@ -486,7 +512,7 @@ def main():
                    "entry": {"cfg4": "aten::_flash_attention_forward", "spec4": "aten::_flash_attention_forward",
                              "chunk256": "aten::_flash_attention_forward",
                              
-                             "cfg5_paged": "fa_fwd_launch (C ABI)",
+                             "cfg5_paged": "fa_fwd_launch (C ABI)", "chunk256_paged": "fa_fwd_launch (C ABI)",
                              "cfg2_bwd": "aten::_scaled_dot_product_flash_attention_backward",
                              "cfg2_mask": "aten::_scaled_dot_product_efficient_attention",
                              "cfg2_mask_bwd": "aten::_scaled_dot_product_efficient_attention_backward"}.get(

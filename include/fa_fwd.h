@@ -151,8 +151,10 @@ typedef struct fa_fwd_params {
      rng_seed_out / rng_offset_out receive the resolved numbers. */
   const int64_t* philox_seed_ptr;
   const int64_t* philox_offset_ptr;
-  /* optional paged KV cache (NULL = k / v are per-sequence tensors as above).  Dense mode, split-KV kernel only
-     (seqlen_q x heads_q / heads_k <= 16, no bias, no dropout_mask, not top-left causal; anything else: FA_ERR_UNSUPPORTED).
+  /* optional paged KV cache (NULL = k / v are per-sequence tensors as above).  Dense mode, no bias, no dropout_mask,
+     not top-left causal (anything else: FA_ERR_UNSUPPORTED).  Decode-shaped calls (seqlen_q x heads_q / heads_k <= 16)
+     run on the split-KV kernel; longer query chunks (a chunk of a chunked prefill against the cache) on the tile
+     kernel, which takes no dropout with a page table.
      k and v then point at pools of pages, [page][row in page][kv head][head_dim]: k_stride_b / v_stride_b are the
      element strides between pages, k_stride_s / v_stride_s between the rows of a page.  Key row r of sequence b lives
      in page block_table[b * block_table_stride + r / page_size] at row r % page_size.  seqlen_k is the longest

@@ -1,6 +1,7 @@
-"""Paged KV cache (fa_fwd_params.block_table) on the split-KV kernel.  The kernel reads the same keys in the same order
-whether a sequence's cache is one tensor or scattered over pages, so the results must equal, bit for bit, the same call
-on the gathered contiguous cache; and that call is checked against the oracle elsewhere (and once more here)."""
+"""Paged KV cache (fa_fwd_params.block_table): decode-shaped calls on the split-KV kernel, prefill chunks on the tile
+kernel.  Either kernel reads the same keys in the same order whether a sequence's cache is one tensor or scattered over
+pages, so the results must equal, bit for bit, the same call on the gathered contiguous cache; and that call is checked
+against the oracle elsewhere (and once more here)."""
 import ctypes
 
 import numpy as np
@@ -101,10 +102,65 @@ def test_paged_refusals():
     assert L.fa_fwd_validate(ctypes.byref(params(page_size=48))) == capi.FA_ERR_UNSUPPORTED      # not whole 32-row blocks
     assert L.fa_fwd_validate(ctypes.byref(params(page_size=0))) == capi.FA_ERR_BAD_ARG
     assert L.fa_fwd_validate(ctypes.byref(params(block_table_stride=1))) == capi.FA_ERR_BAD_ARG   # table too narrow
-    assert L.fa_fwd_validate(ctypes.byref(params(kernel=capi.FA_KERNEL_TILE))) == capi.FA_ERR_UNSUPPORTED
-    assert L.fa_fwd_validate(ctypes.byref(params(seqlen_q=64))) == capi.FA_ERR_UNSUPPORTED        # a prefill chunk
+    assert L.fa_fwd_validate(ctypes.byref(params(kernel=capi.FA_KERNEL_TILE))) == capi.FA_OK      # the tile kernel pages too
+    assert L.fa_fwd_validate(ctypes.byref(params(seqlen_q=64))) == capi.FA_ERR_UNSUPPORTED        # split-KV asked for a chunk
+    assert L.fa_fwd_validate(ctypes.byref(params(seqlen_q=64, kernel=capi.FA_KERNEL_AUTO))) == capi.FA_OK
+    assert L.fa_fwd_validate(ctypes.byref(params(seqlen_q=64, kernel=capi.FA_KERNEL_AUTO, dropout_p=0.1))) == capi.FA_ERR_UNSUPPORTED
+    assert L.fa_fwd_validate(ctypes.byref(params(kernel=capi.FA_KERNEL_TILE, dropout_p=0.1))) == capi.FA_ERR_UNSUPPORTED
+    assert L.fa_fwd_validate(ctypes.byref(params(dropout_p=0.1))) == capi.FA_OK                   # decode-shaped: split-KV
     assert L.fa_fwd_validate(ctypes.byref(params(reserved3=1))) == capi.FA_ERR_BAD_ARG
     kern, ns = ctypes.c_int32(), ctypes.c_int32()
     p = params(kernel=capi.FA_KERNEL_AUTO, seqlen_k=64)   # short caches stay on the split-KV kernel too
     p.block_table_stride = 1
     assert L.fa_fwd_plan(ctypes.byref(p), ctypes.byref(kern), ctypes.byref(ns)) == 0 and kern.value == capi.FA_KERNEL_SPLITKV
+
+
+@pytest.mark.parametrize("dtype,D,page", [(BF, 128, 256), (HF, 64, 32), (BF, 256, 64), (HF, 96, 96), (BF, 128, 32), (HF, 128, 160)])
+@pytest.mark.parametrize("Sq,group,causal", [(64, 4, True), (200, 1, True), (300, 2, False), (17, 4, True), (129, 8, True)])
+def test_paged_prefill_chunk_equals_contiguous_bit_for_bit(dtype, D, page, Sq, group, causal):
+    """A chunk of a chunked prefill against a paged cache runs on the tile kernel (bottom-right causal: the chunk's rows
+    are the cache's last Sq): the same tiles as on the gathered contiguous cache, unsliced and sliced."""
+    B, Hk = 3, 2
+    Hq = Hk * group
+    lens = [9 * page + 17 + Sq, Sq + 1, 3 * page + 1 + Sq]
+    q, kp, vp, table, used, kf, vf = _paged_case(B, Hq, Hk, Sq, D, page, lens, dtype, 900 + D + page + Sq)
+    qd, kpd, vpd, td, ud, kfd, vfd = (t.to(DEV) for t in (q, kp, vp, table, used, kf, vf))
+    kern, nsp = ctypes.c_int32(), ctypes.c_int32()
+    for ns in (0, 1, 3):
+        out_p, lse_p = capi.fa_forward_paged(qd, kpd, vpd, td, ud, is_causal=causal, num_splits=ns,
+                                             kernel=capi.FA_KERNEL_TILE)
+        out_c, lse_c = capi.fa_forward_dense(qd, kfd, vfd, is_causal=causal, kernel=capi.FA_KERNEL_TILE,
+                                             num_splits=ns, seqused_k=ud)
+        assert torch.equal(out_p, out_c) and torch.equal(lse_p, lse_c), ns
+    if Sq * group > 16:   # the automatic plan sends what the split-KV kernel cannot take to the tile kernel
+        out_a, lse_a = capi.fa_forward_paged(qd, kpd, vpd, td, ud, is_causal=causal)
+        assert torch.equal(out_a, out_p) or (out_a.float() - out_p.float()).abs().max() < 4e-3   # (its own slice plan)
+    for b in (0, 1):
+        ro, rl = oracle.sdpa_oracle(q[b:b + 1], kf[b:b + 1, :, :lens[b]], vf[b:b + 1, :, :lens[b]], is_causal=causal)
+        out_close(out_p[b:b + 1].float().cpu().numpy(), ro, dtype)
+        lse_close(lse_p[b:b + 1].cpu().numpy(), rl)
+
+
+def test_paged_prefill_chunk_long_cache():
+    """A 512-token chunk of 8 sequences against caches of up to 16k keys in 64-row pages, heads packed with padding."""
+    B, Hq, Hk, D, page, Sq = 8, 16, 4, 128, 64, 512
+    g = torch.Generator().manual_seed(11)
+    lens = (torch.randint(Sq, 16385, (B,), generator=g)).tolist()
+    max_pages = 16384 // page
+    n_pages = B * max_pages
+    pool = torch.randn(n_pages, page, Hk, D + 8, generator=g).mul_(0.5).to(BF).to(DEV)
+    kpd = pool[..., :D]
+    vpd = torch.randn(n_pages, page, Hk, D, generator=g).mul_(0.5).to(BF).to(DEV)
+    table = torch.randperm(n_pages, generator=g).reshape(B, max_pages).to(torch.int32)
+    td = table.to(DEV)
+    ud = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    qd = (torch.randn(B, Hq, Sq, D, generator=g) * 0.5).to(BF).to(DEV)
+    out_p, lse_p = capi.fa_forward_paged(qd, kpd, vpd, td, ud, is_causal=True)
+    kf = kpd[table.long().to(DEV)].reshape(B, max_pages * page, Hk, D).transpose(1, 2).contiguous()
+    vf = vpd[table.long().to(DEV)].reshape(B, max_pages * page, Hk, D).transpose(1, 2).contiguous()
+    out_c, lse_c = capi.fa_forward_dense(qd, kf, vf, is_causal=True, kernel=capi.FA_KERNEL_TILE, seqused_k=ud)
+    assert torch.equal(out_p, out_c) and torch.equal(lse_p, lse_c)
+    b = int(np.argmin(lens))
+    ro, rl = oracle.sdpa_oracle(qd[b:b + 1].cpu(), kf[b:b + 1, :, :lens[b]].cpu(), vf[b:b + 1, :, :lens[b]].cpu(), is_causal=True)
+    out_close(out_p[b:b + 1].float().cpu().numpy(), ro, BF)
+    lse_close(lse_p[b:b + 1].cpu().numpy(), rl)

@@ -275,8 +275,9 @@ def fa_forward_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, is_ca
 
 def fa_forward_paged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                      seqused_k: torch.Tensor, *, is_causal=False, scale: Optional[float] = None,
-                     num_splits: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Decode / speculative tokens against a paged KV cache.  q [B, Hq, Sq, D] with Sq * (Hq / Hk) <= 16;
+                     num_splits: int = 0, kernel: int = FA_KERNEL_AUTO) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Decode / speculative tokens (Sq * (Hq / Hk) <= 16: the split-KV kernel) or a longer query chunk (a chunk of a
+    chunked prefill: the tile kernel) against a paged KV cache.  q [B, Hq, Sq, D];
     k_pages / v_pages [pages, page_size, Hk, D] (any strides, contiguous last dim; page_size a multiple of 32);
     block_table int32 [B, max_pages] on the device: the pages of each sequence in order; seqused_k int32 [B]: how many
     keys each sequence holds.  -> out [B, Hq, Sq, D], lse [B, Hq, Sq].  Bottom-right causal when `is_causal`."""
@@ -288,7 +289,7 @@ def fa_forward_paged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
     # k / v stand in as [B, seqlen_k, Hk, D] views for the stride fields: batch stride = page stride
     p = make_params(q.transpose(1, 2), k_pages, v_pages, out, lse, scale=scale, is_causal=is_causal,
-                    kernel=FA_KERNEL_SPLITKV, num_splits=num_splits, seqused_k=seqused_k)
+                    kernel=kernel, num_splits=num_splits, seqused_k=seqused_k)
     p.seqlen_k = block_table.shape[1] * page_size
     p.block_table = block_table.data_ptr()
     p.block_table_stride = block_table.stride(0)

@@ -93,6 +93,11 @@ __device__ __forceinline__ void dma16s(const unsigned char* sbase, unsigned voff
                : "m0");
 }
 
+// Same, with a per-lane 64-bit global address and the LDS destination given as a wavefront-uniform LDS byte address.
+__device__ __forceinline__ void dma16v(const unsigned char* gptr, unsigned lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_wave_base), "v"(gptr) : "m0");
+}
+
 // Transposed LDS read: within each group of 16 lanes, lane j receives element (j % 4) of the four 8-byte pieces
 // addressed by lanes 4 i + j / 4 (i = 0..3) of the same group.
 __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {

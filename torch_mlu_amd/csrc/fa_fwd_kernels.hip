@@ -50,7 +50,11 @@ using namespace fa;
 // entries are zeroed in the P operand of the PV product and 1 / (keep probability) is folded into the final normalisation.
 // DMASK (with DROP): also write the keep-mask out for tests; a variant of its own because the extra stores cost
 // registers (30 spilled at head_dim 128) that the plain dropout kernel does not have to pay.
-template <typename T, int DP, int MINB, int BIAS, bool DROP = false, bool DMASK = false>
+// PAGED: K and V are pools of pages [page][row][kv head][D] (dense mode; a.k_sb / a.v_sb are the page strides) and key
+// row r of sequence b lives in page block_table[b][r / page_size]: a prefill chunk against a paged KV cache.  A DMA
+// instruction covers at most 32 consecutive rows that start at a multiple of its length and page_size is a multiple
+// of 32, so the rows of one instruction lie inside one page.
+template <typename T, int DP, int MINB, int BIAS, bool DROP = false, bool DMASK = false, bool PAGED = false>
 __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   constexpr int CPR = DP / 8;          // 16-byte chunks per row
   constexpr int ROWB = DP * 2;         // bytes per LDS row
@@ -186,8 +190,9 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   const int off = a.causal_tl ? 0 : Lk - Lq;  // causal: col visible iff col <= row + off
 
   const unsigned char* qp = a.q + qb + (int64_t)q0 * a.q_ss + (int64_t)h * a.q_sh;
-  const unsigned char* kp = a.k + kb + (int64_t)k0 * a.k_ss + (int64_t)hk * a.k_sh;
-  const unsigned char* vp = a.v + vb + (int64_t)k0 * a.v_ss + (int64_t)hk * a.v_sh;
+  // (PAGED: the pools' first page, this kv head; the page is added per DMA instruction)
+  const unsigned char* kp = a.k + (PAGED ? 0 : kb + (int64_t)k0 * a.k_ss) + (int64_t)hk * a.k_sh;
+  const unsigned char* vp = a.v + (PAGED ? 0 : vb + (int64_t)k0 * a.v_ss) + (int64_t)hk * a.v_sh;
   const int D = a.head_dim;
 
   // ---- DMA bookkeeping ---------------------------------------------------------------------------------
@@ -212,17 +217,73 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   const int last_k = Lk - 1;
   const unsigned lds0 = (unsigned)(uintptr_t)(LDS_AS unsigned char*)smem + wave * 1024;
 
+  // PAGED: the pages of a tile's two 32-row halves and the halves' first rows inside their pages.  The table entries
+  // are scalar loads; they are requested two tiles ahead of the DMA that needs them (page_next: tile j + 1 while tile
+  // j is computed, page_after: tile j + 2), walking the table with a running (entry, row) pair instead of a division.
+  struct PageRef {
+    int pg0, pg1, ro0, ro1;
+  };
+  const int32_t* tbl = nullptr;
+  int psz = 32, lk_idx = 0, lk_ro = 0, lk_max = 0;
+  if constexpr (PAGED) {
+    tbl = a.block_table + (int64_t)b * a.bt_stride;
+    psz = a.page_size;
+    lk_max = max(last_k, 0) / psz;  // the last entry that belongs to this sequence's keys
+  }
+  auto lookup_seek = [&](int j) {  // the next lookup is tile j's
+    lk_idx = (j * BN) / psz;
+    lk_ro = j * BN - lk_idx * psz;
+  };
+  auto lookup_next = [&]() -> PageRef {
+    int i1 = lk_idx, o1 = lk_ro + 32;
+    if (o1 >= psz) {
+      o1 -= psz;
+      ++i1;
+    }
+    // (wavefront-uniform by construction; said so, since the DMA's base address must live in scalar registers)
+    const PageRef r{__builtin_amdgcn_readfirstlane(tbl[min(lk_idx, lk_max)]),
+                    __builtin_amdgcn_readfirstlane(tbl[min(i1, lk_max)]), __builtin_amdgcn_readfirstlane(lk_ro),
+                    __builtin_amdgcn_readfirstlane(o1)};
+    lk_ro += BN;
+    while (lk_ro >= psz) {
+      lk_ro -= psz;
+      ++lk_idx;
+    }
+    return r;
+  };
+  PageRef page_next{0, 0, 0, 0}, page_after{0, 0, 0, 0};
   // One DMA instruction of a tile that lies fully inside the sequence: `which` = 0 (K) or 1 (V), block i of tile j
   // into buffer buf.  Only scalar address arithmetic.  These are issued one at a time between MFMAs so that a
   // wavefront never sits in the (narrow, CU-shared) vector-memory issue queue with nothing else to do.
-  auto issue_one = [&](int j, int buf, int which, int i) {
+  auto issue_one = [&](int j, int buf, int which, int i, const PageRef& pr) {
     const unsigned dst = lds0 + (which ? 2 * TILE : 0) + buf * TILE + i * 4096;
     const unsigned ss = which ? v_ss : k_ss;
-    const unsigned char* base = (which ? vp : kp) + (uint64_t)(unsigned)(j * BN + i * 4 * RPI) * ss;
+    const unsigned char* base;
+    if constexpr (PAGED) {
+      const bool hi = i * 4 * RPI >= 32;  // which half of the tile this instruction's rows are in
+      const int64_t sb = which ? a.v_sb : a.k_sb;
+      base = (which ? vp : kp) + (int64_t)(hi ? pr.pg1 : pr.pg0) * sb +
+             (uint64_t)(unsigned)((hi ? pr.ro1 : pr.ro0) + (i * 4 * RPI) % 32) * ss;
+    } else {
+      base = (which ? vp : kp) + (uint64_t)(unsigned)(j * BN + i * 4 * RPI) * ss;
+    }
     dma16s(base, which ? voff : ((DP == 256 && (i & 1)) ? koff_odd : koff), dst);
   };
   // A whole tile at once, rows clamped to the last valid one (first tile, and the partial tile at the end of K).
   auto issue_tile = [&](int j, int buf) {
+    if constexpr (PAGED) {
+      // per lane: its (clamped) row's page from the table, then a 64-bit address
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int r = min(j * BN + dma_r + i * 4 * RPI, last_k);
+        const int e = r / psz;
+        const int64_t pg = tbl[e];
+        const unsigned ro = (unsigned)(r - e * psz);
+        dma16v(kp + pg * a.k_sb + (uint64_t)ro * k_ss + ((DP == 256 && (i & 1)) ? lck_odd : lck) * 16, lds0 + buf * TILE + i * 4096);
+        dma16v(vp + pg * a.v_sb + (uint64_t)ro * v_ss + lcv * 16, lds0 + 2 * TILE + buf * TILE + i * 4096);
+      }
+      return;
+    }
     const int rmax = last_k - j * BN;  // >= 0: the tile exists
     const unsigned char* kt = kp + (uint64_t)(unsigned)(j * BN) * k_ss;
     const unsigned char* vt = vp + (uint64_t)(unsigned)(j * BN) * v_ss;
@@ -286,6 +347,13 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
   const int row = m0 + 32 * wave + c32;  // this lane's query row (lanes l and l^32 share it)
   if (own) __syncthreads();  // the previous block's last LDS reads are done
   if (ntiles > jt0) issue_tile(jt0, 0);
+  if constexpr (PAGED) {
+    if (ntiles > jt0) {
+      lookup_seek(jt0 + 1);
+      page_next = lookup_next();
+      page_after = lookup_next();
+    }
+  }
 
   // ---- Q fragments (B operand): lane (c32, g) holds Q[row][16 ks + 8 g .. +8] -----------------------------
   // The block's 128 rows come in through LDS like two K tiles (rows 0-63 into K buffer 1, rows 64-127 into V buffer
@@ -375,6 +443,11 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
     const bool more = j + 1 < ntiles;
     const bool spread = more && (j + 2) * BN <= Lk && !(a.is_causal && j * BN > wave_row_hi + off);
     if (more && !spread) issue_tile(j + 1, BUF ^ 1);
+    const PageRef pages = page_next;  // (PAGED) of tile j + 1
+    if constexpr (PAGED) {
+      page_next = page_after;
+      page_after = lookup_next();  // tile j + 3
+    }
 
     // wavefront-uniform skip: every score of this tile is masked for all 32 rows of this wavefront
     if (a.is_causal && j * BN > wave_row_hi + off) return;
@@ -409,7 +482,7 @@ __global__ void __launch_bounds__(256, MINB) fa_tile_kernel(const KArgs a) {
         // next tile's K and V: 2 NI DMA instructions spread over the KS k-steps (K block i, then V block i)
         if (spread) {
 #pragma unroll
-          for (int x = (ks * 2 * NI) / KS; x < ((ks + 1) * 2 * NI) / KS; ++x) issue_one(j + 1, BUF ^ 1, x & 1, x >> 1);
+          for (int x = (ks * 2 * NI) / KS; x < ((ks + 1) * 2 * NI) / KS; ++x) issue_one(j + 1, BUF ^ 1, x & 1, x >> 1, pages);
         }
         if (ks + 2 < KS) {
           ka[ks & 1][0] = *(LDS_AS const s16x8*)(kptr[ks + 2] + BUF * TILE);
@@ -1094,10 +1167,10 @@ KArgs make_args(const fa_fwd_params* p, int kern, int ns, void* ws) {
   return a;
 }
 
-template <typename T, int DP, int MINB, int BIAS, bool DROP = false, bool DMASK = false>
+template <typename T, int DP, int MINB, int BIAS, bool DROP = false, bool DMASK = false, bool PAGED = false>
 int launch_tile(KArgs a, hipStream_t st) {
   constexpr int lds = 4 * 64 * DP * 2 + (BIAS == 2 ? 4 * 4096 : 0);
-  constexpr auto kfn = fa_tile_kernel<T, DP, MINB, BIAS, DROP, DMASK>;
+  constexpr auto kfn = fa_tile_kernel<T, DP, MINB, BIAS, DROP, DMASK, PAGED>;
   if (!ensure_dynamic_lds<kfn>(lds)) return FA_ERR_LAUNCH;
   const int nblk = (a.seqlen_q + 127) / 128;
   a.pair = (DP != 256 && a.n_splits == 1 && a.is_causal && nblk >= 2 &&
@@ -1187,6 +1260,11 @@ int dispatch(const KArgs& a, int kern, hipStream_t st) {
     if (dp == 64) return launch_tile<T, 64, 2, 1>(a, st);
     if (dp == 128) return launch_tile<T, 128, 2, 1>(a, st);
     return launch_tile<T, 256, 1, 1>(a, st);
+  }
+  if (a.block_table) {  // a prefill chunk against a paged KV cache
+    if (dp == 64) return launch_tile<T, 64, 2, 0, false, false, true>(a, st);
+    if (dp == 128) return launch_tile<T, 128, 2, 0, false, false, true>(a, st);
+    return launch_tile<T, 256, 1, 0, false, false, true>(a, st);
   }
   if (dp == 64) return launch_tile<T, 64, 2, false>(a, st);
   if (dp == 128) return launch_tile<T, 128, 2, false>(a, st);

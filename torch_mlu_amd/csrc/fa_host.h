@@ -68,15 +68,20 @@ inline int validate(const fa_fwd_params* p) {
   if ((uintptr_t)p->seqused_k & 3) return FA_ERR_BAD_ARG;
   if (p->reserved3 != 0) return FA_ERR_BAD_ARG;
   if (p->block_table) {
-    // paged K/V: dense mode, a shape the split-KV kernel takes, pages of whole 32-row blocks, a table wide enough
+    // paged K/V: dense mode, pages of whole 32-row blocks, a table wide enough.  Decode-shaped calls (what the
+    // split-KV kernel takes) may use dropout; a prefill chunk (the tile kernel) may not.
     if ((uintptr_t)p->block_table & 3) return FA_ERR_BAD_ARG;
     if (p->page_size <= 0 || p->block_table_stride < 0) return FA_ERR_BAD_ARG;
     if (p->page_size % 32) return FA_ERR_UNSUPPORTED;
     if (p->block_table_stride < ((int64_t)p->seqlen_k + p->page_size - 1) / p->page_size) return FA_ERR_BAD_ARG;
     if (p->cu_seqlens_q || p->bias || (p->dropout_p > 0.f && p->dropout_mask) || p->is_causal == FA_MASK_CAUSAL_TOP_LEFT)
       return FA_ERR_UNSUPPORTED;
-    if (p->kernel != FA_KERNEL_AUTO && p->kernel != FA_KERNEL_SPLITKV) return FA_ERR_UNSUPPORTED;
-    if (p->seqlen_q < 1 || (int64_t)p->seqlen_q * (p->heads_q / p->heads_k) > 16) return FA_ERR_UNSUPPORTED;
+    if (p->seqlen_q < 1) return FA_ERR_UNSUPPORTED;
+    const bool decode_shaped = (int64_t)p->seqlen_q * (p->heads_q / p->heads_k) <= 16;
+    if (p->kernel == FA_KERNEL_SPLITKV && !decode_shaped) return FA_ERR_UNSUPPORTED;
+    if ((p->kernel == FA_KERNEL_TILE || !decode_shaped) && p->dropout_p > 0.f) return FA_ERR_UNSUPPORTED;
+    // the pools' pages are addressed as 64-bit page x stride; rows inside a page as 32-bit row x stride
+    if (p->k_stride_b < 0 || p->v_stride_b < 0) return FA_ERR_BAD_ARG;
   }
   if (p->bias) {
     if (((uintptr_t)p->bias & 7) || p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_q < 0 ||
@@ -95,7 +100,9 @@ inline int validate(const fa_fwd_params* p) {
 inline void plan(const fa_fwd_params* p, int* kernel, int* splits) {
   int kern = p->kernel;
   const int group = p->heads_q / p->heads_k;
-  if (p->block_table) kern = FA_KERNEL_SPLITKV;  // the only kernel that reads a page table (validate() checked the shape)
+  // a page table: decode-shaped calls go to the split-KV kernel, a prefill chunk to the tile kernel's paged variant
+  if (p->block_table && kern == FA_KERNEL_AUTO)
+    kern = ((int64_t)p->seqlen_q * group <= 16) ? FA_KERNEL_SPLITKV : FA_KERNEL_TILE;
   if (kern == FA_KERNEL_AUTO)
     kern = (p->seqlen_q >= 1 && (int64_t)p->seqlen_q * group <= 16 && p->seqlen_k >= 256 && !p->bias && p->is_causal != FA_MASK_CAUSAL_TOP_LEFT && !(p->dropout_p > 0.f && p->dropout_mask))
                ? FA_KERNEL_SPLITKV

@@ -41,7 +41,7 @@ def sdpa(query, key, value, *, is_causal: bool = False, scale: Optional[float] =
 
 def paged_attention(query, key_pages, value_pages, block_table, seqused_k, *, is_causal: bool = False,
                     scale: Optional[float] = None):
-    """Decode (or a few speculative tokens: Sq * Hq / Hk <= 16) against a paged KV cache, through the C ABI
+    """Decode, a few speculative tokens, or a chunk of a chunked prefill against a paged KV cache, through the C ABI
     (`fa_fwd_params.block_table`; the reference's ops have no such argument).  query [B, Hq, Sq, D]; key_pages /
     value_pages [pages, page_size, Hk, D] with page_size a multiple of 32; block_table int32 [B, max_pages] and
     seqused_k int32 [B] on the device.  -> (out [B, Hq, Sq, D], logsumexp [B, Hq, Sq]).  Inference only."""
