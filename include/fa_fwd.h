@@ -113,8 +113,8 @@ typedef struct fa_fwd_params {
   int32_t dtype;     /* FA_DTYPE_* */
   int32_t is_causal; /* FA_MASK_* (0 / 1 keep their old meaning) */
   int32_t kernel;    /* FA_KERNEL_* */
-  int32_t num_splits; /* slices of the key range: 0 = choose, else 1..FA_MAX_SPLITS (split-KV kernel; tile kernel without
-                         dropout, where each query block's tiles are cut into slices) */
+  int32_t num_splits; /* slices of the key range: 0 = choose, else 1..FA_MAX_SPLITS (split-KV kernel; tile kernel, where
+                         each query block's tiles are cut into slices) */
   int32_t reserved;  /* must be 0 */
 
   const void* bias;  /* device or NULL */

@@ -171,9 +171,9 @@ def test_plan_split_count(batch, heads_k, seqlen_k, want):
     (dict(batch=1, heads_q=8, heads_k=8, seqlen_q=4096, seqlen_k=4096), "tile", 2),       # small-batch prefill
     (dict(batch=2, heads_q=8, heads_k=8, seqlen_q=2048, seqlen_k=2048), "tile", 1),       # slices would be too short
     (dict(batch=1, heads_q=64, heads_k=1, seqlen_q=1, seqlen_k=32768), "tile", 8),        # group too wide for split-KV
-    (dict(batch=1, heads_q=32, heads_k=8, seqlen_q=128, seqlen_k=32768, dropout_p=0.1), "tile", 1),
+    (dict(batch=1, heads_q=32, heads_k=8, seqlen_q=128, seqlen_k=32768, dropout_p=0.1), "tile", 16),  # dropout slices too
     (dict(batch=8, heads_q=32, heads_k=8, seqlen_q=4, seqlen_k=32768, dropout_p=0.1), "splitkv", 4),   # dropout: both kernels
-    (dict(batch=8, heads_q=32, heads_k=8, seqlen_q=4, seqlen_k=32768, dropout_p=0.1, dropout_mask=0x9000), "tile", 1),
+    (dict(batch=8, heads_q=32, heads_k=8, seqlen_q=4, seqlen_k=32768, dropout_p=0.1, dropout_mask=0x9000), "tile", 2),
     (dict(batch=8, heads_q=32, heads_k=8, seqlen_q=4, seqlen_k=32768), "splitkv", 4),     # 4 rows x 4 heads = 16 columns
     (dict(batch=8, heads_q=32, heads_k=8, seqlen_q=5, seqlen_k=32768), "tile", 2),        # 20 columns: tile kernel
     (dict(batch=8, heads_q=8, heads_k=8, seqlen_q=16, seqlen_k=32768), "splitkv", 4),

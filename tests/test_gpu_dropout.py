@@ -368,3 +368,30 @@ def test_debug_mask_of_a_sequence_longer_than_stated_stays_inside_its_plane(pair
         got = dbg[b, h].float().cpu().numpy()
         assert (got[:n, :n] == np.where(vis, np.where(keep, 1.0, -1.0), 0.0)).all()
         assert (got[n:] == 0).all() and (got[:, n:] == 0).all()
+
+
+@pytest.mark.parametrize("dtype,D", [(BF, 128), (HF, 64), (BF, 256)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_sliced_tile_kernel_with_dropout(dtype, D, causal):
+    """A chunk against a long K/V with dropout: the tile kernel cuts each query block's key range into slices (the mask
+    is a function of row and key only, so every slice draws the bits the unsliced kernel draws) and the merge applies the
+    keep-probability factor.  Forced slice counts and the automatic plan against the unsliced call and the oracle fed
+    with the documented mask; the debug mask of a sliced call is the unsliced one's."""
+    B, Hq, Hk, Sq, Sk, p, seed, offset = 1, 4, 2, 150, 4096 + 77, 0.2, 4321, 16
+    q, k, v, _ = _inputs(B, Hq, Hk, Sq, Sk, D, dtype, 500 + D)
+    qd, kd, vd = (t.to(DEV) for t in (q, k, v))
+    kw = dict(is_causal=causal, dropout_p=p, philox_seed=seed, philox_offset=offset, kernel=capi.FA_KERNEL_TILE)
+    dbg1 = torch.zeros((B, Hq, Sq, Sk), dtype=dtype, device=DEV)
+    out1, lse1 = capi.fa_forward_dense(qd, kd, vd, num_splits=1, dropout_mask=dbg1, **kw)
+    keep = _expected_mask(seed, offset, B, Hq, Sq, Sk, p)
+    ro, rl = oracle.sdpa_oracle(q, k, v, is_causal=causal, dropout_p=oracle.dropout_effective_p(p), dropout_mask=keep)
+    out_close(out1.float().cpu().numpy(), ro, dtype, tol=3e-2 if dtype == BF else 8e-3)
+    lse_close(lse1.cpu().numpy(), rl)
+    assert _plan_of(qd, kd, vd, **kw)[1] > 1   # the automatic plan slices this shape
+    for ns in (0, 3, 8):
+        dbg = torch.zeros_like(dbg1)
+        out, lse = capi.fa_forward_dense(qd, kd, vd, num_splits=ns, dropout_mask=dbg, **kw)
+        assert torch.equal(dbg, dbg1), ns
+        assert (out.float() - out1.float()).abs().max().item() <= (2e-2 if dtype == BF else 4e-3), ns
+        assert (lse - lse1).abs().max().item() <= 1e-4, ns
+        out_close(out.float().cpu().numpy(), ro, dtype, tol=3e-2 if dtype == BF else 8e-3)

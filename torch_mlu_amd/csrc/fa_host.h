@@ -125,8 +125,9 @@ inline void plan(const fa_fwd_params* p, int* kernel, int* splits) {
     }
     const int nblk = (p->seqlen_k + 31) / 32;
     if (ns > nblk) ns = nblk > 0 ? nblk : 1;
-  } else if (!(p->dropout_p > 0.f) && p->seqlen_q > 0) {
-    // Tile kernel, no dropout (dense or packed, an additive bias and either causal alignment are fine): with few query blocks against a long K/V (chunked prefill, speculative decoding, a
+  } else if (p->seqlen_q > 0) {
+    // Tile kernel (dense or packed; an additive bias, either causal alignment and dropout — whose mask is a function
+    // of the row and the key, not of the slice — are fine): with few query blocks against a long K/V (chunked prefill, speculative decoding, a
     // GQA group too wide for the split-KV kernel) the key range of each block is cut into slices so that the CUs
     // have two workgroups each; a slice keeps at least 32 tiles (2048 keys), or 16 where the chunk is much shorter
     // than the cache, so that a causal mask leaves every slice equally full.  Partials go through the workspace.
