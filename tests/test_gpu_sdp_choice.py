@@ -181,6 +181,49 @@ def test_nested_tensors_reach_the_packed_kernel(causal):
             assert np.abs(got - w).max() <= 2 * 2.0 ** -11 * max(np.abs(w).max(), 0.25)
 
 
+def test_nested_tensors_on_the_mem_efficient_kernels():
+    """Nested q / k / v, inference: the reference sends nested inputs to its mem-efficient kernels first and takes them
+    there without gradients (sdp_utils.cpp:22-24,82-87).  Here they are eligible for both fused backends (flash is asked
+    first); with flash switched off the selector answers mem-efficient and this build's nested wrapper of
+    aten::_scaled_dot_product_efficient_attention packs the sequences for the packed op.  The wrapper also takes a dense
+    attn_bias [B, H, max_q, max_k] indexed from each sequence's first row and key — F.scaled_dot_product_attention
+    itself refuses an explicit mask with nested inputs, so that is reached through the op (PyTorch's own nested wrapper
+    of that op drops the bias).  Query and key lengths differ; with gradients wanted the path is not taken."""
+    H, D = 4, 64
+    lq, lk = [37, 128, 5, 200], [50, 128, 9, 131]
+    qp, q = _nested(lq, H, D, HF, 11)
+    kp, k = _nested(lk, H, D, HF, 12)
+    vp, v = _nested(lk, H, D, HF, 13)
+    qt, kt, vt = (x.transpose(1, 2) for x in (q, k, v))
+    with torch.no_grad(), sdp_kernel(enable_flash=False, enable_math=True, enable_mem_efficient=True):
+        assert torch._fused_sdp_choice(qt, kt, vt, None, 0.0, False) == SDPBackend.EFFICIENT_ATTENTION
+        n0 = torch_mlu_amd.launch_count()
+        out = F.scaled_dot_product_attention(qt, kt, vt)
+        assert torch_mlu_amd.launch_count() == n0 + 1 and out.is_nested
+    for i, o in enumerate(out.transpose(1, 2).unbind()):
+        qi, ki, vi = (p[i].transpose(0, 1)[None] for p in (qp, kp, vp))
+        ref, _ = oracle.sdpa_oracle(qi, ki, vi)
+        out_close(o.transpose(0, 1)[None].float().cpu().numpy(), ref, HF)
+    # with a bias, through the op
+    g = torch.Generator().manual_seed(14)
+    B, mq, mk = len(lq), max(lq), max(lk)
+    bias = (torch.randn(B, 1, mq, mk, generator=g) * 0.5).to(HF)
+    bias[:, :, :, 1::3] = float("-inf")
+    with torch.no_grad():
+        n0 = torch_mlu_amd.launch_count()
+        out = torch.ops.aten._scaled_dot_product_efficient_attention(qt, kt, vt, bias.to(DEV), False)[0]
+        assert torch_mlu_amd.launch_count() == n0 + 1 and out.is_nested
+    bn = bias.double().numpy()
+    for i, o in enumerate(out.transpose(1, 2).unbind()):
+        qi, ki, vi = (p[i].transpose(0, 1)[None] for p in (qp, kp, vp))
+        ref, _ = oracle.sdpa_oracle(qi, ki, vi, attn_bias=bn[i:i + 1, :, :lq[i], :lk[i]])
+        out_close(o.transpose(0, 1)[None].float().cpu().numpy(), ref, HF)
+    # training with nested inputs is not this path's (check_requires_grad_and_nested): flash takes it
+    ql = torch.nested.nested_tensor(qp).to(DEV).requires_grad_()
+    why = torch.ops.torch_mlu_amd._mem_efficient_refusal_reason(ql.transpose(1, 2), kt, vt)
+    assert "training with NT inputs" in why
+
+
 def test_nested_refusals():
     """An empty sequence and a mask are refused for nested inputs with the reference's messages; with only the flash
     backend allowed the call then raises."""

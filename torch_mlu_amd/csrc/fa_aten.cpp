@@ -19,6 +19,8 @@
 //   * LSE is returned as [B, Hq, Sq] (dense) / [Hq, total_q] (packed) without the pad-to-16 of
 //     FlashAttention_internal.cpp:261-265, which is what the installed PyTorch's shape contract says.
 #include <ATen/ATen.h>
+#include <ATen/NestedTensorImpl.h>
+#include <ATen/native/nested/NestedTensorUtils.h>
 #include <ATen/hip/HIPContext.h>
 #include <ATen/hip/HIPGeneratorImpl.h>
 #include <c10/hip/HIPGraphsC10Utils.h>
@@ -31,6 +33,7 @@
 
 #include <atomic>
 #include <cmath>
+#include <cstring>
 #include <limits>
 #include <map>
 #include <mutex>
@@ -555,8 +558,6 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
     std::optional<c10::SymInt> max_seqlen_q, std::optional<c10::SymInt> max_seqlen_k, double dropout_p,
     int64_t custom_mask_type, bool compute_log_sumexp, std::optional<double> scale,
     const std::optional<at::Tensor>& seqlen_k, std::optional<int64_t> window_size) {
-  (void)max_seqlen_q;
-  (void)max_seqlen_k;
   // the reference's checks, in its order (attention.cpp:405-423)
   TORCH_CHECK(query.dim() == 4 && key.dim() == 4 && value.dim() == 4, "query, key and value must be 4-dimensional "
               "(batch, seq_len, num_heads, head_dim)");
@@ -569,7 +570,19 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   // cu_seqlens (attention.cpp:431-466): offsets of the sequences in the rows of the [B * S, H, D] view of the inputs
   const bool packed = cu_seqlens_q.has_value() && cu_seqlens_q->defined();
   TORCH_CHECK(packed == (cu_seqlens_k.has_value() && cu_seqlens_k->defined()), "cu_seqlens_q and cu_seqlens_k must be given together");
-  if (packed) check_efficient_cu_seqlens(*cu_seqlens_q, *cu_seqlens_k, query.size(0));
+  // A second packed convention, the installed PyTorch's own (what its nested-tensor path passes): batch 1, all
+  // sequences' rows one after the other in [1, total, H, D] tensors, cu_seqlens of (number of sequences + 1) entries
+  // and the two maximum lengths.  A bias is then [sequences, H, max_seqlen_q, max_seqlen_k], indexed by sequence and by
+  // the row / key position inside the sequence.
+  const bool ragged = packed && query.size(0) == 1 && cu_seqlens_q->dim() == 1 && cu_seqlens_q->size(0) != 2;
+  if (ragged) {
+    TORCH_CHECK(max_seqlen_q.has_value() && max_seqlen_k.has_value(),
+                "cu_seqlens with batch size 1 need max_seqlen_q and max_seqlen_k");
+    TORCH_CHECK(cu_seqlens_q->size(0) >= 2, "cu_seqlens_q must have at least two entries");
+    check_efficient_cu_seqlens(*cu_seqlens_q, *cu_seqlens_k, cu_seqlens_q->size(0) - 1);
+  } else if (packed) {
+    check_efficient_cu_seqlens(*cu_seqlens_q, *cu_seqlens_k, query.size(0));
+  }
   TORCH_CHECK(!window_size.has_value() || *window_size <= 0, "efficient attention forward: sliding window is not supported");
   TORCH_CHECK(dropout_p >= 0.0 && dropout_p < 1.0, "efficient attention forward: dropout_p must be in [0, 1), got ", dropout_p);
   TORCH_CHECK(custom_mask_type >= 0 && custom_mask_type <= 2, "custom_mask_type must be 0, 1 or 2");
@@ -600,8 +613,12 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   at::Tensor lse = packed ? at::full({Hq, B * Sq}, std::numeric_limits<float>::infinity(), q.options().dtype(at::kFloat))
                           : at::empty({B, Hq, Sq}, q.options().dtype(at::kFloat));
 
+  // what the kernels see as (batch, seqlen_q, seqlen_k): the tensors' own, or the ragged convention's
+  const int64_t nseq = ragged ? cu_seqlens_q->size(0) - 1 : B;
+  const int64_t kSq = ragged ? max_seqlen_q->expect_int() : Sq, kSk = ragged ? max_seqlen_k->expect_int() : Sk;
+  TORCH_CHECK(kSq >= 0 && kSk >= 0 && kSq <= INT32_MAX && kSk <= INT32_MAX && nseq <= INT32_MAX, "sequence length too large");
   at::Tensor bias_e;
-  if (bias.has_value() && bias->defined()) bias_e = bias_for_kernels(*bias, dt, B, Hq, Sq, Sk);
+  if (bias.has_value() && bias->defined()) bias_e = bias_for_kernels(*bias, dt, nseq, Hq, kSq, kSk);
 
   fa_fwd_params p{};
   p.q = q.data_ptr(); p.k = k.data_ptr(); p.v = v.data_ptr(); p.out = output.data_ptr();
@@ -617,11 +634,11 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   } else {
     p.lse_stride_b = lse.stride(0); p.lse_stride_h = lse.stride(1); p.lse_stride_s = lse.stride(2);
   }
-  p.batch = static_cast<int32_t>(B);
+  p.batch = static_cast<int32_t>(nseq);
   p.heads_q = static_cast<int32_t>(Hq);
   p.heads_k = static_cast<int32_t>(Hk);
-  p.seqlen_q = static_cast<int32_t>(Sq);
-  p.seqlen_k = static_cast<int32_t>(Sk);
+  p.seqlen_q = static_cast<int32_t>(kSq);
+  p.seqlen_k = static_cast<int32_t>(kSk);
   p.head_dim = static_cast<int32_t>(D);
   p.scale = softmax_scale;
   p.dtype = dt == at::kBFloat16 ? FA_DTYPE_BF16 : FA_DTYPE_FP16;
@@ -630,10 +647,10 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   p.kernel = FA_KERNEL_AUTO;
   at::Tensor used;
   if (seqlen_k.has_value() && seqlen_k->defined()) {
-    used = checked_seqused_k(*seqlen_k, B, query, key, value, "seqlen_k");
+    used = checked_seqused_k(*seqlen_k, nseq, query, key, value, "seqlen_k");
     p.seqused_k = used.data_ptr<int32_t>();
   }
-  if (bias_e.defined() && Sk > 0) {
+  if (bias_e.defined() && kSk > 0) {
     p.bias = bias_e.data_ptr();
     p.bias_stride_b = bias_e.stride(0); p.bias_stride_h = bias_e.stride(1); p.bias_stride_q = bias_e.stride(2);
   }
@@ -641,7 +658,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
   at::Tensor seed_t = at::empty({}, q.options().dtype(at::kLong));
   at::Tensor offset_t = at::empty({}, q.options().dtype(at::kLong));
   if (dropout_p > 0.0) {
-    take_philox_state(Sq, Sk, p);
+    take_philox_state(kSq, kSk, p);
     p.dropout_p = static_cast<float>(dropout_p);
     p.rng_seed_out = seed_t.data_ptr<int64_t>();
     p.rng_offset_out = offset_t.data_ptr<int64_t>();
@@ -656,7 +673,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, c10::SymInt, c10::Sym
     g_launches.fetch_add(1, std::memory_order_relaxed);
   }
   if (!compute_log_sumexp) lse = packed ? at::empty({Hq, 0}, q.options().dtype(at::kFloat)) : at::empty({B, Hq, 0}, q.options().dtype(at::kFloat));
-  return std::make_tuple(output, lse, seed_t, offset_t, c10::SymInt(Sq), c10::SymInt(Sk));
+  return std::make_tuple(output, lse, seed_t, offset_t, c10::SymInt(kSq), c10::SymInt(kSk));
 }
 
 // ---- _scaled_dot_product_efficient_attention -------------------------------------------------------------------
@@ -673,6 +690,65 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> scaled_dot_product_ef
   (void)mq;
   (void)mk;
   return std::make_tuple(out.transpose(1, 2), lse, seed, offset);
+}
+
+// ---- _scaled_dot_product_efficient_attention on nested (ragged) tensors, inference ------------------------------
+// The reference prefers its mem-efficient kernels for nested inputs and accepts them there without gradients
+// (sdp_utils.cpp:22-24,82-87).  PyTorch's own nested-tensor wrapper of this op drops the attn_bias, so nested inputs
+// with an attn_mask get this one: query / key / value are nested [B, H, S*, D] views of [B, S*, H, D] data (what
+// F.scaled_dot_product_attention is given), packed here into [1, total, H, D] buffers with cu_seqlens from the nested
+// sizes and handed to the packed op above; attn_bias is dense, broadcastable to [B, H, max S_q, max S_k], indexed from
+// each sequence's first row and key.
+namespace {
+struct PackedNested {
+  at::Tensor buf;    // [1, total, H, D]
+  at::Tensor cu;     // int32 [B + 1] on the device
+  at::Tensor sizes;  // the nested sizes of the [B, S*, H, D] tensor
+  int64_t max_len;
+};
+PackedNested pack_nested(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_nested() && t.dim() == 4, name, " must be a nested tensor of 4 dimensions (batch, num_heads, seq_len, head_dim)");
+  const at::Tensor c = t.transpose(1, 2).contiguous();  // [B, S*, H, D], rows of all sequences one after the other
+  const auto* impl = at::native::get_nested_tensor_impl(c);
+  const at::Tensor sizes = impl->get_nested_sizes();  // int64 [B, 3] on the CPU: (S_b, H, D)
+  const int64_t B = sizes.size(0);
+  TORCH_CHECK(B > 0 && sizes.size(1) == 3, name, ": unexpected nested structure");
+  const auto sz = sizes.accessor<int64_t, 2>();
+  const int64_t H = sz[0][1], D = sz[0][2];
+  std::vector<int32_t> cu(B + 1, 0);
+  int64_t total = 0, mx = 0;
+  for (int64_t b = 0; b < B; ++b) {
+    TORCH_CHECK(sz[b][1] == H && sz[b][2] == D, name, ": ragged num_heads or head_dim are not supported");
+    total += sz[b][0];
+    mx = std::max(mx, sz[b][0]);
+    TORCH_CHECK(total <= INT32_MAX, "sequence length too large");
+    cu[b + 1] = static_cast<int32_t>(total);
+  }
+  const at::Tensor buffer = impl->get_buffer();
+  TORCH_CHECK(buffer.numel() == total * H * D, name, ": unexpected nested storage");
+  at::Tensor cu_t = at::empty({B + 1}, at::TensorOptions().dtype(at::kInt).pinned_memory(true));
+  std::memcpy(cu_t.data_ptr<int32_t>(), cu.data(), sizeof(int32_t) * (B + 1));
+  return {buffer.view({1, total, H, D}), cu_t.to(t.device(), /*non_blocking=*/true), sizes, mx};
+}
+}  // namespace
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> scaled_dot_product_efficient_attention_nested(
+    const at::Tensor& query, const at::Tensor& key, const at::Tensor& value, const std::optional<at::Tensor>& attn_bias,
+    bool compute_log_sumexp, double dropout_p, bool is_causal, std::optional<double> scale) {
+  TORCH_CHECK(query.is_nested() && key.is_nested() && value.is_nested(),
+              "nested scaled_dot_product_attention needs query, key and value to be nested tensors");
+  TORCH_CHECK(!(attn_bias.has_value() && attn_bias->defined() && attn_bias->is_nested()), "attn_mask must be a dense tensor");
+  const PackedNested q = pack_nested(query, "query"), k = pack_nested(key, "key"), v = pack_nested(value, "value");
+  TORCH_CHECK(q.cu.size(0) == k.cu.size(0) && at::equal(k.sizes.select(1, 0), v.sizes.select(1, 0)),
+              "query, key and value must hold the same number of sequences, and key and value sequences of equal lengths");
+  auto [out, lse, seed, offset, mq, mk] = efficient_attention_forward(
+      q.buf, k.buf, v.buf, attn_bias, q.cu, k.cu, c10::SymInt(q.max_len), c10::SymInt(k.max_len), dropout_p,
+      is_causal ? 1 : 0, compute_log_sumexp, scale, std::nullopt, std::nullopt);
+  (void)mq;
+  (void)mk;
+  // [1, total, H, D] -> nested [B, S*, H, D] -> the [B, H, S*, D] view the dense wrapper returns too
+  const at::Tensor out_nt = at::native::wrap_buffer(out.view({-1}), q.sizes);
+  return std::make_tuple(out_nt.transpose(1, 2), lse, seed, offset);
 }
 
 // ---- _efficient_attention_backward ----------------------------------------------------------------------------
@@ -874,6 +950,11 @@ void validate_flash_inputs(const at::Tensor& query, const at::Tensor& key, const
 
 // HIP tensors carry the CUDA dispatch key in PyTorch-ROCm; registering here replaces PyTorch's own kernels for
 // the two ops (the dispatcher prints one "overriding a previously registered kernel" warning per op).
+TORCH_LIBRARY_IMPL(aten, NestedTensorCUDA, m) {
+  m.impl("_scaled_dot_product_efficient_attention",
+         TORCH_FN(torch_mlu_amd::scaled_dot_product_efficient_attention_nested));
+}
+
 TORCH_LIBRARY_IMPL(aten, CUDA, m) {
   m.impl("_scaled_dot_product_flash_attention", TORCH_FN(torch_mlu_amd::scaled_dot_product_flash_attention));
   m.impl("_flash_attention_forward", TORCH_FN(torch_mlu_amd::flash_attention_forward));

@@ -52,11 +52,25 @@ bool check_runtime_disabled_flash(const sdp_params&, bool debug) {
 
 bool has_nested_inputs(const sdp_params& p) { return p.query.is_nested() || p.key.is_nested() || p.value.is_nested(); }
 
-// The mem-efficient entry points of this build take dense tensors only.
-bool check_not_nested(const sdp_params& p, bool debug) {
-  if (has_nested_inputs(p)) {
-    if (debug) TORCH_WARN("The mem-efficient kernels of this build take dense tensors only; nested tensors go through "
-                          "the flash kernels.");
+// check_requires_grad_and_nested, sdp_utils.h (reference: sdp_utils.cpp:82-87): the mem-efficient kernels take nested
+// inputs for inference only.
+bool check_requires_grad_and_nested(const sdp_params& p, bool debug) {
+  if (has_nested_inputs(p) && input_requires_grad(p)) {
+    if (debug) TORCH_WARN("Memory efficient attention currently doesn't support training with NT inputs.");
+    return false;
+  }
+  return true;
+}
+
+// Not in the reference: the nested wrapper of this build's mem-efficient op packs three nested tensors that hold the
+// same number of sequences with one head count each (no broadcasting between them).
+bool check_nested_same_structure(const sdp_params& p, bool debug) {
+  const bool all = p.query.is_nested() && p.key.is_nested() && p.value.is_nested();
+  if (!all || p.query.size(0) != p.key.size(0) || p.query.size(0) != p.value.size(0) ||
+      p.key.size(1) != p.value.size(1) || p.key.size(1) <= 0 || p.query.size(1) % p.key.size(1) != 0 ||
+      (!p.enable_gqa && p.query.size(1) != p.key.size(1))) {
+    if (debug) TORCH_WARN("The mem-efficient kernels of this build need nested query, key and value with the same "
+                          "number of sequences and matching head counts.");
     return false;
   }
   return true;
@@ -277,8 +291,17 @@ bool check_this_build_mem_efficient(const sdp_params& p, bool debug) {
 
 // use_mem_efficient_attention, sdp_utils.cpp:76-95
 bool use_mem_efficient_attention(const sdp_params& p, bool debug) {
+  if (has_nested_inputs(p)) {
+    constexpr std::array<bool (*)(const sdp_params&, bool), 8> nested{
+        check_runtime_disabled_mem_efficient, check_requires_grad_and_nested, check_tensor_shapes,
+        check_head_dim_size_mem_efficient,    check_tensor_dtype,             check_nested_inputs,
+        check_nested_same_structure,          check_this_build_mem_efficient};
+    for (auto c : nested)
+      if (!c(p, debug)) return false;
+    return true;
+  }
   constexpr std::array<bool (*)(const sdp_params&, bool), 9> constraints{
-      check_runtime_disabled_mem_efficient, check_not_nested, check_tensor_shapes, check_batch_size_and_num_heads,
+      check_runtime_disabled_mem_efficient, check_requires_grad_and_nested, check_tensor_shapes, check_batch_size_and_num_heads,
       check_head_dim_size_mem_efficient, check_nonzero_sequence_lengths, check_last_dim_stride_equals_1,
       check_tensor_dtype, check_this_build_mem_efficient};
   for (auto c : constraints)
