@@ -289,6 +289,21 @@ def make_workload(name, dev):
         return dict(call=call, check=lambda: (0.0, 0.0), flops=0.0, bytes_kv=2.0 * src.numel() * 2,
                     desc="1 GiB device-to-device copy (counter calibration; bytes = read + written)", dtype="bf16",
                     bound="hbm", kernel="copy")
+    if name == "gemm8k":
+        # calibration workload for the instruction counters: a plain bf16 matrix product from the BLAS library, whose
+        # kernel issues next to no vector instructions beside its MFMAs.  SQ_INSTS_VALU / SQ_INSTS_MFMA of this kernel
+        # tells whether SQ_INSTS_VALU counts the MFMAs themselves (a ratio a little above 1) or not (well below 1).
+        n = 8192
+        a_, b_ = seeded((n, n), 90, bf).to(dev), seeded((n, n), 91, bf).to(dev)
+        c_ = torch.empty((n, n), dtype=bf, device=dev)
+
+        def call():
+            torch.matmul(a_, b_, out=c_)
+            return c_
+
+        return dict(call=call, check=lambda: (0.0, 0.0), flops=2.0 * n * n * n, bytes_kv=3.0 * n * n * 2,
+                    desc=f"bf16 {n} x {n} x {n} matrix product of the BLAS library (instruction-counter calibration)",
+                    dtype="bf16", bound="mfma", kernel="gemm")
     raise SystemExit(f"unknown config {name}")
 
 
@@ -442,7 +457,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "spec4", "chunk256", "chunk256_paged", "copy1g",
+    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "cfg2_bshd", "cfg2_bwd", "cfg2_mask", "cfg2_drop", "cfg2_mask_bwd", "spec4", "chunk256", "chunk256_paged", "copy1g", "gemm8k",
                              "cfg5_paged"])
     ap.add_argument("--no-extras", action="store_true", help="time only --config (for profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -466,7 +481,7 @@ def main():
         n0 = torch_mlu_amd.launch_count()
         eo, el = w["check"]()
         wall, ev_mean, ev_med, ev_min = time_steps(w["call"], steps, warmup)
-        assert name in ("copy1g", "cfg5_paged", "chunk256_paged") or torch_mlu_amd.launch_count() >= n0 + steps + warmup, \
+        assert name in ("copy1g", "gemm8k", "cfg5_paged", "chunk256_paged") or torch_mlu_amd.launch_count() >= n0 + steps + warmup, \
             "the registered HIP path did not run"
         r = {"config": name, "workload": w["desc"], "ms_per_step": wall, "kernel_ms_mean": ev_mean,
              "kernel_ms_median": ev_med, "kernel_ms_min": ev_min, "tflops": w["flops"] / wall / 1e9,
