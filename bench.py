@@ -25,21 +25,23 @@ import torch
 
 PEAK_MFMA_TFLOPS = 2500.0  # dense bf16 / fp16
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same file,
+# HBM bytes per step (all launches of one op call), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same file,
 # each scaled by what the same counter reads for the 1 GiB copy of --config copy1g (2.000 and 1.000); the runs and
-# their commands are recorded under profiles/ (all of one session on one box, after the last kernel change).  Counters
-# cannot be read from inside a timed run, so these are the recorded values (None: not profiled).
+# their commands are recorded under profiles/, all of them from one session on one box after the last kernel change.
+# Counters cannot be read from inside a timed run, so these are the recorded values (absent: not profiled).
 TRAFFIC_BYTES = {
-    "cfg2": int((520.5 + 130.0) * 2 ** 20),
-    "cfg3": int((212.9 + 130.0) * 2 ** 20),
-    "cfg4": int((286.1 + 68.2) * 2 ** 20),
-    "cfg5": int(2.0006 * 2 ** 30 + 0.52 * 2 ** 20),
-    "cfg2_bwd": int((1849.0 + 388.0) * 2 ** 20),  # the three launches of one backward together
-    "cfg2_mask": int(2.10 * 2 ** 30 + 130.0 * 2 ** 20),
-    "cfg2_drop": int((515.5 + 130.0) * 2 ** 20),
-    "cfg2_mask_bwd": int((3.84 + 2.24 + 1.97) * 2 ** 30 + (156.0 + 128.0 + 128.0) * 2 ** 20),  # three launches
-    "spec4": int(1.0011 * 2 ** 30 + (2.1 + 2.1 + 0.3) * 2 ** 20),  # split-KV + merge launches
-    "chunk256": int((222.3 + 32.6 + 32.6 + 2.1) * 2 ** 20),        # sliced tile + merge launches
+    "cfg2": 682075258,
+    "cfg3": 359938145,
+    "cfg4": 372175500,
+    "cfg5": 2148688012,
+    "cfg5_paged": 2149101678,
+    "spec4": 1079667993,
+    "chunk256": 276249529,
+    "chunk256_paged": 277739884,
+    "cfg2_drop": 676919019,
+    "cfg2_mask": 2397523482,
+    "cfg2_bwd": 2321356559,
+    "cfg2_mask_bwd": 8904146882,
 }
 
 
