@@ -164,3 +164,25 @@ def test_paged_prefill_chunk_long_cache():
     ro, rl = oracle.sdpa_oracle(qd[b:b + 1].cpu(), kf[b:b + 1, :, :lens[b]].cpu(), vf[b:b + 1, :, :lens[b]].cpu(), is_causal=True)
     out_close(out_p[b:b + 1].float().cpu().numpy(), ro, BF)
     lse_close(lse_p[b:b + 1].cpu().numpy(), rl)
+
+
+@pytest.mark.parametrize("Sq,causal", [(1, False), (4, True), (200, True)])
+def test_paged_pool_with_head_major_pages(Sq, causal):
+    """The pools' layout is whatever the stride fields say: pages held as [kv head][row][D] in memory (a kv head's rows
+    contiguous, the layout that decodes fastest) give the bits of the row-major pages, on either kernel."""
+    B, Hk, group, D, page = 3, 2, 4, 128, 64
+    Hq = Hk * group
+    lens = [7 * page + 5 + Sq, Sq + 3, 2 * page + Sq]
+    q, kp, vp, table, used, kf, vf = _paged_case(B, Hq, Hk, Sq, D, page, lens, BF, 1300 + Sq)
+    qd, kpd, vpd, td, ud = (t.to(DEV) for t in (q, kp, vp, table, used))
+    # the same values, stored [pages, Hk, page, D] and seen through a [pages, page, Hk, D] view
+    kph = kpd.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    vph = vpd.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    assert kph.stride(1) == D and kph.stride(2) == page * D
+    for ns in (0, 1, 2):
+        a = capi.fa_forward_paged(qd, kpd, vpd, td, ud, is_causal=causal, num_splits=ns)
+        b = capi.fa_forward_paged(qd, kph, vph, td, ud, is_causal=causal, num_splits=ns)
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]), ns
+    ro, rl = oracle.sdpa_oracle(q[:1], kf[:1, :, :lens[0]], vf[:1, :, :lens[0]], is_causal=causal)
+    out_close(b[0][:1].float().cpu().numpy(), ro, BF)
+    lse_close(b[1][:1].cpu().numpy(), rl)
